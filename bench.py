@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Benchmark: greedy decode tok/s at the Llama-2-7B shape (W8A32, batch 1) on one MI355X.
+
+A step is one token: one replay of the captured per-token graph (embedding row, 32 layers of
+rmsnorm+QKV+RoPE / attention / Wo / rmsnorm+W1,W3+SwiGLU / W2, final rmsnorm + fp32 classifier +
+argmax).  Weights are seeded N(0, 0.02)-like values quantized with the reference's group-int8
+encoder on the GPU; the prompt is 32 seeded ids; everything is resident in HBM before the clock
+starts.  One JSON line is printed.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+WORKLOADS = {
+    # name: (dim, hidden, layers, heads, kv_heads, vocab, seq_len, shared), seed, prompt ids
+    "llama2-7b-shape": ((4096, 11008, 32, 32, 32, 32000, 4096, 0), 103, 32),
+    "llama2-13b-shape": ((5120, 13824, 40, 40, 40, 32000, 4096, 0), 105, 32),
+    "stories110m-shape": ((768, 2048, 12, 12, 12, 32000, 1024, 1), 102, 16),
+    "stories15m-shape": ((288, 768, 6, 6, 6, 32000, 256, 1), 101, 8),
+}
+HBM_PEAK_GBS = 8000.0
+
+
+def synth_prompt(seed, n, vocab):
+    """ids uniform in [3, vocab) from the same counter-based generator the weights use (stream 0xFFFF)."""
+    M = (1 << 64) - 1
+    base = (seed * 0x9E3779B97F4A7C15 + 0xFFFF * 0xD1B54A32D192ED03) & M
+    out = []
+    for i in range(n):
+        z = (base + i + 0x9E3779B97F4A7C15) & M
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+        z ^= z >> 31
+        out.append(3 + (z >> 33) % (vocab - 3))
+    return np.array(out, dtype=np.int32)
+
+
+def cpu_baseline(shape, seed, prompt, gpu_tokens, budget_steps):
+    """The CPU oracle (a C restatement of llama2j's CPU mode, same row/head-parallel decomposition,
+    OpenMP over the host cores) timed on a bounded sample of the same workload, by the reference's
+    own rule: clock starts after the first forward, tok/s = (forwards - 1) / elapsed."""
+    from oracle import binding as orc
+    t0 = time.time()
+    m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
+                  vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
+    m.fill_synth(seed, 0.02)
+    fill_s = time.time() - t0
+    toks, _, sec = m.generate_greedy(prompt, budget_steps)
+    same = bool(np.array_equal(toks, gpu_tokens[:len(toks)]))
+    cores = orc.lib().orc_num_threads()
+    m.close()
+    return {
+        "value": round((len(toks) - 1) / sec, 4) if sec > 0 else None,
+        "unit": "tok/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "first %d forwards of the same workload (same seeded weights and prompt); C restatement of "
+                  "llama2j CPU mode, reference never executed (no JVM); weights generated in %.1f s" % (len(toks), fill_s),
+        "tokens_match_gpu": same,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=288, help="tokens decoded in the timed region (32 prompt + 256 greedy)")
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--workload", default="llama2-7b-shape", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-steps", type=int, default=13, help="forwards of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (batch-1 decode, no multi-GPU split); --gpus %d is not supported" % a.gpus,
+              file=sys.stderr)
+        return 2
+
+    import llama2j_amd as l2j
+    from llama2j_amd import KERNEL
+
+    shape, seed, n_prompt = WORKLOADS[a.workload]
+    steps = min(a.steps, shape[6])
+    g = l2j.Transformer(l2j.Config(*shape))
+    t0 = time.time()
+    g.fill_synthetic(seed, 0.02)
+    g.finalize()
+    load_s = time.time() - t0
+    prompt = synth_prompt(seed, n_prompt, shape[5])
+
+    if a.warmup > 0:
+        g.decode_greedy(prompt, min(a.warmup, shape[6]))
+        g.reset()
+    g.sync()
+    t0 = time.perf_counter()
+    tokens, sec_after_first = g.decode_greedy(prompt, steps)
+    g.sync()
+    wall = time.perf_counter() - t0
+    done = len(tokens)
+    if done != steps:
+        print("bench.py: decode stopped after %d of %d steps (token 1 emitted)" % (done, steps), file=sys.stderr)
+
+    mean_pos = (done - 1) / 2.0
+    bytes_tok = g.bytes_per_token(int(round(mean_pos)))
+    tok_s = done / wall
+    out = {
+        "metric": "decode tok/s at Llama-2-7B shape W8A32; matvec HBM GB/s vs 8 TB/s peak",
+        "value": round(tok_s, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": done,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall / done * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8 weights x f32 activations (W8A32), f32 accumulate",
+        "data": "synthetic: seeded N(0,0.02)-like weights quantized by the reference's group-int8 encoder, seeded prompt ids",
+        "config": {"workload": "%s: dim %d, hidden %d, %d layers, %d heads, vocab %d, seq_len %d; batch 1 greedy, "
+                               "%d prompt ids + %d generated" % ((a.workload,) + shape[:4] + shape[5:7] + (n_prompt, done - n_prompt)),
+                   "weights_load_s": round(load_s, 2)},
+        "tok_s_reference_rule": round((done - 1) / sec_after_first, 2) if sec_after_first > 0 else None,
+        "bytes_per_token": bytes_tok,
+        "stream_roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / bytes_tok, 1),
+        "frac_of_stream_roofline": round(tok_s * bytes_tok / (HBM_PEAK_GBS * 1e9), 4),
+    }
+
+    if not a.no_kernels:
+        pos = int(round(mean_pos))
+        kern = {}
+        for k in range(6):
+            us, b = g.time_kernel(k, pos, rounds=3)
+            kern[KERNEL.NAMES[k]] = {"us": round(us, 3), "bytes": b, "GBps": round(b / us * 1e-3, 1),
+                                     "frac": round(b / us * 1e-3 / HBM_PEAK_GBS, 4)}
+        out["kernels"] = kern
+        dom = kern["w13"]
+        traffic = None
+        tpath = os.path.join(ROOT, "profiles", "w13_traffic.json")
+        if a.workload == "llama2-7b-shape" and os.path.exists(tpath):
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        out["roofline"] = {"bound": "hbm", "kernel": "k_matvec<MV_W13> (rmsnorm + W1,W3 matvec + SwiGLU)",
+                           "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
+                           "traffic": traffic}
+    else:
+        out["roofline"] = None
+
+    if a.cpu_steps > 1:
+        g_tokens = tokens.copy()
+        g.close()
+        out["cpu_baseline"] = cpu_baseline(shape, seed, prompt, g_tokens, min(a.cpu_steps, steps))
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,162 @@
+/*
+ * libllama2j_hip.so - C ABI of the MI355X (gfx950) mode of llama2j's per-token forward pass.
+ *
+ * The library owns every device buffer (weights, activations, KV cache), takes llama2j's own
+ * weight formats, and replays the whole token as one captured hipGraph on one GPU.  It is the
+ * seam a `Mode.HIP` plugs into beside the reference's CPU and CUDA modes: each entry point
+ * names the reference interface it replaces (paths relative to the reference root,
+ * J/ = src/main/java/com/lastbot/llama2j/, K/ = J/kernel/).
+ *
+ * Conventions: plain C, no exceptions cross the boundary, 0 = success and negative = error
+ * (the text is in l2j_last_error(), thread local).  Entry points that run the forward pass are
+ * not re-entrant per context; uploads are thread safe (the reference uploads from ten threads,
+ * J/TransformerWeights.java:52,204).  There is no CPU fallback: without a GPU l2j_create fails.
+ */
+#ifndef LLAMA2J_HIP_H
+#define LLAMA2J_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct l2j_ctx l2j_ctx;
+
+enum {
+    L2J_OK = 0,
+    L2J_E_ARG = -1,    /* bad argument (null, out of range token/pos, unsupported shape) */
+    L2J_E_SIZE = -2,   /* byte/float count does not match the tensor (J/TransformerWeights.java:228-232) */
+    L2J_E_STATE = -3,  /* call not legal in this state (forward before finalize, upload after) */
+    L2J_E_HIP = -4,    /* a HIP runtime call failed (J/ContextCUDA.java:296-304) */
+    L2J_E_OOM = -5,    /* device or host allocation failed (J/ContextCPU.java:20-26) */
+    L2J_E_IO = -6      /* file missing, short or malformed */
+};
+
+/* J/Config.java:6-14 plus the two facts J/Run.java:550,572 derives; the first seven fields are
+ * the 7-int header of the checkpoint (J/Run.java:563-569). */
+typedef struct {
+    int32_t dim, hidden_dim, n_layers, n_heads, n_kv_heads, vocab_size, seq_len;
+    int32_t shared_weights; /* classifier == embedding (J/Run.java:572) */
+    int32_t group_size;     /* 256 only (J/Run.java:27) */
+    int32_t bits;           /* 8 only   (J/Run.java:28) */
+    int32_t device;         /* HIP device ordinal */
+    uint32_t flags;         /* L2J_F_* */
+} l2j_config;
+
+#define L2J_F_EXACT_SILU 1u /* use exact sigmoid instead of the reference's lookup table (K/Silu.java:30) */
+
+/* Tensors in checkpoint file order (J/TransformerWeights.java:50-122). */
+enum l2j_tensor {
+    L2J_TOK_EMB = 0, L2J_RMS_ATT, L2J_WQ, L2J_WK, L2J_WV, L2J_WO, L2J_RMS_FFN,
+    L2J_W1, L2J_W2, L2J_W3, L2J_RMS_FINAL, L2J_WCLS, L2J_TENSOR_COUNT
+};
+
+/* Read-back taps, named after J/RunState.java:20-34.  L2J_B_K / L2J_B_V are the rows written to the
+ * cache at the current position.  Per-layer taps (layer >= 0) are filled by l2j_forward_taps. */
+enum l2j_buffer {
+    L2J_B_X = 0,      /* residual stream; per-layer: after the FFN residual (J/Run.java:158) */
+    L2J_B_XB,         /* per-layer: attention output before Wo (J/Run.java:129) */
+    L2J_B_XB2,        /* per-layer: residual stream after the attention residual (J/Run.java:136) */
+    L2J_B_HB,         /* per-layer: SwiGLU output (J/Run.java:152) */
+    L2J_B_Q,          /* per-layer: q after RoPE (J/Run.java:88) */
+    L2J_B_K,          /* per-layer: k after RoPE */
+    L2J_B_V,          /* per-layer: v */
+    L2J_B_LOGITS,     /* J/Run.java:168 */
+    L2J_B_KCACHE,     /* (layer, seq_len, kv_dim) fp32, J/RunState.java:101 ; `off` counts from the layer base */
+    L2J_B_VCACHE,
+    L2J_B_COUNT
+};
+
+/* = new ContextCUDA + RunState device half (J/Context.java:16-23, J/RunState.java:107-166). */
+int l2j_create(const l2j_config *cfg, l2j_ctx **out);
+/* = Context.close / RunState.close (J/Run.java:697-701, J/ContextCUDA.java:311-323). */
+void l2j_destroy(l2j_ctx *ctx);
+const char *l2j_last_error(void);
+int l2j_device_count(void);
+
+/* = allocateQuantAndCopyToDevice (J/ContextCUDA.java:138-158, J/TransformerWeights.java:238-257).
+ * `ref_bytes` is the exact payload of a .quant cache: ceil(n/256) groups of 264 bytes
+ * (big-endian fp32 min, max, then 256 unsigned codes; J/Quant.java:156-193).  The memory is
+ * borrowed for the call only.  nbytes must equal ceil(n/256)*264. */
+int l2j_upload_quant(l2j_ctx *ctx, int tensor, const uint8_t *ref_bytes, uint64_t nbytes);
+/* One layer of a per-layer tensor, so no caller needs a buffer above 2^31 bytes (the reference's
+ * own int offsets overflow at 13B, J/TransformerWeights.java:89).  Legal only when a layer's float
+ * count is a multiple of 256. */
+int l2j_upload_quant_layer(l2j_ctx *ctx, int tensor, int layer, const uint8_t *ref_bytes, uint64_t nbytes);
+/* = allocateAndCopyToDevice for the fp32 tensors (J/TransformerWeights.java:125-141):
+ * L2J_TOK_EMB and L2J_WCLS (ignored when shared). */
+int l2j_upload_f32(l2j_ctx *ctx, int tensor, const float *data, uint64_t nfloats);
+/* = Quant.encode (J/Quant.java:156-193) run on the GPU straight into the device layout:
+ * a quant tensor given as fp32, `first` = float offset inside the tensor (multiple of 256 unless
+ * it is the only call).  Bit-identical codes and min/max to the reference's encoder. */
+int l2j_upload_f32_quantize(l2j_ctx *ctx, int tensor, uint64_t first, const float *data, uint64_t nfloats);
+/* Serialises a device tensor back to .quant payload bytes (groups [group0, group0+ngroups)). */
+int l2j_read_quant(l2j_ctx *ctx, int tensor, uint64_t group0, uint64_t ngroups, uint8_t *ref_bytes_out);
+/* Benchmark input: fills every tensor on the device with seeded values
+ * ((sum of the four 16-bit fields of splitmix64(seed*0x9E3779B97F4A7C15 + stream*0xD1B54A32D192ED03 + i))
+ *  - 131070) * (sigma / 37837.2265625f), stream 0 = embedding, 1..10 = quant tensors in file
+ * order, 11 = classifier, and quantizes the ten quant tensors with the reference's encoder. */
+int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
+
+/* Ends the load phase: tables (RoPE K/ApplyRope.java:34-59, SiLU K/Silu.java:47-57) are built,
+ * the KV cache is zeroed and the per-token graph is captured. */
+int l2j_finalize(l2j_ctx *ctx);
+/* Zeroes the KV cache (a fresh RunState, J/RunState.java:141-151). */
+int l2j_reset(l2j_ctx *ctx);
+
+/* = Run.transformer + the logits copy (J/Run.java:44-51, 625-632).  logits may be NULL. */
+int l2j_forward(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_null);
+/* = Run.transformer + Sampler.argmax (J/Sampler.java:46-57) with a 4-byte read-back. */
+int l2j_forward_argmax(l2j_ctx *ctx, int32_t token, int32_t pos, int32_t *next);
+/* Same result as l2j_forward but launched kernel by kernel, copying every per-layer tap
+ * (the pattern of Mode.TEST, J/Run.java:186-303). */
+int l2j_forward_taps(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_null);
+/* = the token loop of Run.main with temperature 0 (J/Run.java:599-603, 611-685): BOS first,
+ * prompt ids forced as outputs, first-max argmax afterwards, stop after emitting token 1.
+ * out_tokens (capacity min(steps, seq_len), or seq_len when steps <= 0) receives `next` of every
+ * executed iteration, *n_out the final pos.  *seconds (may be NULL) = GPU time from the end of
+ * the first iteration to the end of the last one (J/Run.java:682-684, 703-706). */
+int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps,
+                      int32_t *out_tokens, int32_t *n_out, double *seconds);
+
+/* Activation / cache taps.  layer < 0 reads the live buffer, layer >= 0 the per-layer tap.
+ * `off` and `n` are in floats. */
+int l2j_read(l2j_ctx *ctx, int which, int layer, uint64_t off, float *dst, uint64_t n);
+/* Seeds or restores rows [pos0, pos0+npos) of one layer's KV cache (kv_dim floats per row). */
+int l2j_write_kv(l2j_ctx *ctx, int layer, int32_t pos0, int32_t npos, const float *k, const float *v);
+int l2j_sync(l2j_ctx *ctx);
+
+/* Measurement: launches one kernel class once per layer (cold weights, as inside a token) `rounds`
+ * times at position `pos` and returns the mean kernel time from the start/stop events of each launch. */
+enum l2j_kernel_class { L2J_K_QKV = 0, L2J_K_ATTENTION, L2J_K_WO, L2J_K_W13, L2J_K_W2, L2J_K_CLASSIFIER, L2J_K_COUNT };
+int l2j_time_kernel(l2j_ctx *ctx, int kernel_class, int32_t pos, int32_t rounds, double *mean_us,
+                    uint64_t *algorithmic_bytes);
+/* Algorithmic bytes one token streams at position pos: weights in the reference's storage format
+ * (264 bytes per 256 weights, fp32 classifier and embedding row) plus KV cache read and write. */
+uint64_t l2j_bytes_per_token(const l2j_config *cfg, int32_t pos);
+
+/* ---- host side of the load path (no GPU needed) ---------------------------------------- */
+/* = Quant.numberOfBytesByFloatSize / Quant.encode / Quant.decode (J/Quant.java:39-48,156-193,79-108). */
+uint64_t l2j_quant_nbytes(uint64_t nfloats);
+int l2j_quant_encode(const float *in, uint64_t nfloats, uint8_t *out);
+int l2j_quant_decode(const uint8_t *enc, uint64_t float_index, uint64_t size, float *out);
+/* = BinFileWriter.write / the cache read in readAsQuant (J/BinFileWriter.java:20-34,
+ * J/TransformerWeights.java:219-221): little-endian int32 byte count, then the bytes. */
+int l2j_write_quant_file(const char *path, const uint8_t *bytes, uint64_t nbytes);
+int64_t l2j_read_quant_file(const char *path, uint8_t *dst, uint64_t cap);
+/* Cache file name rule `<dir>/<base>_<tensor>_256_8.quant` (J/TransformerWeights.java:194,
+ * J/Quant.java:195-197).  Returns the length written to `out` or a negative error. */
+int l2j_quant_cache_path(const char *bin_path, int tensor, char *out, int cap);
+/* Reads the 7-int header (J/Run.java:563-573) into cfg (group 256, bits 8, device 0, flags 0). */
+int l2j_read_checkpoint_header(const char *bin_path, l2j_config *cfg);
+/* = the TransformerWeights constructor (J/TransformerWeights.java:43-144,191-356) + Context +
+ * RunState: reads the llama2.c v0 checkpoint, takes each `.quant` cache when present, otherwise
+ * quantizes (on the GPU) and, when write_caches != 0, writes the cache; uploads; finalizes. */
+int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int write_caches, l2j_ctx **out);
+int l2j_get_config(l2j_ctx *ctx, l2j_config *cfg);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

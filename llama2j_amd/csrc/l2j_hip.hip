@@ -1,0 +1,904 @@
+// libllama2j_hip.so: device side of the C ABI declared in include/llama2j_hip.h.
+// Owns device memory, converts the reference's weight formats to the streaming layout, captures
+// the per-token launch sequence as a hipGraph and replays it.
+#include "kernels.hpp"
+
+#include <hip/hip_ext.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/llama2j_hip.h"
+#include "host_internal.h"
+
+using namespace l2j;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string &msg)
+{
+    g_err = msg;
+    return code;
+}
+
+#define HIPCHK(expr)                                                                              \
+    do {                                                                                          \
+        hipError_t e_ = (expr);                                                                   \
+        if (e_ != hipSuccess)                                                                     \
+            return fail(e_ == hipErrorOutOfMemory ? L2J_E_OOM : L2J_E_HIP,                        \
+                        std::string(#expr) + ": " + hipGetErrorString(e_));                      \
+    } while (0)
+
+struct QTensor {
+    uint8_t *codes = nullptr;  // one byte per weight, flat, padded to whole groups
+    float2 *gs = nullptr;      // ((max-min)/255, min) per group
+    float2 *mm = nullptr;      // (min, max) per group
+    uint64_t nfloats = 0, ngroups = 0;
+    uint64_t groups_loaded = 0;
+};
+
+int env_int(const char *name, int dflt)
+{
+    const char *v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+}  // namespace
+
+struct l2j_ctx {
+    l2j_config cfg{};
+    int head_size = 0, kv_dim = 0, kv_mul = 0;
+    int n_cu = 256;
+    hipStream_t stream = nullptr;
+    std::mutex upload_mu;
+    bool finalized = false;
+
+    QTensor qt[L2J_TENSOR_COUNT];
+    float *emb = nullptr, *wcls = nullptr;
+    bool emb_loaded = false, wcls_loaded = false;
+
+    // activations
+    float *x = nullptr, *xb = nullptr, *hb = nullptr, *q = nullptr, *logits = nullptr;
+    float *kcache = nullptr, *vcache = nullptr;
+    float2 *rope = nullptr;
+    float *silu = nullptr;
+    float *attn_part = nullptr;
+    unsigned *counters = nullptr;  // n_heads attention counters + 1 classifier counter
+    float *cls_val = nullptr;
+    int *cls_idx = nullptr;
+    DevState *st = nullptr;
+    int *prompt = nullptr, *out_tokens = nullptr;
+    DevState *h_st = nullptr;  // pinned
+    int *h_tokens = nullptr;   // pinned, seq_len
+
+    // per-layer taps (allocated on first l2j_forward_taps)
+    float *taps[L2J_B_COUNT] = {};
+
+    // launch shapes
+    int mv_threads = 512, mv_blocks_per_cu = 2, attn_nsplit = 32, attn_chunk_max = 0, cls_blocks = 512;
+
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    std::vector<hipEvent_t> events;
+};
+
+namespace {
+
+uint64_t tensor_floats(const l2j_config &c, int t)
+{
+    const uint64_t L = c.n_layers, dim = c.dim, hid = c.hidden_dim, hs = c.dim / c.n_heads;
+    const uint64_t kvd = (uint64_t)c.n_kv_heads * hs;
+    switch (t) {
+    case L2J_TOK_EMB: case L2J_WCLS: return (uint64_t)c.vocab_size * dim;
+    case L2J_RMS_ATT: case L2J_RMS_FFN: return L * dim;
+    case L2J_WQ: case L2J_WO: return L * dim * dim;
+    case L2J_WK: case L2J_WV: return L * dim * kvd;
+    case L2J_W1: case L2J_W2: case L2J_W3: return L * dim * hid;
+    case L2J_RMS_FINAL: return dim;
+    default: return 0;
+    }
+}
+
+bool is_quant(int t) { return t >= L2J_RMS_ATT && t <= L2J_RMS_FINAL; }
+bool per_layer(int t) { return t >= L2J_RMS_ATT && t <= L2J_W3; }
+
+int validate_config(const l2j_config &c)
+{
+    if (c.dim <= 0 || c.hidden_dim <= 0 || c.n_layers <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 || c.vocab_size <= 0 ||
+        c.seq_len <= 0)
+        return fail(L2J_E_ARG, "config: every dimension must be positive");
+    if (c.group_size != 256 || c.bits != 8) return fail(L2J_E_ARG, "config: only group_size 256 / 8 bits (J/Run.java:27-28)");
+    if (c.dim % c.n_heads || c.n_heads % c.n_kv_heads) return fail(L2J_E_ARG, "config: dim %% n_heads or n_heads %% n_kv_heads != 0");
+    const int hs = c.dim / c.n_heads;
+    if (hs % 4 || hs > 256) return fail(L2J_E_ARG, "config: head_size must be a multiple of 4, at most 256");
+    if (c.dim % 16 || c.hidden_dim % 16 || (c.n_kv_heads * hs) % 16)
+        return fail(L2J_E_ARG, "config: dim, hidden_dim and kv_dim must be multiples of 16 (16-byte weight loads)");
+    if ((uint64_t)c.hidden_dim * 4 + c.hidden_dim / 4 + 256 > 160 * 1024)
+        return fail(L2J_E_ARG, "config: hidden_dim does not fit the 160 KB LDS");
+    return L2J_OK;
+}
+
+template <typename T>
+int dev_alloc(T **p, uint64_t count)
+{
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(p), std::max<uint64_t>(count, 1) * sizeof(T)));
+    return L2J_OK;
+}
+
+size_t mv_smem(int n) { return (size_t)n * 4 + (size_t)(n / 16) * 4 + 64 * sizeof(float); }
+
+struct LayerPtrs {
+    MatvecArgs qkv, wo, w13, w2;
+    AttnArgs attn;
+};
+
+QMat qmat(const l2j_ctx *c, int t, uint64_t off)
+{
+    QMat m;
+    m.codes = c->qt[t].codes;
+    m.gs = c->qt[t].gs;
+    m.off = (long)off;
+    return m;
+}
+
+void layer_args(const l2j_ctx *c, int l, LayerPtrs &p)
+{
+    const l2j_config &g = c->cfg;
+    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim;
+    const uint64_t kvoff = (uint64_t)l * g.seq_len * kvd;
+
+    MatvecArgs a{};
+    a.xin = c->x; a.n = g.dim;
+    a.rms.codes = c->qt[L2J_RMS_ATT].codes; a.rms.mm = c->qt[L2J_RMS_ATT].mm; a.rms.off = (long)(l * dim);
+    a.m0 = qmat(c, L2J_WQ, l * dim * dim); a.m1 = qmat(c, L2J_WK, l * dim * kvd); a.m2 = qmat(c, L2J_WV, l * dim * kvd);
+    a.d0 = g.dim; a.d1 = c->kv_dim; a.d2 = c->kv_dim;
+    a.out0 = c->q; a.out1 = c->kcache + kvoff; a.out2 = c->vcache + kvoff;
+    a.rope = c->rope; a.head_size = c->head_size; a.kv_dim = c->kv_dim;
+    a.silu_table = c->silu; a.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0; a.st = c->st;
+    p.qkv = a;
+
+    AttnArgs t{};
+    t.q = c->q; t.kc = c->kcache + kvoff; t.vc = c->vcache + kvoff; t.out = c->xb; t.part = c->attn_part;
+    t.counters = c->counters; t.st = c->st; t.n_heads = g.n_heads; t.kv_mul = c->kv_mul; t.head_size = c->head_size;
+    t.kv_dim = c->kv_dim; t.nsplit = c->attn_nsplit; t.chunk_max = c->attn_chunk_max;
+    t.sqrt_hs = sqrtf((float)c->head_size);  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
+    p.attn = t;
+
+    MatvecArgs o = a;
+    o.xin = c->xb; o.n = g.dim; o.m0 = qmat(c, L2J_WO, l * dim * dim); o.d0 = g.dim; o.d1 = o.d2 = 0; o.out0 = c->x;
+    p.wo = o;
+
+    MatvecArgs f = a;
+    f.xin = c->x; f.n = g.dim;
+    f.rms.codes = c->qt[L2J_RMS_FFN].codes; f.rms.mm = c->qt[L2J_RMS_FFN].mm; f.rms.off = (long)(l * dim);
+    f.m0 = qmat(c, L2J_W1, l * dim * hid); f.m1 = qmat(c, L2J_W3, l * dim * hid); f.d0 = g.hidden_dim; f.d1 = g.hidden_dim; f.d2 = 0;
+    f.out0 = c->hb;
+    p.w13 = f;
+
+    MatvecArgs w = a;
+    w.xin = c->hb; w.n = g.hidden_dim; w.m0 = qmat(c, L2J_W2, l * dim * hid); w.d0 = g.dim; w.d1 = w.d2 = 0; w.out0 = c->x;
+    p.w2 = w;
+}
+
+ClsArgs cls_args(const l2j_ctx *c)
+{
+    ClsArgs a{};
+    a.xin = c->x; a.n = c->cfg.dim;
+    a.rms.codes = c->qt[L2J_RMS_FINAL].codes; a.rms.mm = c->qt[L2J_RMS_FINAL].mm; a.rms.off = 0;
+    a.w = c->wcls; a.vocab = c->cfg.vocab_size; a.logits = c->logits;
+    a.part_val = c->cls_val; a.part_idx = c->cls_idx; a.counter = c->counters + c->cfg.n_heads;
+    a.st = c->st; a.prompt = c->prompt; a.out_tokens = c->out_tokens;
+    return a;
+}
+
+int mv_grid(const l2j_ctx *c, int npairs)
+{
+    const int wpb = c->mv_threads / 64;
+    return std::max(1, std::min((npairs + wpb - 1) / wpb, c->n_cu * c->mv_blocks_per_cu));
+}
+
+struct Launch {
+    dim3 grid, block;
+    size_t smem;
+};
+
+Launch shape_of(const l2j_ctx *c, int kclass)
+{
+    const l2j_config &g = c->cfg;
+    Launch L{};
+    L.block = dim3(c->mv_threads);
+    switch (kclass) {
+    case L2J_K_QKV: L.grid = dim3(mv_grid(c, (g.dim + 2 * c->kv_dim) / 2)); L.smem = mv_smem(g.dim); break;
+    case L2J_K_WO: L.grid = dim3(mv_grid(c, (g.dim + 1) / 2)); L.smem = mv_smem(g.dim); break;
+    case L2J_K_W13: L.grid = dim3(mv_grid(c, g.hidden_dim)); L.smem = mv_smem(g.dim); break;
+    case L2J_K_W2: L.grid = dim3(mv_grid(c, (g.dim + 1) / 2)); L.smem = mv_smem(g.hidden_dim); break;
+    case L2J_K_CLASSIFIER: L.grid = dim3(c->cls_blocks); L.smem = mv_smem(g.dim) + 64 * sizeof(float); break;
+    case L2J_K_ATTENTION:
+        L.grid = dim3(g.n_heads * c->attn_nsplit);
+        L.block = dim3(kAttnThreads);
+        L.smem = (size_t)(c->attn_chunk_max + kAttnThreads / 64 + (kAttnThreads / 64) * c->head_size) * sizeof(float);
+        break;
+    }
+    return L;
+}
+
+template <typename K, typename A>
+hipError_t launch1(K kernel, const Launch &L, hipStream_t s, const A &args, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
+{
+    if (e0) {
+        hipExtLaunchKernelGGL(kernel, L.grid, L.block, (unsigned)L.smem, s, e0, e1, 0, args);
+    } else {
+        hipLaunchKernelGGL(kernel, L.grid, L.block, L.smem, s, args);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_class(const l2j_ctx *c, int kclass, const LayerPtrs &p, hipStream_t s, hipEvent_t e0 = nullptr,
+                        hipEvent_t e1 = nullptr)
+{
+    const Launch L = shape_of(c, kclass);
+    switch (kclass) {
+    case L2J_K_QKV: return launch1(k_matvec<MV_QKV>, L, s, p.qkv, e0, e1);
+    case L2J_K_WO: return launch1(k_matvec<MV_RES>, L, s, p.wo, e0, e1);
+    case L2J_K_W13: return launch1(k_matvec<MV_W13>, L, s, p.w13, e0, e1);
+    case L2J_K_W2: return launch1(k_matvec<MV_RES>, L, s, p.w2, e0, e1);
+    case L2J_K_ATTENTION:
+        if (c->head_size <= 64) return launch1(k_attention<16>, L, s, p.attn, e0, e1);
+        if (c->head_size <= 128) return launch1(k_attention<32>, L, s, p.attn, e0, e1);
+        return launch1(k_attention<64>, L, s, p.attn, e0, e1);
+    case L2J_K_CLASSIFIER: return launch1(k_classifier, L, s, cls_args(c), e0, e1);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t tap_copy(l2j_ctx *c, int which, int l, const float *src, uint64_t n, hipStream_t s)
+{
+    return hipMemcpyAsync(c->taps[which] + (uint64_t)l * n, src, n * sizeof(float), hipMemcpyDeviceToDevice, s);
+}
+
+// The launch sequence of one token (J/Run.java:62-169).  With taps, per-layer copies follow each kernel.
+hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
+{
+    const l2j_config &g = c->cfg;
+    hipError_t e;
+    hipLaunchKernelGGL(k_embed, dim3((g.dim / 4 + 255) / 256), dim3(256), 0, s, c->emb, c->st, c->x, g.dim);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    for (int l = 0; l < g.n_layers; l++) {
+        LayerPtrs p;
+        layer_args(c, l, p);
+        if ((e = launch_class(c, L2J_K_QKV, p, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_ATTENTION, p, s)) != hipSuccess) return e;
+        if (taps) {
+            // rows of the caches at the current position; pos is known on the host in this mode
+            const uint64_t row = (uint64_t)c->h_st->pos * c->kv_dim;
+            if ((e = tap_copy(c, L2J_B_Q, l, c->q, g.dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_K, l, p.qkv.out1 + row, c->kv_dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_V, l, p.qkv.out2 + row, c->kv_dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_XB, l, c->xb, g.dim, s)) != hipSuccess) return e;
+        }
+        if ((e = launch_class(c, L2J_K_WO, p, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_XB2, l, c->x, g.dim, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_W13, p, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_HB, l, c->hb, g.hidden_dim, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_W2, p, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_X, l, c->x, g.dim, s)) != hipSuccess) return e;
+    }
+    LayerPtrs none{};
+    return launch_class(c, L2J_K_CLASSIFIER, none, s);
+}
+
+int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
+{
+    c->h_st->token = token;
+    c->h_st->pos = pos;
+    c->h_st->n_prompt = n_prompt;
+    c->h_st->pad = 0;
+    HIPCHK(hipMemcpyAsync(c->st, c->h_st, sizeof(DevState), hipMemcpyHostToDevice, c->stream));
+    return L2J_OK;
+}
+
+int check_forward_args(l2j_ctx *c, int32_t token, int32_t pos)
+{
+    if (!c) return fail(L2J_E_ARG, "null context");
+    if (!c->finalized) return fail(L2J_E_STATE, "forward before l2j_finalize");
+    if (token < 0 || token >= c->cfg.vocab_size) return fail(L2J_E_ARG, "token out of range");
+    if (pos < 0 || pos >= c->cfg.seq_len) return fail(L2J_E_ARG, "pos out of range");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    return L2J_OK;
+}
+
+int unpack_into(l2j_ctx *c, QTensor &t, uint64_t group0, const uint8_t *ref_bytes, uint64_t ngroups)
+{
+    // staged through a device buffer in slices of at most 64 MiB
+    const uint64_t slice_groups = (64ull << 20) / kGroupBytes;
+    uint8_t *stage = nullptr;
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(ngroups, slice_groups) * kGroupBytes));
+    int rc = L2J_OK;
+    for (uint64_t g = 0; g < ngroups && rc == L2J_OK; g += slice_groups) {
+        const uint64_t ng = std::min(slice_groups, ngroups - g);
+        hipError_t e = hipMemcpy(stage, ref_bytes + g * kGroupBytes, ng * kGroupBytes, hipMemcpyHostToDevice);
+        if (e == hipSuccess) {
+            const int grid = (int)std::min<uint64_t>(ng, 1u << 20);
+            hipLaunchKernelGGL(k_unpack_groups, dim3(grid), dim3(64), 0, c->stream, stage, (long)ng, t.codes + (group0 + g) * kGroup,
+                               t.gs + group0 + g, t.mm + group0 + g);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        }
+        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("upload: ") + hipGetErrorString(e));
+    }
+    (void)hipFree(stage);
+    return rc;
+}
+
+void destroy_graph(l2j_ctx *c)
+{
+    if (c->graph_exec) (void)hipGraphExecDestroy(c->graph_exec);
+    if (c->graph) (void)hipGraphDestroy(c->graph);
+    c->graph_exec = nullptr;
+    c->graph = nullptr;
+}
+
+uint64_t quant_bytes_of(uint64_t weights) { return (weights / kGroup) * kGroupBytes + (weights % kGroup ? kGroupBytes : 0); }
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------
+
+extern "C" {
+
+const char *l2j_last_error(void) { return g_err.c_str(); }
+
+void l2j_set_error_(const char *msg) { g_err = msg ? msg : ""; }
+
+int l2j_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int l2j_create(const l2j_config *cfg, l2j_ctx **out)
+{
+    if (!cfg || !out) return fail(L2J_E_ARG, "l2j_create: null argument");
+    *out = nullptr;
+    int rc = validate_config(*cfg);
+    if (rc) return rc;
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev == 0)
+        return fail(L2J_E_HIP, "l2j_create: no HIP device (this library has no CPU fallback)");
+    if (cfg->device < 0 || cfg->device >= ndev) return fail(L2J_E_ARG, "l2j_create: device ordinal out of range");
+    HIPCHK(hipSetDevice(cfg->device));
+    l2j_ctx *c = new (std::nothrow) l2j_ctx();
+    if (!c) return fail(L2J_E_OOM, "l2j_create: host allocation failed");
+    c->cfg = *cfg;
+    c->head_size = cfg->dim / cfg->n_heads;
+    c->kv_dim = cfg->n_kv_heads * c->head_size;
+    c->kv_mul = cfg->n_heads / cfg->n_kv_heads;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, cfg->device) == hipSuccess && prop.multiProcessorCount > 0) c->n_cu = prop.multiProcessorCount;
+    c->mv_threads = std::min(1024, std::max(64, env_int("L2J_MV_THREADS", 512) / 64 * 64));
+    c->mv_blocks_per_cu = std::max(1, env_int("L2J_MV_BLOCKS_PER_CU", 2));
+    c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
+    c->cls_blocks = std::max(1, std::min(env_int("L2J_CLS_BLOCKS", c->n_cu * c->mv_blocks_per_cu), (cfg->vocab_size + 1) / 2));
+    int cm = std::max((cfg->seq_len + c->attn_nsplit - 1) / c->attn_nsplit, kAttnMinChunk);
+    c->attn_chunk_max = (cm + 3) / 4 * 4;
+
+#define TRY(expr)                \
+    do {                         \
+        rc = (expr);             \
+        if (rc) {                \
+            l2j_destroy(c);      \
+            return rc;           \
+        }                        \
+    } while (0)
+#define TRYHIP(expr)                                                                               \
+    do {                                                                                           \
+        hipError_t e2_ = (expr);                                                                   \
+        if (e2_ != hipSuccess) {                                                                   \
+            l2j_destroy(c);                                                                        \
+            return fail(e2_ == hipErrorOutOfMemory ? L2J_E_OOM : L2J_E_HIP, std::string(#expr) + ": " + hipGetErrorString(e2_)); \
+        }                                                                                          \
+    } while (0)
+
+    TRYHIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    for (int t = 0; t < L2J_TENSOR_COUNT; t++) {
+        if (!is_quant(t)) continue;
+        QTensor &q = c->qt[t];
+        q.nfloats = tensor_floats(*cfg, t);
+        q.ngroups = (q.nfloats + kGroup - 1) / kGroup;
+        TRY(dev_alloc(&q.codes, q.ngroups * kGroup + 64));
+        TRY(dev_alloc(&q.gs, q.ngroups));
+        TRY(dev_alloc(&q.mm, q.ngroups));
+    }
+    const uint64_t vd = (uint64_t)cfg->vocab_size * cfg->dim;
+    TRY(dev_alloc(&c->emb, vd));
+    if (cfg->shared_weights) c->wcls = c->emb;
+    else TRY(dev_alloc(&c->wcls, vd));
+    const uint64_t kvn = (uint64_t)cfg->n_layers * cfg->seq_len * c->kv_dim;
+    TRY(dev_alloc(&c->x, cfg->dim));
+    TRY(dev_alloc(&c->xb, cfg->dim));
+    TRY(dev_alloc(&c->hb, cfg->hidden_dim));
+    TRY(dev_alloc(&c->q, cfg->dim));
+    TRY(dev_alloc(&c->logits, cfg->vocab_size));
+    TRY(dev_alloc(&c->kcache, kvn));
+    TRY(dev_alloc(&c->vcache, kvn));
+    TRY(dev_alloc(&c->rope, (uint64_t)cfg->seq_len * (c->head_size / 2)));
+    TRY(dev_alloc(&c->silu, kSiluTable));
+    TRY(dev_alloc(&c->attn_part, (uint64_t)cfg->n_heads * c->attn_nsplit * (c->head_size + 2)));
+    TRY(dev_alloc(&c->counters, cfg->n_heads + 1));
+    TRY(dev_alloc(&c->cls_val, c->cls_blocks));
+    TRY(dev_alloc(&c->cls_idx, c->cls_blocks));
+    TRY(dev_alloc(&c->st, 1));
+    TRY(dev_alloc(&c->prompt, cfg->seq_len));
+    TRY(dev_alloc(&c->out_tokens, cfg->seq_len));
+    TRYHIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_st), sizeof(DevState), hipHostMallocDefault));
+    TRYHIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_tokens), (size_t)cfg->seq_len * sizeof(int), hipHostMallocDefault));
+    TRYHIP(hipMemset(c->counters, 0, (cfg->n_heads + 1) * sizeof(unsigned)));
+    TRYHIP(hipMemset(c->prompt, 0, (size_t)cfg->seq_len * sizeof(int)));
+    TRYHIP(hipMemset(c->out_tokens, 0, (size_t)cfg->seq_len * sizeof(int)));
+    TRYHIP(hipMemset(c->st, 0, sizeof(DevState)));
+    TRYHIP(hipMemset(c->kcache, 0, kvn * sizeof(float)));
+    TRYHIP(hipMemset(c->vcache, 0, kvn * sizeof(float)));
+    // dynamic LDS above the default limit (large hidden_dim)
+    const int need = (int)mv_smem(std::max(cfg->dim, cfg->hidden_dim)) + 256;
+    if (need > 64 * 1024) {
+        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_RES>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
+        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_QKV>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
+        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_W13>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
+        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_classifier), hipFuncAttributeMaxDynamicSharedMemorySize, need));
+    }
+#undef TRY
+#undef TRYHIP
+    *out = c;
+    return L2J_OK;
+}
+
+void l2j_destroy(l2j_ctx *c)
+{
+    if (!c) return;
+    (void)hipSetDevice(c->cfg.device);
+    if (c->stream) (void)hipStreamSynchronize(c->stream);
+    destroy_graph(c);
+    for (hipEvent_t ev : c->events) (void)hipEventDestroy(ev);
+    for (int t = 0; t < L2J_TENSOR_COUNT; t++) {
+        (void)hipFree(c->qt[t].codes);
+        (void)hipFree(c->qt[t].gs);
+        (void)hipFree(c->qt[t].mm);
+    }
+    if (c->wcls != c->emb) (void)hipFree(c->wcls);
+    (void)hipFree(c->emb);
+    float *bufs[] = {c->x, c->xb, c->hb, c->q, c->logits, c->kcache, c->vcache, c->silu, c->attn_part, c->cls_val};
+    for (float *b : bufs) (void)hipFree(b);
+    (void)hipFree(c->rope);
+    (void)hipFree(c->counters);
+    (void)hipFree(c->cls_idx);
+    (void)hipFree(c->st);
+    (void)hipFree(c->prompt);
+    (void)hipFree(c->out_tokens);
+    for (float *t : c->taps) (void)hipFree(t);
+    if (c->h_st) (void)hipHostFree(c->h_st);
+    if (c->h_tokens) (void)hipHostFree(c->h_tokens);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+int l2j_get_config(l2j_ctx *c, l2j_config *cfg)
+{
+    if (!c || !cfg) return fail(L2J_E_ARG, "null argument");
+    *cfg = c->cfg;
+    return L2J_OK;
+}
+
+static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t ngroups, const uint8_t *bytes, uint64_t nbytes)
+{
+    if (nbytes != ngroups * kGroupBytes)
+        return fail(L2J_E_SIZE, "totalByteSize != quant.numberOfBytesByFloatSize(floatSize)");
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    QTensor &t = c->qt[tensor];
+    int rc = unpack_into(c, t, group0, bytes, ngroups);
+    if (rc == L2J_OK) t.groups_loaded += ngroups;
+    return rc;
+}
+
+int l2j_upload_quant(l2j_ctx *c, int tensor, const uint8_t *ref_bytes, uint64_t nbytes)
+{
+    if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
+    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+    c->qt[tensor].groups_loaded = 0;
+    return upload_quant_range(c, tensor, 0, c->qt[tensor].ngroups, ref_bytes, nbytes);
+}
+
+int l2j_upload_quant_layer(l2j_ctx *c, int tensor, int layer, const uint8_t *ref_bytes, uint64_t nbytes)
+{
+    if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
+    if (!is_quant(tensor) || !per_layer(tensor)) return fail(L2J_E_ARG, "not a per-layer quantized tensor");
+    if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+    const uint64_t per = c->qt[tensor].nfloats / c->cfg.n_layers;
+    if (per % kGroup) return fail(L2J_E_ARG, "layer size is not a multiple of the group size; upload the whole tensor");
+    return upload_quant_range(c, tensor, (uint64_t)layer * (per / kGroup), per / kGroup, ref_bytes, nbytes);
+}
+
+int l2j_upload_f32(l2j_ctx *c, int tensor, const float *data, uint64_t nfloats)
+{
+    if (!c || !data) return fail(L2J_E_ARG, "null argument");
+    if (tensor != L2J_TOK_EMB && tensor != L2J_WCLS) return fail(L2J_E_ARG, "only the embedding and the classifier are fp32");
+    if (nfloats != (uint64_t)c->cfg.vocab_size * c->cfg.dim) return fail(L2J_E_SIZE, "float count != vocab_size * dim");
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    if (tensor == L2J_WCLS && c->cfg.shared_weights) return L2J_OK;  // J/TransformerWeights.java:122
+    HIPCHK(hipMemcpy(tensor == L2J_TOK_EMB ? c->emb : c->wcls, data, nfloats * sizeof(float), hipMemcpyHostToDevice));
+    (tensor == L2J_TOK_EMB ? c->emb_loaded : c->wcls_loaded) = true;
+    return L2J_OK;
+}
+
+int l2j_upload_f32_quantize(l2j_ctx *c, int tensor, uint64_t first, const float *data, uint64_t nfloats)
+{
+    if (!c || !data) return fail(L2J_E_ARG, "null argument");
+    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+    QTensor &t = c->qt[tensor];
+    if (first % kGroup) return fail(L2J_E_ARG, "first must be a multiple of the group size");
+    if (first + nfloats > t.nfloats) return fail(L2J_E_SIZE, "range exceeds the tensor");
+    if (nfloats % kGroup && first + nfloats != t.nfloats) return fail(L2J_E_ARG, "only the tensor's tail may be a partial group");
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const uint64_t slice = 16ull << 20;  // floats per staging slice (64 MiB)
+    float *stage = nullptr;
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(slice, std::max<uint64_t>(nfloats, 1)) * sizeof(float)));
+    int rc = L2J_OK;
+    for (uint64_t o = 0; o < nfloats && rc == L2J_OK; o += slice) {
+        const uint64_t nf = std::min(slice, nfloats - o);
+        const uint64_t ng = (nf + kGroup - 1) / kGroup;
+        hipError_t e = hipMemcpy(stage, data + o, nf * sizeof(float), hipMemcpyHostToDevice);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(256), 0, c->stream, stage, (long)nf,
+                               (long)((first + o) / kGroup), (long)ng, (long)t.nfloats, 0ull, 0.0f, t.codes, t.gs, t.mm);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        }
+        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("quantize: ") + hipGetErrorString(e));
+        else t.groups_loaded += ng;
+    }
+    (void)hipFree(stage);
+    return rc;
+}
+
+int l2j_read_quant(l2j_ctx *c, int tensor, uint64_t group0, uint64_t ngroups, uint8_t *out)
+{
+    if (!c || !out) return fail(L2J_E_ARG, "null argument");
+    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+    QTensor &t = c->qt[tensor];
+    if (group0 + ngroups > t.ngroups) return fail(L2J_E_SIZE, "group range exceeds the tensor");
+    if (ngroups == 0) return L2J_OK;
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const uint64_t slice_groups = (64ull << 20) / kGroupBytes;
+    uint8_t *stage = nullptr;
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(ngroups, slice_groups) * kGroupBytes));
+    int rc = L2J_OK;
+    for (uint64_t g = 0; g < ngroups && rc == L2J_OK; g += slice_groups) {
+        const uint64_t ng = std::min(slice_groups, ngroups - g);
+        hipLaunchKernelGGL(k_pack_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(64), 0, c->stream, stage, (long)ng,
+                           t.codes + (group0 + g) * kGroup, t.mm + group0 + g);
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        if (e == hipSuccess) e = hipMemcpy(out + g * kGroupBytes, stage, ng * kGroupBytes, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("read_quant: ") + hipGetErrorString(e));
+    }
+    (void)hipFree(stage);
+    return rc;
+}
+
+int l2j_fill_synthetic(l2j_ctx *c, uint64_t seed, float sigma)
+{
+    if (!c) return fail(L2J_E_ARG, "null context");
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const float scale = sigma / 37837.2265625f;
+    auto base_of = [&](uint32_t stream) { return seed * 0x9E3779B97F4A7C15ULL + (uint64_t)stream * 0xD1B54A32D192ED03ULL; };
+    const uint64_t vd = (uint64_t)c->cfg.vocab_size * c->cfg.dim;
+    hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->emb, (long)vd, base_of(0), scale);
+    HIPCHK(hipGetLastError());
+    if (c->wcls != c->emb) {
+        hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->wcls, (long)vd, base_of(11), scale);
+        HIPCHK(hipGetLastError());
+    }
+    for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++) {
+        QTensor &q = c->qt[t];
+        hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(q.ngroups, 1u << 20)), dim3(256), 0, c->stream,
+                           (const float *)nullptr, 0L, 0L, (long)q.ngroups, (long)q.nfloats, base_of((uint32_t)t), scale, q.codes, q.gs,
+                           q.mm);
+        HIPCHK(hipGetLastError());
+        q.groups_loaded = q.ngroups;
+    }
+    HIPCHK(hipStreamSynchronize(c->stream));
+    c->emb_loaded = c->wcls_loaded = true;
+    return L2J_OK;
+}
+
+int l2j_finalize(l2j_ctx *c)
+{
+    if (!c) return fail(L2J_E_ARG, "null context");
+    std::lock_guard<std::mutex> lock(c->upload_mu);
+    if (c->finalized) return fail(L2J_E_STATE, "already finalized");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    if (!c->emb_loaded) return fail(L2J_E_STATE, "token_embedding_table was not uploaded");
+    if (!c->cfg.shared_weights && !c->wcls_loaded) return fail(L2J_E_STATE, "wcls was not uploaded");
+    for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++)
+        if (c->qt[t].groups_loaded < c->qt[t].ngroups)
+            return fail(L2J_E_STATE, std::string("tensor not fully uploaded: ") + l2j_host::tensor_stem(t));
+
+    // RoPE table (K/ApplyRope.java:34-59): freq = (float)(1.0 / pow(10000.0f, (i % hs) / (float) hs)),
+    // val = pos * freq in fp32, cos/sin in double then narrowed.  Only i % head_size matters.
+    const int hs = c->head_size, half = hs / 2, S = c->cfg.seq_len;
+    std::vector<float2> rope((size_t)S * half);
+    for (int k = 0; k < half; k++) {
+        const float ex = (float)(2 * k) / (float)hs;
+        const float freq = (float)(1.0 / std::pow((double)10000.0f, (double)ex));
+        for (int pos = 0; pos < S; pos++) {
+            const float val = (float)pos * freq;
+            rope[(size_t)pos * half + k] = make_float2((float)std::cos((double)val), (float)std::sin((double)val));
+        }
+    }
+    HIPCHK(hipMemcpy(c->rope, rope.data(), rope.size() * sizeof(float2), hipMemcpyHostToDevice));
+    // sigmoid table (K/Silu.java:47-57)
+    std::vector<float> tab(kSiluTable);
+    for (int i = 0; i < kSiluTable; i++) {
+        const double v = ((double)i / (double)kSiluTable) * 10.0 - 5.0;
+        tab[i] = (float)(1.0 / (1.0 + std::exp(-v)));
+    }
+    HIPCHK(hipMemcpy(c->silu, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice));
+
+    // capture the token
+    HIPCHK(hipStreamSynchronize(c->stream));
+    HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+    hipError_t le = launch_token(c, c->stream, false);
+    hipError_t ce = hipStreamEndCapture(c->stream, &c->graph);
+    if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
+    HIPCHK(ce);
+    HIPCHK(hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0));
+    c->finalized = true;
+    return L2J_OK;
+}
+
+int l2j_reset(l2j_ctx *c)
+{
+    if (!c) return fail(L2J_E_ARG, "null context");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const uint64_t kvn = (uint64_t)c->cfg.n_layers * c->cfg.seq_len * c->kv_dim;
+    HIPCHK(hipMemsetAsync(c->kcache, 0, kvn * sizeof(float), c->stream));
+    HIPCHK(hipMemsetAsync(c->vcache, 0, kvn * sizeof(float), c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return L2J_OK;
+}
+
+int l2j_sync(l2j_ctx *c)
+{
+    if (!c) return fail(L2J_E_ARG, "null context");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return L2J_OK;
+}
+
+int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
+{
+    int rc = check_forward_args(c, token, pos);
+    if (rc) return rc;
+    if ((rc = set_state(c, token, pos, 0))) return rc;
+    HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+    if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return L2J_OK;
+}
+
+int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
+{
+    if (!next) return fail(L2J_E_ARG, "null argument");
+    int rc = check_forward_args(c, token, pos);
+    if (rc) return rc;
+    if ((rc = set_state(c, token, pos, 0))) return rc;
+    HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+    HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    *next = c->h_tokens[0];
+    return L2J_OK;
+}
+
+int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
+{
+    int rc = check_forward_args(c, token, pos);
+    if (rc) return rc;
+    const uint64_t L = c->cfg.n_layers;
+    const int which[] = {L2J_B_X, L2J_B_XB, L2J_B_XB2, L2J_B_HB, L2J_B_Q, L2J_B_K, L2J_B_V};
+    for (int w : which) {
+        if (c->taps[w]) continue;
+        const uint64_t n = w == L2J_B_HB ? c->cfg.hidden_dim : (w == L2J_B_K || w == L2J_B_V) ? c->kv_dim : c->cfg.dim;
+        if ((rc = dev_alloc(&c->taps[w], L * n))) return rc;
+    }
+    if ((rc = set_state(c, token, pos, 0))) return rc;
+    hipError_t e = launch_token(c, c->stream, true);
+    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
+    if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    return L2J_OK;
+}
+
+int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, int32_t *out_tokens, int32_t *n_out,
+                      double *seconds)
+{
+    if (!c || !out_tokens || !n_out || (n_prompt > 0 && !prompt) || n_prompt < 0) return fail(L2J_E_ARG, "bad argument");
+    if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const int S = c->cfg.seq_len;
+    if (steps <= 0 || steps > S) steps = S;  // J/Run.java:599-603
+    const int np = std::min(n_prompt, S);
+    for (int i = 0; i < np; i++)
+        if (prompt[i] < 0 || prompt[i] >= c->cfg.vocab_size) return fail(L2J_E_ARG, "prompt id out of range");
+    if (np > 0) {
+        memcpy(c->h_tokens, prompt, (size_t)np * sizeof(int));
+        HIPCHK(hipMemcpyAsync(c->prompt, c->h_tokens, (size_t)np * sizeof(int), hipMemcpyHostToDevice, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+    }
+    int rc = set_state(c, 1, 0, np);  // token 1 = BOS at pos 0 (J/Run.java:614)
+    if (rc) return rc;
+
+    // One event after every token of a batch: the stop rule (next == 1) is checked per batch, and the
+    // clock runs from the end of the first token to the end of the token that ended the loop.
+    const int batch = 32;
+    while ((int)c->events.size() < batch + 1) {
+        hipEvent_t ev;
+        HIPCHK(hipEventCreate(&ev));
+        c->events.push_back(ev);
+    }
+    hipEvent_t ev_first = c->events[batch];
+    float total_ms = 0.f;
+    int pos = 0;
+    bool stopped = false;
+    while (pos < steps && !stopped) {
+        const int nb = std::min(batch, steps - pos);
+        for (int i = 0; i < nb; i++) {
+            HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+            if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
+            HIPCHK(hipEventRecord(c->events[i], c->stream));
+        }
+        HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        int used = nb;
+        for (int i = 0; i < nb; i++) {
+            out_tokens[pos + i] = c->h_tokens[i];
+            if (c->h_tokens[i] == 1) {  // J/Run.java:670-672
+                used = i + 1;
+                stopped = true;
+                break;
+            }
+        }
+        if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
+        pos += used;
+    }
+    *n_out = pos;
+    if (seconds) *seconds = (double)total_ms * 1e-3;
+    return L2J_OK;
+}
+
+int l2j_read(l2j_ctx *c, int which, int layer, uint64_t off, float *dst, uint64_t n)
+{
+    if (!c || !dst) return fail(L2J_E_ARG, "null argument");
+    if (which < 0 || which >= L2J_B_COUNT) return fail(L2J_E_ARG, "unknown buffer");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const l2j_config &g = c->cfg;
+    const float *src = nullptr;
+    uint64_t len = 0;
+    if (which == L2J_B_KCACHE || which == L2J_B_VCACHE) {
+        if (layer < 0 || layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        len = (uint64_t)g.seq_len * c->kv_dim;
+        src = (which == L2J_B_KCACHE ? c->kcache : c->vcache) + (uint64_t)layer * len;
+    } else if (which == L2J_B_LOGITS) {
+        src = c->logits; len = g.vocab_size;
+    } else if (layer < 0) {
+        switch (which) {
+        case L2J_B_X: src = c->x; len = g.dim; break;
+        case L2J_B_XB: src = c->xb; len = g.dim; break;
+        case L2J_B_HB: src = c->hb; len = g.hidden_dim; break;
+        case L2J_B_Q: src = c->q; len = g.dim; break;
+        default: return fail(L2J_E_ARG, "this buffer only exists as a per-layer tap");
+        }
+    } else {
+        if (layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        if (!c->taps[which]) return fail(L2J_E_STATE, "no taps recorded: call l2j_forward_taps first");
+        len = which == L2J_B_HB ? g.hidden_dim : (which == L2J_B_K || which == L2J_B_V) ? c->kv_dim : g.dim;
+        src = c->taps[which] + (uint64_t)layer * len;
+    }
+    if (off + n > len) return fail(L2J_E_SIZE, "read past the end of the buffer");
+    HIPCHK(hipStreamSynchronize(c->stream));
+    HIPCHK(hipMemcpy(dst, src + off, n * sizeof(float), hipMemcpyDeviceToHost));
+    return L2J_OK;
+}
+
+int l2j_write_kv(l2j_ctx *c, int layer, int32_t pos0, int32_t npos, const float *k, const float *v)
+{
+    if (!c || !k || !v) return fail(L2J_E_ARG, "null argument");
+    if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+    if (pos0 < 0 || npos < 0 || (int64_t)pos0 + npos > c->cfg.seq_len) return fail(L2J_E_ARG, "positions out of range");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const uint64_t o = ((uint64_t)layer * c->cfg.seq_len + pos0) * c->kv_dim, n = (uint64_t)npos * c->kv_dim;
+    HIPCHK(hipStreamSynchronize(c->stream));
+    HIPCHK(hipMemcpy(c->kcache + o, k, n * sizeof(float), hipMemcpyHostToDevice));
+    HIPCHK(hipMemcpy(c->vcache + o, v, n * sizeof(float), hipMemcpyHostToDevice));
+    return L2J_OK;
+}
+
+uint64_t l2j_bytes_per_token(const l2j_config *g, int32_t pos)
+{
+    if (!g) return 0;
+    const uint64_t L = g->n_layers, dim = g->dim, hid = g->hidden_dim;
+    const uint64_t kvd = (uint64_t)g->n_kv_heads * (g->dim / g->n_heads);
+    const uint64_t mat = L * (2 * dim * dim + 2 * dim * kvd + 3 * dim * hid);
+    return quant_bytes_of(mat) + 2 * quant_bytes_of(L * dim) + quant_bytes_of(dim) + (uint64_t)g->vocab_size * dim * 4 + dim * 4 +
+           2 * L * (uint64_t)(pos + 1) * kvd * 4 + 2 * L * kvd * 4;
+}
+
+int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double *mean_us, uint64_t *bytes)
+{
+    if (!c || !mean_us) return fail(L2J_E_ARG, "null argument");
+    if (kclass < 0 || kclass >= L2J_K_COUNT || rounds <= 0) return fail(L2J_E_ARG, "bad kernel class or rounds");
+    int rc = check_forward_args(c, 1, pos);
+    if (rc) return rc;
+    const l2j_config &g = c->cfg;
+    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim;
+    uint64_t b = 0;
+    switch (kclass) {
+    case L2J_K_QKV: b = quant_bytes_of(dim * dim + 2 * dim * kvd) + quant_bytes_of(dim); break;
+    case L2J_K_ATTENTION: b = 2ull * (pos + 1) * kvd * 4; break;
+    case L2J_K_WO: b = quant_bytes_of(dim * dim); break;
+    case L2J_K_W13: b = quant_bytes_of(2 * dim * hid) + quant_bytes_of(dim); break;
+    case L2J_K_W2: b = quant_bytes_of(dim * hid); break;
+    case L2J_K_CLASSIFIER: b = (uint64_t)g.vocab_size * dim * 4 + quant_bytes_of(dim); break;
+    }
+    if (bytes) *bytes = b;
+    const int per_round = kclass == L2J_K_CLASSIFIER ? 1 : g.n_layers;
+    while ((int)c->events.size() < 2 * per_round + 33) {
+        hipEvent_t ev;
+        HIPCHK(hipEventCreate(&ev));
+        c->events.push_back(ev);
+    }
+    if ((rc = set_state(c, 1, pos, 0))) return rc;
+    // The activations hold whatever the last forward left; timing does not depend on their values.
+    // The classifier advances the device position, so the state is rewritten every round.
+    double total_ms = 0.0;
+    long count = 0;
+    for (int r = 0; r < rounds; r++) {
+        if ((rc = set_state(c, 1, pos, 0))) return rc;
+        for (int l = 0; l < per_round; l++) {
+            LayerPtrs p{};
+            if (kclass != L2J_K_CLASSIFIER) layer_args(c, l, p);
+            hipError_t e = launch_class(c, kclass, p, c->stream, c->events[33 + 2 * l], c->events[34 + 2 * l]);
+            if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
+        }
+        HIPCHK(hipStreamSynchronize(c->stream));
+        for (int l = 0; l < per_round; l++) {
+            float ms = 0.f;
+            HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * l], c->events[34 + 2 * l]));
+            total_ms += ms;
+            count++;
+        }
+    }
+    *mean_us = total_ms * 1e3 / (double)count;
+    return L2J_OK;
+}
+
+}  // extern "C"

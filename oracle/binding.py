@@ -17,6 +17,7 @@ GROUP_BYTES = 264
 
 T_RMS_ATT, T_WQ, T_WK, T_WV, T_WO, T_RMS_FFN, T_W1, T_W2, T_W3, T_RMS_FINAL = range(10)
 T_COUNT = 10
+TAP_Q, TAP_K, TAP_V, TAP_ATT_OUT, TAP_X_ATT, TAP_HB, TAP_X_FFN = range(7)
 B_X, B_XB, B_XB2, B_HB, B_HB2, B_Q, B_K, B_V, B_ATT, B_LOGITS, B_KCACHE, B_VCACHE, B_TMP1 = range(13)
 
 
@@ -79,6 +80,8 @@ def lib():
         "orc_model_wcls_ptr": (fp, [vp]),
         "orc_model_buffer": (fp, [vp, C.c_int]),
         "orc_model_reset": (None, [vp]),
+        "orc_model_enable_taps": (C.c_int, [vp]),
+        "orc_model_tap": (fp, [vp, C.c_int, C.c_int]),
         "orc_forward": (None, [vp, C.c_int, C.c_int]),
         "orc_forward_layers": (None, [vp, C.c_int, C.c_int, C.c_int]),
         "orc_generate_greedy": (C.c_int, [vp, i32p, C.c_int, C.c_int, i32p, fp, C.POINTER(C.c_double)]),
@@ -269,6 +272,14 @@ class Model:
              B_KCACHE: c.n_layers * c.seq_len * self.kv_dim, B_VCACHE: c.n_layers * c.seq_len * self.kv_dim,
              B_TMP1: max(c.dim, c.vocab_size) * 4}[which]
         return np.ctypeslib.as_array(lib().orc_model_buffer(self.h, which), shape=(n,))
+
+    def enable_taps(self):
+        if lib().orc_model_enable_taps(self.h):
+            raise MemoryError("taps")
+
+    def tap(self, which, layer):
+        n = self.cfg.hidden_dim if which == TAP_HB else self.kv_dim if which in (TAP_K, TAP_V) else self.cfg.dim
+        return np.ctypeslib.as_array(lib().orc_model_tap(self.h, which, layer), shape=(n,))
 
     def fill_synth(self, seed, sigma=0.02):
         lib().orc_model_fill_synth(self.h, seed, C.c_float(sigma))

@@ -453,6 +453,7 @@ struct orc_model {
     int64_t tmp1_len;
     float *rope_cos, *rope_sin;
     float silu_table[SILU_TABLE_SIZE];
+    float *taps[ORC_TAP_COUNT]; /* per-layer copies, NULL unless enabled */
 };
 
 static const char *const TENSOR_NAMES[ORC_T_COUNT] = {
@@ -538,6 +539,7 @@ orc_model *orc_model_new(const orc_config *cfg)
 void orc_model_free(orc_model *m)
 {
     if (!m) return;
+    for (int t = 0; t < ORC_TAP_COUNT; t++) free(m->taps[t]);
     for (int t = 0; t < ORC_T_COUNT; t++) free(m->quant[t]);
     if (m->wcls != m->emb) free(m->wcls);
     free(m->emb);
@@ -606,6 +608,36 @@ void orc_model_reset(orc_model *m)
     memset(m->att, 0, (size_t)m->cfg.n_heads * m->cfg.seq_len * sizeof(float));
 }
 
+static int64_t tap_len(const orc_model *m, int which)
+{
+    switch (which) {
+    case ORC_TAP_HB: return m->cfg.hidden_dim;
+    case ORC_TAP_K: case ORC_TAP_V: return m->kv_dim;
+    default: return m->cfg.dim;
+    }
+}
+
+int orc_model_enable_taps(orc_model *m)
+{
+    for (int t = 0; t < ORC_TAP_COUNT; t++) {
+        if (m->taps[t]) continue;
+        m->taps[t] = zalloc_f((int64_t)m->cfg.n_layers * tap_len(m, t));
+        if (!m->taps[t]) return -1;
+    }
+    return 0;
+}
+
+float *orc_model_tap(orc_model *m, int which, int layer)
+{
+    if (which < 0 || which >= ORC_TAP_COUNT || !m->taps[which]) return NULL;
+    return m->taps[which] + (int64_t)layer * tap_len(m, which);
+}
+
+static void tap(orc_model *m, int which, int layer, const float *src)
+{
+    if (m->taps[which]) memcpy(orc_model_tap(m, which, layer), src, (size_t)tap_len(m, which) * sizeof(float));
+}
+
 static void forward_impl(orc_model *m, int token, int pos, int n_layers_run, int run_head)
 {
     /* J/Run.java:62-169 */
@@ -631,6 +663,9 @@ static void forward_impl(orc_model *m, int token, int pos, int n_layers_run, int
         int64_t loff = (int64_t)l * p->seq_len * kv_dim;                                      /* :91 */
         memcpy(m->key_cache + loff + (int64_t)pos * kv_dim, m->k, (size_t)kv_dim * sizeof(float));   /* :95 */
         memcpy(m->value_cache + loff + (int64_t)pos * kv_dim, m->v, (size_t)kv_dim * sizeof(float)); /* :99 */
+        tap(m, ORC_TAP_Q, l, m->q);
+        tap(m, ORC_TAP_K, l, m->k);
+        tap(m, ORC_TAP_V, l, m->v);
 
 #pragma omp parallel for schedule(static)
         for (int h = 0; h < p->n_heads; h++) {                                                /* :102-131 */
@@ -647,8 +682,10 @@ static void forward_impl(orc_model *m, int token, int pos, int n_layers_run, int
                                      head_size, kv_dim, att_index);
         }
 
+        tap(m, ORC_TAP_ATT_OUT, l, m->xb);
         orc_matmul_i8(m->xb2, m->xb, m->quant[ORC_T_WO], (int64_t)l * dim * dim, dim, dim);    /* :134 */
         orc_accum(m->x, m->xb2, dim);                                                         /* :136 */
+        tap(m, ORC_TAP_X_ATT, l, m->x);
 
         orc_rms(m->tmp1, m->x, dim);                                                          /* :142 */
         orc_wns_i8(m->xb, m->x, m->quant[ORC_T_RMS_FFN], (int64_t)l * dim, m->tmp1, dim);     /* :143 */
@@ -657,9 +694,11 @@ static void forward_impl(orc_model *m, int token, int pos, int n_layers_run, int
         orc_matmul_i8(m->hb2, m->xb, m->quant[ORC_T_W3], (int64_t)l * dim * hidden_dim, dim, hidden_dim); /* :148 */
 
         orc_silu(m->hb, m->hb2, m->silu_table, hidden_dim);                                   /* :152 */
+        tap(m, ORC_TAP_HB, l, m->hb);
 
         orc_matmul_i8(m->xb, m->hb, m->quant[ORC_T_W2], (int64_t)l * dim * hidden_dim, hidden_dim, dim); /* :155 */
         orc_accum(m->x, m->xb, dim);                                                          /* :158 */
+        tap(m, ORC_TAP_X_FFN, l, m->x);
     }
     if (!run_head) return;
 

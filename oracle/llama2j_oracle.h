@@ -89,6 +89,12 @@ enum { ORC_B_X = 0, ORC_B_XB, ORC_B_XB2, ORC_B_HB, ORC_B_HB2, ORC_B_Q, ORC_B_K, 
 float *orc_model_buffer(orc_model *m, int which);
 void orc_model_reset(orc_model *m);                            /* zero KV cache and tmp1 (fresh RunState) */
 
+/* per-layer taps, copied during forward once enabled: q,k (after RoPE), v, attention output,
+ * x after the attention residual, SwiGLU output, x after the FFN residual */
+enum { ORC_TAP_Q = 0, ORC_TAP_K, ORC_TAP_V, ORC_TAP_ATT_OUT, ORC_TAP_X_ATT, ORC_TAP_HB, ORC_TAP_X_FFN, ORC_TAP_COUNT };
+int orc_model_enable_taps(orc_model *m);
+float *orc_model_tap(orc_model *m, int which, int layer);
+
 void orc_forward(orc_model *m, int token, int pos);            /* J/Run.java:62-169 */
 /* Like orc_forward but stops after `n_layers_run` layers and skips the head; for op-level taps. */
 void orc_forward_layers(orc_model *m, int token, int pos, int n_layers_run);
