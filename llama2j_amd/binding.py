@@ -64,7 +64,8 @@ class Config(C.Structure):
 
 
 def lib_path():
-    return os.path.join(_HERE, "libllama2j_hip.so")
+    """The in-tree library; L2J_LIB_PATH selects another build of the same ABI (kernel experiments)."""
+    return os.environ.get("L2J_LIB_PATH") or os.path.join(_HERE, "libllama2j_hip.so")
 
 
 def build_library():

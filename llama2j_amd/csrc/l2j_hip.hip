@@ -2,6 +2,7 @@
 // Owns device memory, converts the reference's weight formats to the streaming layout, captures
 // the per-token launch sequence as a hipGraph and replays it.
 #include "kernels.hpp"
+#include "phase_kernels.hpp"
 
 #include <hip/hip_ext.h>
 
@@ -70,10 +71,7 @@ struct l2j_ctx {
     float *kcache = nullptr, *vcache = nullptr;
     float2 *rope = nullptr;
     float *silu = nullptr;
-    float *attn_part = nullptr;
     unsigned *counters = nullptr;  // n_heads attention counters + 1 classifier counter
-    float *cls_val = nullptr;
-    int *cls_idx = nullptr;
     DevState *st = nullptr;
     int *prompt = nullptr, *out_tokens = nullptr;
     DevState *h_st = nullptr;  // pinned
@@ -82,8 +80,13 @@ struct l2j_ctx {
     // per-layer taps (allocated on first l2j_forward_taps)
     float *taps[L2J_B_COUNT] = {};
 
-    // launch shapes
-    int mv_threads = 512, mv_blocks_per_cu = 2, attn_nsplit = 32, attn_chunk_max = 0, cls_blocks = 512;
+
+    // launch shape of the phase kernels and their scratch
+    int pk_grid = 0, pk_threads = 1024, attn_threads = 256, attn_grid = 0, attn_nsplit = 1, attn_rows = 32;
+    float *cls_val = nullptr;
+    int *cls_idx = nullptr;
+    float *attn_part = nullptr;
+    float *rmsw = nullptr;  // dequantized rmsnorm weights: att (L*dim), ffn (L*dim), final (dim)
 
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -133,13 +136,6 @@ int dev_alloc(T **p, uint64_t count)
     return L2J_OK;
 }
 
-size_t mv_smem(int n) { return (size_t)n * 4 + (size_t)(n / 16) * 4 + 64 * sizeof(float); }
-
-struct LayerPtrs {
-    MatvecArgs qkv, wo, w13, w2;
-    AttnArgs attn;
-};
-
 QMat qmat(const l2j_ctx *c, int t, uint64_t off)
 {
     QMat m;
@@ -149,112 +145,100 @@ QMat qmat(const l2j_ctx *c, int t, uint64_t off)
     return m;
 }
 
-void layer_args(const l2j_ctx *c, int l, LayerPtrs &p)
+size_t mv_smem(int n) { return (size_t)n * 4 + (size_t)(n / 16) * 4 + 64 * sizeof(float); }
+
+int attn_lpr(const l2j_ctx *c) { return c->head_size <= 64 ? 16 : c->head_size <= 128 ? 32 : 64; }
+
+size_t attn_smem(const l2j_ctx *c)
 {
-    const l2j_config &g = c->cfg;
-    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim;
-    const uint64_t kvoff = (uint64_t)l * g.seq_len * kvd;
-
-    MatvecArgs a{};
-    a.xin = c->x; a.n = g.dim;
-    a.rms.codes = c->qt[L2J_RMS_ATT].codes; a.rms.mm = c->qt[L2J_RMS_ATT].mm; a.rms.off = (long)(l * dim);
-    a.m0 = qmat(c, L2J_WQ, l * dim * dim); a.m1 = qmat(c, L2J_WK, l * dim * kvd); a.m2 = qmat(c, L2J_WV, l * dim * kvd);
-    a.d0 = g.dim; a.d1 = c->kv_dim; a.d2 = c->kv_dim;
-    a.out0 = c->q; a.out1 = c->kcache + kvoff; a.out2 = c->vcache + kvoff;
-    a.rope = c->rope; a.head_size = c->head_size; a.kv_dim = c->kv_dim;
-    a.silu_table = c->silu; a.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0; a.st = c->st;
-    p.qkv = a;
-
-    AttnArgs t{};
-    t.q = c->q; t.kc = c->kcache + kvoff; t.vc = c->vcache + kvoff; t.out = c->xb; t.part = c->attn_part;
-    t.counters = c->counters; t.st = c->st; t.n_heads = g.n_heads; t.kv_mul = c->kv_mul; t.head_size = c->head_size;
-    t.kv_dim = c->kv_dim; t.nsplit = c->attn_nsplit; t.chunk_max = c->attn_chunk_max;
-    t.sqrt_hs = sqrtf((float)c->head_size);  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
-    p.attn = t;
-
-    MatvecArgs o = a;
-    o.xin = c->xb; o.n = g.dim; o.m0 = qmat(c, L2J_WO, l * dim * dim); o.d0 = g.dim; o.d1 = o.d2 = 0; o.out0 = c->x;
-    p.wo = o;
-
-    MatvecArgs f = a;
-    f.xin = c->x; f.n = g.dim;
-    f.rms.codes = c->qt[L2J_RMS_FFN].codes; f.rms.mm = c->qt[L2J_RMS_FFN].mm; f.rms.off = (long)(l * dim);
-    f.m0 = qmat(c, L2J_W1, l * dim * hid); f.m1 = qmat(c, L2J_W3, l * dim * hid); f.d0 = g.hidden_dim; f.d1 = g.hidden_dim; f.d2 = 0;
-    f.out0 = c->hb;
-    p.w13 = f;
-
-    MatvecArgs w = a;
-    w.xin = c->hb; w.n = g.hidden_dim; w.m0 = qmat(c, L2J_W2, l * dim * hid); w.d0 = g.dim; w.d1 = w.d2 = 0; w.out0 = c->x;
-    p.w2 = w;
+    const int nent = (c->attn_threads / 64) * (64 / attn_lpr(c));
+    return (size_t)(2 * nent + nent * c->head_size) * sizeof(float);
 }
 
-ClsArgs cls_args(const l2j_ctx *c)
+// Arguments of the phases of layer l (J/Run.java:76-159).
+MatvecPhase matvec_phase(const l2j_ctx *c, int kclass, int l)
 {
-    ClsArgs a{};
-    a.xin = c->x; a.n = c->cfg.dim;
-    a.rms.codes = c->qt[L2J_RMS_FINAL].codes; a.rms.mm = c->qt[L2J_RMS_FINAL].mm; a.rms.off = 0;
-    a.w = c->wcls; a.vocab = c->cfg.vocab_size; a.logits = c->logits;
-    a.part_val = c->cls_val; a.part_idx = c->cls_idx; a.counter = c->counters + c->cfg.n_heads;
+    const l2j_config &g = c->cfg;
+    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim, L = g.n_layers;
+    const uint64_t kvoff = (uint64_t)l * g.seq_len * kvd;
+    MatvecPhase d{};
+    d.emb = c->emb; d.rope = c->rope; d.silu = c->silu; d.st = c->st;
+    d.head_size = c->head_size; d.kv_dim = c->kv_dim; d.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0;
+    switch (kclass) {
+    case L2J_K_QKV:
+        d.n = g.dim; d.from_emb = l == 0; d.xin = c->x; d.rmsw = c->rmsw + (uint64_t)l * dim;
+        d.d0 = g.dim; d.d1 = d.d2 = c->kv_dim;
+        d.m0 = qmat(c, L2J_WQ, l * dim * dim); d.m1 = qmat(c, L2J_WK, l * dim * kvd); d.m2 = qmat(c, L2J_WV, l * dim * kvd);
+        d.out0 = c->q; d.out1 = c->kcache + kvoff; d.out2 = c->vcache + kvoff;
+        break;
+    case L2J_K_WO:
+        d.n = g.dim; d.xin = c->xb; d.d0 = g.dim; d.m0 = qmat(c, L2J_WO, l * dim * dim);
+        d.out0 = c->x; d.res_src = c->x; d.res_emb = l == 0;
+        break;
+    case L2J_K_W13:
+        d.n = g.dim; d.xin = c->x; d.rmsw = c->rmsw + (L + l) * dim; d.d0 = g.hidden_dim;
+        d.m0 = qmat(c, L2J_W1, l * dim * hid); d.m1 = qmat(c, L2J_W3, l * dim * hid); d.out0 = c->hb;
+        break;
+    default:  // L2J_K_W2
+        d.n = g.hidden_dim; d.xin = c->hb; d.d0 = g.dim; d.m0 = qmat(c, L2J_W2, l * dim * hid);
+        d.out0 = c->x; d.res_src = c->x;
+        break;
+    }
+    return d;
+}
+
+AttnPhase attn_phase(const l2j_ctx *c, int l)
+{
+    const uint64_t kvoff = (uint64_t)l * c->cfg.seq_len * c->kv_dim;
+    AttnPhase t{};
+    t.q = c->q; t.kc = c->kcache + kvoff; t.vc = c->vcache + kvoff; t.out = c->xb; t.part = c->attn_part;
+    t.counters = c->counters; t.st = c->st; t.n_heads = c->cfg.n_heads; t.kv_mul = c->kv_mul; t.head_size = c->head_size;
+    t.kv_dim = c->kv_dim; t.nsplit = c->attn_nsplit; t.rows_per_split = c->attn_rows;
+    t.sqrt_hs = sqrtf((float)c->head_size);  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
+    return t;
+}
+
+ClsPhase cls_phase(const l2j_ctx *c)
+{
+    ClsPhase a{};
+    a.xin = c->x; a.rmsw = c->rmsw + 2ull * c->cfg.n_layers * c->cfg.dim; a.w = c->wcls; a.n = c->cfg.dim; a.vocab = c->cfg.vocab_size;
+    a.logits = c->logits; a.part_val = c->cls_val; a.part_idx = c->cls_idx; a.nparts = c->pk_grid;
     a.st = c->st; a.prompt = c->prompt; a.out_tokens = c->out_tokens;
     return a;
 }
 
-int mv_grid(const l2j_ctx *c, int npairs)
-{
-    const int wpb = c->mv_threads / 64;
-    return std::max(1, std::min((npairs + wpb - 1) / wpb, c->n_cu * c->mv_blocks_per_cu));
-}
-
-struct Launch {
-    dim3 grid, block;
-    size_t smem;
-};
-
-Launch shape_of(const l2j_ctx *c, int kclass)
-{
-    const l2j_config &g = c->cfg;
-    Launch L{};
-    L.block = dim3(c->mv_threads);
-    switch (kclass) {
-    case L2J_K_QKV: L.grid = dim3(mv_grid(c, (g.dim + 2 * c->kv_dim) / 2)); L.smem = mv_smem(g.dim); break;
-    case L2J_K_WO: L.grid = dim3(mv_grid(c, (g.dim + 1) / 2)); L.smem = mv_smem(g.dim); break;
-    case L2J_K_W13: L.grid = dim3(mv_grid(c, g.hidden_dim)); L.smem = mv_smem(g.dim); break;
-    case L2J_K_W2: L.grid = dim3(mv_grid(c, (g.dim + 1) / 2)); L.smem = mv_smem(g.hidden_dim); break;
-    case L2J_K_CLASSIFIER: L.grid = dim3(c->cls_blocks); L.smem = mv_smem(g.dim) + 64 * sizeof(float); break;
-    case L2J_K_ATTENTION:
-        L.grid = dim3(g.n_heads * c->attn_nsplit);
-        L.block = dim3(kAttnThreads);
-        L.smem = (size_t)(c->attn_chunk_max + kAttnThreads / 64 + (kAttnThreads / 64) * c->head_size) * sizeof(float);
-        break;
-    }
-    return L;
-}
-
 template <typename K, typename A>
-hipError_t launch1(K kernel, const Launch &L, hipStream_t s, const A &args, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
+hipError_t launch1(K kernel, dim3 grid, dim3 block, size_t smem, hipStream_t s, const A &args, hipEvent_t e0, hipEvent_t e1)
 {
     if (e0) {
-        hipExtLaunchKernelGGL(kernel, L.grid, L.block, (unsigned)L.smem, s, e0, e1, 0, args);
+        hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)smem, s, e0, e1, 0, args);
     } else {
-        hipLaunchKernelGGL(kernel, L.grid, L.block, L.smem, s, args);
+        hipLaunchKernelGGL(kernel, grid, block, smem, s, args);
     }
     return hipGetLastError();
 }
 
-hipError_t launch_class(const l2j_ctx *c, int kclass, const LayerPtrs &p, hipStream_t s, hipEvent_t e0 = nullptr,
-                        hipEvent_t e1 = nullptr)
+// One kernel class of layer l.  Optional start/stop events bracket the kernel itself.
+hipError_t launch_class(const l2j_ctx *c, int kclass, int l, hipStream_t s, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
 {
-    const Launch L = shape_of(c, kclass);
+    const dim3 grid(c->pk_grid), block(c->pk_threads);
     switch (kclass) {
-    case L2J_K_QKV: return launch1(k_matvec<MV_QKV>, L, s, p.qkv, e0, e1);
-    case L2J_K_WO: return launch1(k_matvec<MV_RES>, L, s, p.wo, e0, e1);
-    case L2J_K_W13: return launch1(k_matvec<MV_W13>, L, s, p.w13, e0, e1);
-    case L2J_K_W2: return launch1(k_matvec<MV_RES>, L, s, p.w2, e0, e1);
-    case L2J_K_ATTENTION:
-        if (c->head_size <= 64) return launch1(k_attention<16>, L, s, p.attn, e0, e1);
-        if (c->head_size <= 128) return launch1(k_attention<32>, L, s, p.attn, e0, e1);
-        return launch1(k_attention<64>, L, s, p.attn, e0, e1);
-    case L2J_K_CLASSIFIER: return launch1(k_classifier, L, s, cls_args(c), e0, e1);
+    case L2J_K_QKV: return launch1(k_matvec<PH_QKV>, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
+    case L2J_K_W13: return launch1(k_matvec<PH_W13>, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
+    case L2J_K_WO:
+    case L2J_K_W2: {
+        const int n = kclass == L2J_K_WO ? c->cfg.dim : c->cfg.hidden_dim;
+        return launch1(k_matvec<PH_RES>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
+    }
+    case L2J_K_ATTENTION: {
+        const dim3 ag(c->attn_grid), ab(c->attn_threads);
+        const int lpr = attn_lpr(c);
+        if (lpr == 16) return launch1(k_attention<16>, ag, ab, attn_smem(c), s, attn_phase(c, l), e0, e1);
+        if (lpr == 32) return launch1(k_attention<32>, ag, ab, attn_smem(c), s, attn_phase(c, l), e0, e1);
+        return launch1(k_attention<64>, ag, ab, attn_smem(c), s, attn_phase(c, l), e0, e1);
+    }
+    case L2J_K_CLASSIFIER:
+        return launch1(k_classifier, grid, block, mv_smem(c->cfg.dim), s, cls_phase(c), e0, e1);
     }
     return hipErrorInvalidValue;
 }
@@ -264,36 +248,38 @@ hipError_t tap_copy(l2j_ctx *c, int which, int l, const float *src, uint64_t n, 
     return hipMemcpyAsync(c->taps[which] + (uint64_t)l * n, src, n * sizeof(float), hipMemcpyDeviceToDevice, s);
 }
 
-// The launch sequence of one token (J/Run.java:62-169).  With taps, per-layer copies follow each kernel.
+// The launch sequence of one token (J/Run.java:62-169).  With taps, per-layer copies follow each
+// kernel (the pattern of Mode.TEST).
 hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
 {
     const l2j_config &g = c->cfg;
     hipError_t e;
-    hipLaunchKernelGGL(k_embed, dim3((g.dim / 4 + 255) / 256), dim3(256), 0, s, c->emb, c->st, c->x, g.dim);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
     for (int l = 0; l < g.n_layers; l++) {
-        LayerPtrs p;
-        layer_args(c, l, p);
-        if ((e = launch_class(c, L2J_K_QKV, p, s)) != hipSuccess) return e;
-        if ((e = launch_class(c, L2J_K_ATTENTION, p, s)) != hipSuccess) return e;
-        if (taps) {
-            // rows of the caches at the current position; pos is known on the host in this mode
+        const uint64_t kvoff = (uint64_t)l * g.seq_len * c->kv_dim;
+        if ((e = launch_class(c, L2J_K_QKV, l, s)) != hipSuccess) return e;
+        if (taps) {  // rows of the caches at the current position; pos is known on the host in this mode
             const uint64_t row = (uint64_t)c->h_st->pos * c->kv_dim;
             if ((e = tap_copy(c, L2J_B_Q, l, c->q, g.dim, s)) != hipSuccess) return e;
-            if ((e = tap_copy(c, L2J_B_K, l, p.qkv.out1 + row, c->kv_dim, s)) != hipSuccess) return e;
-            if ((e = tap_copy(c, L2J_B_V, l, p.qkv.out2 + row, c->kv_dim, s)) != hipSuccess) return e;
-            if ((e = tap_copy(c, L2J_B_XB, l, c->xb, g.dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_K, l, c->kcache + kvoff + row, c->kv_dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_V, l, c->vcache + kvoff + row, c->kv_dim, s)) != hipSuccess) return e;
         }
-        if ((e = launch_class(c, L2J_K_WO, p, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_ATTENTION, l, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_XB, l, c->xb, g.dim, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_WO, l, s)) != hipSuccess) return e;
         if (taps && (e = tap_copy(c, L2J_B_XB2, l, c->x, g.dim, s)) != hipSuccess) return e;
-        if ((e = launch_class(c, L2J_K_W13, p, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_W13, l, s)) != hipSuccess) return e;
         if (taps && (e = tap_copy(c, L2J_B_HB, l, c->hb, g.hidden_dim, s)) != hipSuccess) return e;
-        if ((e = launch_class(c, L2J_K_W2, p, s)) != hipSuccess) return e;
+        if ((e = launch_class(c, L2J_K_W2, l, s)) != hipSuccess) return e;
         if (taps && (e = tap_copy(c, L2J_B_X, l, c->x, g.dim, s)) != hipSuccess) return e;
     }
-    LayerPtrs none{};
-    return launch_class(c, L2J_K_CLASSIFIER, none, s);
+    if ((e = launch_class(c, L2J_K_CLASSIFIER, 0, s)) != hipSuccess) return e;
+    hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, s, cls_phase(c));
+    return hipGetLastError();
 }
+
+hipError_t launch_one_token(l2j_ctx *c) { return hipGraphLaunch(c->graph_exec, c->stream); }
+
+int check_barrier_error(l2j_ctx *) { return L2J_OK; }
 
 int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
 {
@@ -387,12 +373,6 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     c->kv_mul = cfg->n_heads / cfg->n_kv_heads;
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, cfg->device) == hipSuccess && prop.multiProcessorCount > 0) c->n_cu = prop.multiProcessorCount;
-    c->mv_threads = std::min(1024, std::max(64, env_int("L2J_MV_THREADS", 512) / 64 * 64));
-    c->mv_blocks_per_cu = std::max(1, env_int("L2J_MV_BLOCKS_PER_CU", 2));
-    c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
-    c->cls_blocks = std::max(1, std::min(env_int("L2J_CLS_BLOCKS", c->n_cu * c->mv_blocks_per_cu), (cfg->vocab_size + 1) / 2));
-    int cm = std::max((cfg->seq_len + c->attn_nsplit - 1) / c->attn_nsplit, kAttnMinChunk);
-    c->attn_chunk_max = (cm + 3) / 4 * 4;
 
 #define TRY(expr)                \
     do {                         \
@@ -435,10 +415,7 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     TRY(dev_alloc(&c->vcache, kvn));
     TRY(dev_alloc(&c->rope, (uint64_t)cfg->seq_len * (c->head_size / 2)));
     TRY(dev_alloc(&c->silu, kSiluTable));
-    TRY(dev_alloc(&c->attn_part, (uint64_t)cfg->n_heads * c->attn_nsplit * (c->head_size + 2)));
     TRY(dev_alloc(&c->counters, cfg->n_heads + 1));
-    TRY(dev_alloc(&c->cls_val, c->cls_blocks));
-    TRY(dev_alloc(&c->cls_idx, c->cls_blocks));
     TRY(dev_alloc(&c->st, 1));
     TRY(dev_alloc(&c->prompt, cfg->seq_len));
     TRY(dev_alloc(&c->out_tokens, cfg->seq_len));
@@ -450,14 +427,6 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     TRYHIP(hipMemset(c->st, 0, sizeof(DevState)));
     TRYHIP(hipMemset(c->kcache, 0, kvn * sizeof(float)));
     TRYHIP(hipMemset(c->vcache, 0, kvn * sizeof(float)));
-    // dynamic LDS above the default limit (large hidden_dim)
-    const int need = (int)mv_smem(std::max(cfg->dim, cfg->hidden_dim)) + 256;
-    if (need > 64 * 1024) {
-        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_RES>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
-        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_QKV>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
-        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_matvec<MV_W13>), hipFuncAttributeMaxDynamicSharedMemorySize, need));
-        TRYHIP(hipFuncSetAttribute(reinterpret_cast<const void *>(k_classifier), hipFuncAttributeMaxDynamicSharedMemorySize, need));
-    }
 #undef TRY
 #undef TRYHIP
     *out = c;
@@ -478,11 +447,14 @@ void l2j_destroy(l2j_ctx *c)
     }
     if (c->wcls != c->emb) (void)hipFree(c->wcls);
     (void)hipFree(c->emb);
-    float *bufs[] = {c->x, c->xb, c->hb, c->q, c->logits, c->kcache, c->vcache, c->silu, c->attn_part, c->cls_val};
+    float *bufs[] = {c->x, c->xb, c->hb, c->q, c->logits, c->kcache, c->vcache, c->silu};
     for (float *b : bufs) (void)hipFree(b);
     (void)hipFree(c->rope);
-    (void)hipFree(c->counters);
+    (void)hipFree(c->cls_val);
     (void)hipFree(c->cls_idx);
+    (void)hipFree(c->attn_part);
+    (void)hipFree(c->rmsw);
+    (void)hipFree(c->counters);
     (void)hipFree(c->st);
     (void)hipFree(c->prompt);
     (void)hipFree(c->out_tokens);
@@ -664,7 +636,44 @@ int l2j_finalize(l2j_ctx *c)
     }
     HIPCHK(hipMemcpy(c->silu, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice));
 
-    // capture the token
+    // rmsnorm weights dequantized once with the reference's expression
+    {
+        const uint64_t dim = c->cfg.dim, L = c->cfg.n_layers;
+        int rc2;
+        if ((rc2 = dev_alloc(&c->rmsw, (2 * L + 1) * dim))) return rc2;
+        const int src[3] = {L2J_RMS_ATT, L2J_RMS_FFN, L2J_RMS_FINAL};
+        float *dst[3] = {c->rmsw, c->rmsw + L * dim, c->rmsw + 2 * L * dim};
+        for (int i = 0; i < 3; i++) {
+            const long n = (long)c->qt[src[i]].nfloats;
+            hipLaunchKernelGGL(k_dequant_rms, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, c->stream, c->qt[src[i]].codes,
+                               c->qt[src[i]].mm, n, dst[i]);
+            HIPCHK(hipGetLastError());
+        }
+    }
+    // launch shapes: one 1024-thread workgroup per compute unit for the weight-streaming kernels
+    {
+        const int nmax = std::max(c->cfg.dim, c->cfg.hidden_dim);
+        c->pk_threads = std::min(1024, std::max(64, env_int("L2J_THREADS", 1024) / 64 * 64));
+        c->pk_grid = std::max(1, env_int("L2J_GRID", c->n_cu * std::max(1, 1024 / c->pk_threads)));
+        c->attn_threads = std::min(1024, std::max(64, env_int("L2J_ATTN_THREADS", 256) / 64 * 64));
+        c->attn_rows = std::max(1, env_int("L2J_ATTN_ROWS", 32));
+        c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
+        c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
+        const size_t need = std::max(mv_smem(nmax), attn_smem(c));
+        if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
+        if (need > 64 * 1024) {
+            const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
+                                reinterpret_cast<const void *>(k_matvec<PH_RES>),
+                                reinterpret_cast<const void *>(k_classifier)};
+            for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
+        }
+        int rc2;
+        if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
+        if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
+        if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
+    }
+
+    // capture one token
     HIPCHK(hipStreamSynchronize(c->stream));
     HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
     hipError_t le = launch_token(c, c->stream, false);
@@ -700,10 +709,10 @@ int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
     int rc = check_forward_args(c, token, pos);
     if (rc) return rc;
     if ((rc = set_state(c, token, pos, 0))) return rc;
-    HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+    HIPCHK(launch_one_token(c));
     if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
-    return L2J_OK;
+    return check_barrier_error(c);
 }
 
 int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
@@ -712,11 +721,11 @@ int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
     int rc = check_forward_args(c, token, pos);
     if (rc) return rc;
     if ((rc = set_state(c, token, pos, 0))) return rc;
-    HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+    HIPCHK(launch_one_token(c));
     HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
     *next = c->h_tokens[0];
-    return L2J_OK;
+    return check_barrier_error(c);
 }
 
 int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
@@ -772,12 +781,13 @@ int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32
     while (pos < steps && !stopped) {
         const int nb = std::min(batch, steps - pos);
         for (int i = 0; i < nb; i++) {
-            HIPCHK(hipGraphLaunch(c->graph_exec, c->stream));
+            HIPCHK(launch_one_token(c));
             if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
             HIPCHK(hipEventRecord(c->events[i], c->stream));
         }
         HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
         HIPCHK(hipStreamSynchronize(c->stream));
+        if ((rc = check_barrier_error(c))) return rc;
         int used = nb;
         for (int i = 0; i < nb; i++) {
             out_tokens[pos + i] = c->h_tokens[i];
@@ -876,17 +886,13 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
         HIPCHK(hipEventCreate(&ev));
         c->events.push_back(ev);
     }
-    if ((rc = set_state(c, 1, pos, 0))) return rc;
     // The activations hold whatever the last forward left; timing does not depend on their values.
-    // The classifier advances the device position, so the state is rewritten every round.
     double total_ms = 0.0;
     long count = 0;
     for (int r = 0; r < rounds; r++) {
         if ((rc = set_state(c, 1, pos, 0))) return rc;
         for (int l = 0; l < per_round; l++) {
-            LayerPtrs p{};
-            if (kclass != L2J_K_CLASSIFIER) layer_args(c, l, p);
-            hipError_t e = launch_class(c, kclass, p, c->stream, c->events[33 + 2 * l], c->events[34 + 2 * l]);
+            hipError_t e = launch_class(c, kclass, l, c->stream, c->events[33 + 2 * l], c->events[34 + 2 * l]);
             if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
         }
         HIPCHK(hipStreamSynchronize(c->stream));

@@ -1,0 +1,489 @@
+// The per-token forward pass (J/Run.java:62-169) as a chain of gfx950 kernels, one per phase:
+//   per layer   k_matvec<PH_QKV>   rmsnorm + Wq,Wk,Wv matvec + RoPE + KV-cache store
+//               k_attention        decode attention, split over the sequence, online softmax
+//               k_matvec<PH_RES>   Wo matvec + residual
+//               k_matvec<PH_W13>   rmsnorm + W1,W3 matvec + SwiGLU (the reference's sigmoid table)
+//               k_matvec<PH_RES>   W2 matvec + residual
+//   once        k_classifier       final rmsnorm + fp32 classifier + per-workgroup first-max
+//               k_finish           fold the maxima, step the token loop state
+// captured once in a hipGraph and replayed per token.
+//
+// Every kernel is HBM-bandwidth bound (batch-1 GEMV: no reuse, so no MFMA): int8 codes are streamed
+// with 16-byte nontemporal loads, one wavefront per pair of sub-rows, the activation vector is staged
+// in LDS once per workgroup (one 1024-thread workgroup per compute unit), accumulation is fp32 and the
+// 64-lane reduction uses DPP.  All arguments are passed by value so that every pointer is a kernel
+// argument (global address space, scalar base + 32-bit lane offset addressing).
+#pragma once
+
+#include "kernels.hpp"
+
+namespace l2j {
+
+__device__ __forceinline__ float ld_coh(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coh(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int ld_coh(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coh(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2 };
+
+// One matvec phase.  Passed by value.
+struct MatvecPhase {
+    int n;          // input vector length (multiple of 16)
+    int from_emb;   // the input vector is the embedding row of the current token (QKV of layer 0)
+    int res_emb;    // PH_RES: the residual input is the embedding row of the current token (Wo of layer 0)
+    int d0, d1, d2; // rows: QKV (dim, kv_dim, kv_dim); W13 (hidden); RES (dim)
+    const float *xin;   // input vector (ignored when from_emb)
+    const float *rmsw;  // dequantized rmsnorm weights (fp32) or null: input = rmsw[e] * (ss * x[e])
+    QMat m0, m1, m2;
+    float *out0, *out1, *out2;  // QKV: q, key cache of the layer, value cache of the layer; W13: hb; RES: x
+    const float *res_src;       // PH_RES: residual input (ignored when res_emb)
+    const float *emb;           // token embedding table
+    const float2 *rope;         // (cos, sin) at [pos * head_size/2 + (i % head_size)/2]
+    const float *silu;          // sigmoid table
+    const DevState *st;
+    int head_size, kv_dim, exact_silu;
+};
+
+// ---- activation vector -> LDS ------------------------------------------------------------------
+// LDS layout for an n-float vector (nch = n/16 chunks): float4 xs[q*nch + c] holds x[16c+4q .. 16c+4q+3],
+// so that lane c of a wave reads consecutive 16-byte words for a fixed q (bank-conflict free);
+// sumx[c] = sum of the 16 activations of chunk c (for the group-minimum term of the dequantization).
+
+__device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
+                                             float *sumx, float *red)
+{
+    const int nch = n >> 4, tid = threadIdx.x, T = blockDim.x;
+    if (rmsw) {
+        float ssq = 0.0f;
+        for (int c = tid; c < nch; c += T) {
+            const float4 *xp = reinterpret_cast<const float4 *>(xin + 16 * c);
+            const float4 a = xp[0], b = xp[1], cc = xp[2], d = xp[3];
+            xs[c] = a;
+            xs[nch + c] = b;
+            xs[2 * nch + c] = cc;
+            xs[3 * nch + c] = d;
+            ssq += (a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w) + (b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w) +
+                   (cc.x * cc.x + cc.y * cc.y + cc.z * cc.z + cc.w * cc.w) + (d.x * d.x + d.y * d.y + d.z * d.z + d.w * d.w);
+        }
+        ssq = block_sum(ssq, red);
+        // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
+        const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
+        for (int c = tid; c < nch; c += T) {
+            const float4 *wp = reinterpret_cast<const float4 *>(rmsw + 16 * c);
+            float s = 0.0f;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                float4 xv = xs[q * nch + c];
+                const float4 wv = wp[q];
+                // out = weight * (ss * x)   (K/WeightNormalizeAndScale.java:73)
+                xv.x = __fmul_rn(wv.x, __fmul_rn(ss, xv.x));
+                xv.y = __fmul_rn(wv.y, __fmul_rn(ss, xv.y));
+                xv.z = __fmul_rn(wv.z, __fmul_rn(ss, xv.z));
+                xv.w = __fmul_rn(wv.w, __fmul_rn(ss, xv.w));
+                s += (xv.x + xv.y) + (xv.z + xv.w);
+                xs[q * nch + c] = xv;
+            }
+            sumx[c] = s;
+        }
+    } else {
+        for (int c = tid; c < nch; c += T) {
+            const float4 *xp = reinterpret_cast<const float4 *>(xin + 16 * c);
+            const float4 a = xp[0], b = xp[1], cc = xp[2], d = xp[3];
+            xs[c] = a;
+            xs[nch + c] = b;
+            xs[2 * nch + c] = cc;
+            xs[3 * nch + c] = d;
+            sumx[c] = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w)) + ((cc.x + cc.y) + (cc.z + cc.w)) +
+                      ((d.x + d.y) + (d.z + d.w));
+        }
+    }
+    __syncthreads();
+}
+
+// ---- W8A32 matvec: an item is a pair of rows, one wavefront per item ---------------------------------
+
+constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
+
+template <int MODE>
+__global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
+{
+    extern __shared__ float4 smem4[];
+    const int n = d.n, nch = n >> 4;
+    float4 *xs = smem4;
+    float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
+    float *red = sumx + nch;  // 16 floats
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int W = blockDim.x >> 6, G = gridDim.x;
+    const int token = d.st->token, pos = d.st->pos;
+    const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
+
+    const int nitems = MODE == PH_QKV ? (d.d0 + d.d1 + d.d2) >> 1 : MODE == PH_RES ? (d.d0 + 1) >> 1 : d.d0;
+    const float *res = d.res_emb ? emb_row : d.res_src;
+
+    // The codes of an item: two sub-rows, each a scalar base pointer + the lane's 16-byte chunk index.
+    const uint8_t *cb0 = nullptr, *cb1 = nullptr;  // first code of each sub-row (uniform)
+    const float2 *gb0 = nullptr, *gb1 = nullptr;   // scale entry of the group holding that code
+    unsigned r0 = 0, r1 = 0;                       // position of that code inside its group
+    int which = 0, r = 0;
+    bool has1 = true;
+    auto resolve = [&](int item) {
+        long f0, f1;
+        QMat m = d.m0, mb = d.m0;
+        which = 0;
+        has1 = true;
+        if (MODE == PH_QKV) {  // rows (2p, 2p+1) of q, k or v: RoPE rotates the pair
+            r = 2 * item;
+            if (r >= d.d0 + d.d1) { which = 2; r -= d.d0 + d.d1; m = d.m2; }
+            else if (r >= d.d0) { which = 1; r -= d.d0; m = d.m1; }
+            mb = m;
+            f0 = m.off + (long)r * n;
+            f1 = f0 + n;
+        } else if (MODE == PH_W13) {  // row p of w1 and row p of w3: SwiGLU needs both
+            r = item;
+            mb = d.m1;
+            f0 = m.off + (long)r * n;
+            f1 = mb.off + (long)r * n;
+        } else {  // rows (2p, 2p+1)
+            r = 2 * item;
+            has1 = r + 1 < d.d0;
+            f0 = m.off + (long)r * n;
+            f1 = has1 ? f0 + n : f0;
+        }
+        cb0 = m.codes + f0; gb0 = m.gs + (f0 >> 8); r0 = (unsigned)(f0 & 255);
+        cb1 = mb.codes + f1; gb1 = mb.gs + (f1 >> 8); r1 = (unsigned)(f1 & 255);
+    };
+    uint4 w0[kTU], w1[kTU];
+    float2 s0[kTU], s1[kTU];
+    auto issue = [&](int base) {
+#pragma unroll
+        for (int u = 0; u < kTU; u++) {
+            const int c = base + 64 * u + lane;
+            const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 below)
+            w0[u] = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
+            w1[u] = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc);
+            s0[u] = gb0[(r0 + 16u * cc) >> 8];
+            s1[u] = gb1[(r1 + 16u * cc) >> 8];
+        }
+    };
+
+    // Items are dealt block-minor (item -> workgroup item % G), so every compute unit gets the same
+    // number of rows even when the rows do not fill all waves.
+    int item = wave * G + blockIdx.x;
+    // The weights do not depend on the input vector: the first loads go out before it is staged, so
+    // HBM latency overlaps the rmsnorm prologue.
+    bool first = item < nitems;
+    if (first) {
+        resolve(item);
+        issue(0);
+    }
+    stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red);
+
+    for (; item < nitems; item += W * G) {
+        if (!first) resolve(item);
+        float resv0 = 0.0f, resv1 = 0.0f;
+        if (MODE == PH_RES && lane == 0) {  // in flight while the row streams
+            resv0 = res[r];
+            if (has1) resv1 = res[r + 1];
+        }
+        float acc0 = 0.0f, acc1 = 0.0f;
+        for (int base = 0; base < nch; base += 64 * kTU) {
+            if (!(first && base == 0)) issue(base);
+#pragma unroll
+            for (int u = 0; u < kTU; u++) {
+                const int c = base + 64 * u + lane;
+                const bool ok = c < nch;
+                const int cc = ok ? c : nch - 1;
+                const float4 x0 = xs[cc], x1 = xs[nch + cc], x2 = xs[2 * nch + cc], x3 = xs[3 * nch + cc];
+                const float sx = sumx[cc];
+                // sum (code*rm + min)*x = rm * sum code*x + min * sum x over the chunk
+                const float t0 = fmaf(s0[u].x, dot16(w0[u], x0, x1, x2, x3), s0[u].y * sx);
+                const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
+                acc0 += ok ? t0 : 0.0f;
+                acc1 += ok ? t1 : 0.0f;
+            }
+        }
+        first = false;
+        acc0 = wave_sum(acc0);
+        acc1 = wave_sum(acc1);
+        if (lane == 0) {
+            if (MODE == PH_QKV) {
+                float v0 = acc0, v1 = acc1;
+                if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
+                    const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
+                    v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
+                    v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
+                }
+                float *dst = which == 0 ? d.out0 + r : (which == 1 ? d.out1 : d.out2) + (long)pos * d.kv_dim + r;
+                dst[0] = v0;
+                dst[1] = v1;
+            } else if (MODE == PH_W13) {
+                const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
+                d.out0[r] = __fmul_rn(acc0, __fmul_rn(s, acc1));
+            } else {
+                d.out0[r] = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
+                if (has1) d.out0[r + 1] = __fadd_rn(resv1, acc1);
+            }
+        }
+    }
+}
+
+// ---- decode attention: workgroup = (head, split); waves share the split's rows; online softmax ----
+
+struct AttnPhase {
+    const float *q;        // (n_heads * head_size) after RoPE
+    const float *kc;       // this layer's key cache (seq_len, kv_dim)
+    const float *vc;       // this layer's value cache
+    float *out;            // xb (dim)
+    float *part;           // (n_heads, nsplit, head_size + 2) partial (max, sum, acc)
+    unsigned *counters;    // (n_heads) arrival counters, zero between launches
+    const DevState *st;
+    int n_heads, kv_mul, head_size, kv_dim, nsplit, rows_per_split;
+    float sqrt_hs;
+};
+
+constexpr int kAU = 2;  // cache rows in flight per lane group (K and V each)
+
+// LPR = lanes per cache row: each lane owns 4 consecutive floats of the head (head_size <= 4*LPR).
+template <int LPR>
+__global__ void __launch_bounds__(1024) k_attention(const AttnPhase a)
+{
+    extern __shared__ float smem[];
+    constexpr int RPW = 64 / LPR;
+    const int hs = a.head_size, W = blockDim.x >> 6, tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nent = W * RPW;
+    float *sm_m = smem;                 // nent
+    float *sm_l = sm_m + nent;          // nent
+    float *sm_acc = sm_l + nent;        // nent * hs
+    __shared__ int s_last;
+
+    const int len = a.st->pos + 1;
+    int nsplit = (len + a.rows_per_split - 1) / a.rows_per_split;  // short contexts: fewer, fuller splits
+    if (nsplit > a.nsplit) nsplit = a.nsplit;
+    const int chunk = (len + nsplit - 1) / nsplit;
+    const int nact = (len + chunk - 1) / chunk;
+    const int j = lane % LPR, slot = wave * RPW + lane / LPR;
+    const bool active = 4 * j < hs;
+
+    for (int it = blockIdx.x; it < a.n_heads * nact; it += gridDim.x) {
+        const int h = it % a.n_heads, s = it / a.n_heads;
+        const int t0 = s * chunk, t1 = min(len, t0 + chunk);
+        const long col = (long)(h / a.kv_mul) * hs + 4 * j;
+        float4 q4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (active) q4 = *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
+        float m = -3.402823466e+38f, l = 0.0f;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int tb = t0 + slot; tb < t1; tb += nent * kAU) {
+            float4 k4[kAU], v4[kAU];
+            bool ok[kAU];
+#pragma unroll
+            for (int u = 0; u < kAU; u++) {
+                const int t = tb + u * nent;
+                ok[u] = t < t1;
+                k4[u] = v4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (ok[u] && active) {
+                    k4[u] = load_stream(reinterpret_cast<const float4 *>(a.kc + (long)t * a.kv_dim + col));
+                    v4[u] = load_stream(reinterpret_cast<const float4 *>(a.vc + (long)t * a.kv_dim + col));
+                }
+            }
+            float sc[kAU], mb = m;
+#pragma unroll
+            for (int u = 0; u < kAU; u++) {
+                // att[t] = (q . k_t) / sqrt(head_size)   (K/AttentionLoop.java:36-48)
+                sc[u] = __fdiv_rn(group_sum<LPR>(dot4(q4, k4[u])), a.sqrt_hs);
+                if (ok[u]) mb = fmaxf(mb, sc[u]);
+            }
+            // Online softmax, shifted by the running maximum of the scores.  The reference shifts by a
+            // running maximum of element products (K/AttentionLoop.java:44-51); softmax is shift
+            // invariant, so only rounding differs.
+            const float scale = expf(m - mb);  // 0 on the first batch (m = -FLT_MAX)
+            l *= scale;
+            acc.x *= scale; acc.y *= scale; acc.z *= scale; acc.w *= scale;
+#pragma unroll
+            for (int u = 0; u < kAU; u++) {
+                const float p = ok[u] ? expf(sc[u] - mb) : 0.0f;
+                l += p;
+                acc.x = fmaf(p, v4[u].x, acc.x);  // K/AccumWeightedValue.java:48-62
+                acc.y = fmaf(p, v4[u].y, acc.y);
+                acc.z = fmaf(p, v4[u].z, acc.z);
+                acc.w = fmaf(p, v4[u].w, acc.w);
+            }
+            m = mb;
+        }
+        __syncthreads();  // LDS reuse across items
+        if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
+        if (active) *reinterpret_cast<float4 *>(sm_acc + slot * hs + 4 * j) = acc;
+        __syncthreads();
+        // fold the row slots in a fixed order, so the result does not depend on timing
+        float M = -3.402823466e+38f, L = 0.0f, o = 0.0f;
+        for (int e = 0; e < nent; e++) M = fmaxf(M, sm_m[e]);
+        if (tid < hs) {
+            for (int e = 0; e < nent; e++) {
+                const float w = expf(sm_m[e] - M);  // empty slots: exp(-huge) = 0
+                L = fmaf(sm_l[e], w, L);
+                o = fmaf(sm_acc[e * hs + tid], w, o);
+            }
+        }
+        if (nact == 1) {
+            if (tid < hs) a.out[h * hs + tid] = __fdiv_rn(o, L);
+            continue;
+        }
+        // Several splits: partials travel through memory with device-scope relaxed atomics (write-through
+        // stores, cache-bypassing loads), which is far cheaper here than a fence that writes back and
+        // invalidates the L2 of every XCD.  The split that arrives last folds them in split order.
+        float *mypart = a.part + ((long)h * a.nsplit + s) * (hs + 2);
+        if (tid < hs) st_coh(mypart + 2 + tid, o);
+        if (tid == 0) { st_coh(mypart, M); st_coh(mypart + 1, L); }
+        __syncthreads();  // the partial stores of every wave have completed
+        if (tid == 0) s_last = (__hip_atomic_fetch_add(a.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(nact - 1));
+        __syncthreads();
+        if (!s_last) continue;
+        const float *hp = a.part + (long)h * a.nsplit * (hs + 2);
+        if (tid < hs) {
+            float MM = -3.402823466e+38f, LL = 0.0f, oo = 0.0f;
+            for (int i0 = 0; i0 < nact; i0 += 8) {
+                float pm[8], pl[8], po[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float *pp = hp + (long)min(i0 + i, nact - 1) * (hs + 2);
+                    pm[i] = ld_coh(pp);
+                    pl[i] = ld_coh(pp + 1);
+                    po[i] = ld_coh(pp + 2 + tid);
+                }
+                float mb = MM;
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+                    if (i0 + i < nact) mb = fmaxf(mb, pm[i]);
+                const float scale = expf(MM - mb);
+                LL *= scale;
+                oo *= scale;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    if (i0 + i < nact) {
+                        const float w = expf(pm[i] - mb);
+                        LL = fmaf(pl[i], w, LL);
+                        oo = fmaf(po[i], w, oo);
+                    }
+                }
+                MM = mb;
+            }
+            a.out[h * hs + tid] = __fdiv_rn(oo, LL);
+        }
+        if (tid == 0) st_coh(a.counters + h, 0u);
+    }
+}
+
+// ---- final rmsnorm + fp32 classifier + per-workgroup first-max -----------------------------------
+
+struct ClsPhase {
+    const float *xin;    // residual stream
+    const float *rmsw;   // dequantized rms_final_weight
+    const float *w;      // (vocab, dim) fp32
+    int n, vocab;
+    float *logits;
+    float *part_val;     // one per workgroup
+    int *part_idx;
+    int nparts;
+    DevState *st;
+    const int *prompt;   // seq_len
+    int *out_tokens;     // seq_len
+};
+
+constexpr int kCU = 8;
+
+__global__ void __launch_bounds__(1024) k_classifier(const ClsPhase a)
+{
+    extern __shared__ float4 smem4[];
+    const int n = a.n, nch = n >> 4, n4 = n >> 2;
+    float4 *xs = smem4;
+    float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
+    float *red = sumx + nch;
+    float *bval = red + 16;
+    int *bidx = reinterpret_cast<int *>(red + 32);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int W = blockDim.x >> 6, G = gridDim.x;
+
+    stage_vector(a.xin, n, a.rmsw, xs, sumx, red);
+
+    float best_v = -__builtin_inff();
+    int best_i = 0x7fffffff;
+    for (int row = wave * G + blockIdx.x; row < a.vocab; row += W * G) {
+        const float4 *wr = reinterpret_cast<const float4 *>(a.w + (long)row * n);
+        float acc = 0.0f;
+        for (int base = 0; base < n4; base += 64 * kCU) {
+            float4 pre[kCU];
+#pragma unroll
+            for (int u = 0; u < kCU; u++) {
+                const int c = base + 64 * u + lane;
+                pre[u] = load_stream(wr + (c < n4 ? c : n4 - 1));
+            }
+#pragma unroll
+            for (int u = 0; u < kCU; u++) {
+                const int c = base + 64 * u + lane;
+                const bool ok = c < n4;
+                const int cc = ok ? c : n4 - 1;
+                const float t = dot4(pre[u], xs[(cc & 3) * nch + (cc >> 2)]);
+                acc += ok ? t : 0.0f;
+            }
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            a.logits[row] = acc;
+            if (better(acc, row, best_v, best_i)) { best_v = acc; best_i = row; }
+        }
+    }
+    if (lane == 0) { bval[wave] = best_v; bidx[wave] = best_i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < W; w++)
+            if (better(bval[w], bidx[w], best_v, best_i)) { best_v = bval[w]; best_i = bidx[w]; }
+        a.part_val[blockIdx.x] = best_v;
+        a.part_idx[blockIdx.x] = best_i;
+    }
+}
+
+// First index of the strict maximum (J/Sampler.java:46-57), then the token-loop step
+// (J/Run.java:635-642, 668, 680): forced prompt id or argmax, then advance.  One workgroup.
+__global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
+{
+    __shared__ float bval[16];
+    __shared__ int bidx[16];
+    float bv = -__builtin_inff();
+    int bi = 0x7fffffff;
+    for (int b = threadIdx.x; b < a.nparts; b += blockDim.x) {
+        const float v = a.part_val[b];
+        const int i = a.part_idx[b];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off);
+        const int oi = __shfl_xor(bi, off);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bval[threadIdx.x >> 6] = bv; bidx[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++)
+            if (better(bval[w], bidx[w], bv, bi)) { bv = bval[w]; bi = bidx[w]; }
+        if (bi == 0x7fffffff) bi = 0;  // all NaN: the reference's scan never leaves index 0
+        const int pos = a.st->pos;
+        const int next = pos < a.st->n_prompt ? a.prompt[pos] : bi;
+        a.out_tokens[pos] = next;
+        a.st->token = next;
+        a.st->pos = pos + 1;
+    }
+}
+
+// rmsnorm weights dequantized once (K/WeightNormalizeAndScale.java:71-72): value = byte / 255f * range + min
+__global__ void k_dequant_rms(const uint8_t *__restrict__ codes, const float2 *__restrict__ mm, long n, float *__restrict__ out)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float2 v = mm[i >> 8];
+        out[i] = __fadd_rn(__fmul_rn(__fdiv_rn((float)codes[i], 255.0f), __fsub_rn(v.y, v.x)), v.x);
+    }
+}
+
+}  // namespace l2j

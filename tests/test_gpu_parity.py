@@ -144,7 +144,7 @@ def test_per_layer_taps_match_oracle(orc, shape):
     np.testing.assert_array_equal(g.read(BUFFER.XB, layer=0), g.read(BUFFER.V, layer=0)[i // hs // kv_mul * hs + i % hs])
 
 
-def test_graph_replay_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
+def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
     m, g = make_pair(orc, TINY[1], seed=31, realistic=True)
     outs = []
     for rep in range(3):
@@ -154,8 +154,11 @@ def test_graph_replay_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
     np.testing.assert_array_equal(outs[0], outs[1])
     np.testing.assert_array_equal(outs[0], outs[2])
     g.reset()
+    # the kernel-by-kernel path (used for taps) folds attention splits in another order: equal to rounding
     eager = np.stack([g.forward_taps(5 + p, p).copy() for p in range(6)])
-    np.testing.assert_array_equal(outs[0], eager)
+    eager2 = np.stack([g.forward_taps(5 + p, p).copy() for p in range(6)])
+    np.testing.assert_array_equal(eager, eager2)
+    assert rel_err(outs[0], eager) < 1e-5
     # fused argmax == first-max of the logits the same forward produced
     g.reset()
     for p in range(6):
