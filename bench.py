@@ -76,6 +76,8 @@ def main():
     ap.add_argument("--workload", default="llama2-7b-shape", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-steps", type=int, default=13, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on ONE GPU (batch-1 decode, no multi-GPU split); --gpus %d is not supported" % a.gpus,
@@ -131,6 +133,8 @@ def main():
         "frac_of_stream_roofline": round(tok_s * bytes_tok / (HBM_PEAK_GBS * 1e9), 4),
     }
 
+    if a.calibrate_copy > 0:
+        g.calibration_copy(a.calibrate_copy << 20, 3)
     if not a.no_kernels:
         pos = int(round(mean_pos))
         kern = {}
@@ -139,14 +143,15 @@ def main():
             kern[KERNEL.NAMES[k]] = {"us": round(us, 3), "bytes": b, "GBps": round(b / us * 1e-3, 1),
                                      "frac": round(b / us * 1e-3 / HBM_PEAK_GBS, 4)}
         out["kernels"] = kern
+        # dominant kernel: the W1/W3 matvec streams the largest share of every token's bytes
         dom = kern["w13"]
         traffic = None
-        tpath = os.path.join(ROOT, "profiles", "w13_traffic.json")
+        tpath = os.path.join(ROOT, "profiles", "k_matvec_w13_llama2-7b_traffic.json")
         if a.workload == "llama2-7b-shape" and os.path.exists(tpath):
             traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        out["roofline"] = {"bound": "hbm", "kernel": "k_matvec<MV_W13> (rmsnorm + W1,W3 matvec + SwiGLU)",
+        out["roofline"] = {"bound": "hbm", "kernel": "k_matvec<PH_W13> (rmsnorm + W1,W3 matvec + SwiGLU), one launch per layer",
                            "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
-                           "traffic": traffic}
+                           "algorithmic_bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"], "traffic": traffic}
     else:
         out["roofline"] = None
 

@@ -2,7 +2,8 @@
  * libllama2j_hip.so - C ABI of the MI355X (gfx950) mode of llama2j's per-token forward pass.
  *
  * The library owns every device buffer (weights, activations, KV cache), takes llama2j's own
- * weight formats, and replays the whole token as one captured hipGraph on one GPU.  It is the
+ * weight formats, and replays the whole token (a chain of hand-written gfx950 kernels) as one captured
+ * hipGraph on one GPU.  It is the
  * seam a `Mode.HIP` plugs into beside the reference's CPU and CUDA modes: each entry point
  * names the reference interface it replaces (paths relative to the reference root,
  * J/ = src/main/java/com/lastbot/llama2j/, K/ = J/kernel/).
@@ -132,6 +133,9 @@ int l2j_sync(l2j_ctx *ctx);
 enum l2j_kernel_class { L2J_K_QKV = 0, L2J_K_ATTENTION, L2J_K_WO, L2J_K_W13, L2J_K_W2, L2J_K_CLASSIFIER, L2J_K_COUNT };
 int l2j_time_kernel(l2j_ctx *ctx, int kernel_class, int32_t pos, int32_t rounds, double *mean_us,
                     uint64_t *algorithmic_bytes);
+/* Measurement: runs k_copy16 (reads nbytes, writes nbytes) `rounds` times; hardware byte counters of the
+ * other kernels are scaled by what the same counters report for this kernel of known size. */
+int l2j_calibration_copy(l2j_ctx *ctx, uint64_t nbytes, int32_t rounds);
 /* Algorithmic bytes one token streams at position pos: weights in the reference's storage format
  * (264 bytes per 256 weights, fp32 classifier and embedding row) plus KV cache read and write. */
 uint64_t l2j_bytes_per_token(const l2j_config *cfg, int32_t pos);

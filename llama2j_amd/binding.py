@@ -102,6 +102,7 @@ def _signatures():
         "l2j_write_kv": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, fp, fp]),
         "l2j_sync": (C.c_int, [vp]),
         "l2j_time_kernel": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
+        "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
         "l2j_bytes_per_token": (C.c_uint64, [cfgp, C.c_int32]),
         "l2j_quant_nbytes": (C.c_uint64, [C.c_uint64]),
         "l2j_quant_encode": (C.c_int, [fp, C.c_uint64, u8p]),
@@ -327,6 +328,9 @@ class Transformer:
         b = C.c_uint64(0)
         _check(lib().l2j_time_kernel(self._h, kernel_class, pos, rounds, C.byref(us), C.byref(b)))
         return us.value, b.value
+
+    def calibration_copy(self, nbytes, rounds=3):
+        _check(lib().l2j_calibration_copy(self._h, nbytes, rounds))
 
     def bytes_per_token(self, pos):
         return int(lib().l2j_bytes_per_token(C.byref(self.config), pos))

@@ -285,4 +285,10 @@ __global__ void __launch_bounds__(256) k_encode_groups(const float *__restrict__
     }
 }
 
+// Plain copy of n 16-byte words: the known-size kernel against which hardware byte counters are scaled.
+__global__ void __launch_bounds__(256) k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, long n)
+{
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 }  // namespace l2j

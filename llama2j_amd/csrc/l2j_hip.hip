@@ -277,7 +277,12 @@ hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
     return hipGetLastError();
 }
 
-hipError_t launch_one_token(l2j_ctx *c) { return hipGraphLaunch(c->graph_exec, c->stream); }
+// L2J_MODE=eager launches the kernels one by one instead of replaying the graph (for tools that do not
+// follow graph launches).
+hipError_t launch_one_token(l2j_ctx *c)
+{
+    return c->graph_exec ? hipGraphLaunch(c->graph_exec, c->stream) : launch_token(c, c->stream, false);
+}
 
 int check_barrier_error(l2j_ctx *) { return L2J_OK; }
 
@@ -675,6 +680,11 @@ int l2j_finalize(l2j_ctx *c)
 
     // capture one token
     HIPCHK(hipStreamSynchronize(c->stream));
+    const char *mode = getenv("L2J_MODE");
+    if (mode && strcmp(mode, "eager") == 0) {
+        c->finalized = true;
+        return L2J_OK;
+    }
     HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
     hipError_t le = launch_token(c, c->stream, false);
     hipError_t ce = hipStreamEndCapture(c->stream, &c->graph);
@@ -849,6 +859,26 @@ int l2j_write_kv(l2j_ctx *c, int layer, int32_t pos0, int32_t npos, const float 
     HIPCHK(hipStreamSynchronize(c->stream));
     HIPCHK(hipMemcpy(c->kcache + o, k, n * sizeof(float), hipMemcpyHostToDevice));
     HIPCHK(hipMemcpy(c->vcache + o, v, n * sizeof(float), hipMemcpyHostToDevice));
+    return L2J_OK;
+}
+
+int l2j_calibration_copy(l2j_ctx *c, uint64_t nbytes, int32_t rounds)
+{
+    if (!c || nbytes < 16 || rounds <= 0) return fail(L2J_E_ARG, "bad argument");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    uint4 *a = nullptr, *b = nullptr;
+    const long n = (long)(nbytes / 16);
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(&a), (size_t)n * 16));
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&b), (size_t)n * 16);
+    if (e == hipSuccess) e = hipMemsetAsync(a, 1, (size_t)n * 16, c->stream);
+    for (int r = 0; r < rounds && e == hipSuccess; r++) {
+        hipLaunchKernelGGL(k_copy16, dim3(c->n_cu * 8), dim3(256), 0, c->stream, a, b, n);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    (void)hipFree(a);
+    (void)hipFree(b);
+    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("calibration copy: ") + hipGetErrorString(e));
     return L2J_OK;
 }
 
