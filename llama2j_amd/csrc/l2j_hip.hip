@@ -228,6 +228,8 @@ hipError_t launch_class(const l2j_ctx *c, int kclass, int l, hipStream_t s, hipE
     case L2J_K_WO:
     case L2J_K_W2: {
         const int n = kclass == L2J_K_WO ? c->cfg.dim : c->cfg.hidden_dim;
+        if (n / 16 > 64 * kTU)  // long rows: one row per wave keeps every wave busy
+            return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
         return launch1(k_matvec<PH_RES>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
     }
     case L2J_K_ATTENTION: {
@@ -668,7 +670,7 @@ int l2j_finalize(l2j_ctx *c)
         if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
         if (need > 64 * 1024) {
             const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
-                                reinterpret_cast<const void *>(k_matvec<PH_RES>),
+                                reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
                                 reinterpret_cast<const void *>(k_classifier)};
             for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
         }

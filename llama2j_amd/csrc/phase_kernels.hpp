@@ -25,13 +25,13 @@ __device__ __forceinline__ int ld_coh(const int *p) { return __hip_atomic_load(p
 __device__ __forceinline__ void st_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coh(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2 };
+enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2, PH_ROW = 3 };  // PH_RES: row pairs + residual; PH_ROW: one row per wave + residual
 
 // One matvec phase.  Passed by value.
 struct MatvecPhase {
     int n;          // input vector length (multiple of 16)
     int from_emb;   // the input vector is the embedding row of the current token (QKV of layer 0)
-    int res_emb;    // PH_RES: the residual input is the embedding row of the current token (Wo of layer 0)
+    int res_emb;    // PH_RES / PH_ROW: the residual input is the embedding row of the current token (Wo of layer 0)
     int d0, d1, d2; // rows: QKV (dim, kv_dim, kv_dim); W13 (hidden); RES (dim)
     const float *xin;   // input vector (ignored when from_emb)
     const float *rmsw;  // dequantized rmsnorm weights (fp32) or null: input = rmsw[e] * (ss * x[e])
@@ -144,26 +144,34 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
             mb = d.m1;
             f0 = m.off + (long)r * n;
             f1 = mb.off + (long)r * n;
-        } else {  // rows (2p, 2p+1)
+        } else if (MODE == PH_RES) {  // rows (2p, 2p+1)
             r = 2 * item;
             has1 = r + 1 < d.d0;
             f0 = m.off + (long)r * n;
             f1 = has1 ? f0 + n : f0;
+        } else {  // PH_ROW, long rows: one row per wave so every wave has work; sub-row 1 is the same row, kTU*64 chunks on
+            r = item;
+            f0 = m.off + (long)r * n;
+            f1 = f0;
         }
         cb0 = m.codes + f0; gb0 = m.gs + (f0 >> 8); r0 = (unsigned)(f0 & 255);
         cb1 = mb.codes + f1; gb1 = mb.gs + (f1 >> 8); r1 = (unsigned)(f1 & 255);
     };
     uint4 w0[kTU], w1[kTU];
     float2 s0[kTU], s1[kTU];
+    // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
+    constexpr int kStep = MODE == PH_ROW ? 2 * 64 * kTU : 64 * kTU;
+    constexpr int kOff1 = MODE == PH_ROW ? 64 * kTU : 0;
     auto issue = [&](int base) {
 #pragma unroll
         for (int u = 0; u < kTU; u++) {
-            const int c = base + 64 * u + lane;
+            const int c = base + 64 * u + lane, c1 = c + kOff1;
             const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 below)
+            const unsigned cc1 = c1 < nch ? c1 : nch - 1;
             w0[u] = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
-            w1[u] = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc);
+            w1[u] = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc1);
             s0[u] = gb0[(r0 + 16u * cc) >> 8];
-            s1[u] = gb1[(r1 + 16u * cc) >> 8];
+            s1[u] = gb1[(r1 + 16u * cc1) >> 8];
         }
     };
 
@@ -182,12 +190,12 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
     for (; item < nitems; item += W * G) {
         if (!first) resolve(item);
         float resv0 = 0.0f, resv1 = 0.0f;
-        if (MODE == PH_RES && lane == 0) {  // in flight while the row streams
+        if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {  // in flight while the row streams
             resv0 = res[r];
-            if (has1) resv1 = res[r + 1];
+            if (MODE == PH_RES && has1) resv1 = res[r + 1];
         }
         float acc0 = 0.0f, acc1 = 0.0f;
-        for (int base = 0; base < nch; base += 64 * kTU) {
+        for (int base = 0; base < nch; base += kStep) {
             if (!(first && base == 0)) issue(base);
 #pragma unroll
             for (int u = 0; u < kTU; u++) {
@@ -198,9 +206,18 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
                 const float sx = sumx[cc];
                 // sum (code*rm + min)*x = rm * sum code*x + min * sum x over the chunk
                 const float t0 = fmaf(s0[u].x, dot16(w0[u], x0, x1, x2, x3), s0[u].y * sx);
-                const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
                 acc0 += ok ? t0 : 0.0f;
-                acc1 += ok ? t1 : 0.0f;
+                if (MODE == PH_ROW) {
+                    const int c1 = c + kOff1;
+                    const bool ok1 = c1 < nch;
+                    const int cc1 = ok1 ? c1 : nch - 1;
+                    const float4 y0 = xs[cc1], y1 = xs[nch + cc1], y2 = xs[2 * nch + cc1], y3 = xs[3 * nch + cc1];
+                    const float t1 = fmaf(s1[u].x, dot16(w1[u], y0, y1, y2, y3), s1[u].y * sumx[cc1]);
+                    acc1 += ok1 ? t1 : 0.0f;
+                } else {
+                    const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
+                    acc1 += ok ? t1 : 0.0f;
+                }
             }
         }
         first = false;
@@ -220,9 +237,11 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
             } else if (MODE == PH_W13) {
                 const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
                 d.out0[r] = __fmul_rn(acc0, __fmul_rn(s, acc1));
-            } else {
+            } else if (MODE == PH_RES) {
                 d.out0[r] = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
                 if (has1) d.out0[r + 1] = __fadd_rn(resv1, acc1);
+            } else {
+                d.out0[r] = __fadd_rn(resv0, acc0 + acc1);
             }
         }
     }
