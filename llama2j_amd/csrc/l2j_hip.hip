@@ -66,8 +66,11 @@ struct l2j_ctx {
     float *emb = nullptr, *wcls = nullptr;
     bool emb_loaded = false, wcls_loaded = false;
 
-    // activations
+    // Activations.  Every vector of a token has an address of its own (stride = length rounded up to 256
+    // bytes): x holds the 2L+1 versions of the residual stream (version 2l+1 after the attention residual of
+    // layer l, 2l+2 after its FFN residual), xb, hb and q one vector per layer.
     float *x = nullptr, *xb = nullptr, *hb = nullptr, *q = nullptr, *logits = nullptr;
+    uint64_t sd = 0, sh = 0;  // strides of dim-long and hidden_dim-long vectors, in floats
     float *kcache = nullptr, *vcache = nullptr;
     float2 *rope = nullptr;
     float *silu = nullptr;
@@ -87,6 +90,16 @@ struct l2j_ctx {
     int *cls_idx = nullptr;
     float *attn_part = nullptr;
     float *rmsw = nullptr;  // dequantized rmsnorm weights: att (L*dim), ffn (L*dim), final (dim)
+
+    // k_token: a range of layers (by default the whole token) per launch, grid barriers between the phases
+    bool fused = false;
+    int layers_per_launch = 0;
+    unsigned *bar_ctr = nullptr;  // kBarStride words per barrier instance, 5 instances per layer
+    int nbar = 0;
+    int *fault = nullptr;         // set by a kernel whose barrier wait ran out
+    int *h_fault = nullptr;       // pinned
+    int fused_attn_rows = 64;
+    TokenGeom geom{};             // set by l2j_finalize
 
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
@@ -149,62 +162,71 @@ size_t mv_smem(int n) { return (size_t)n * 4 + (size_t)(n / 16) * 4 + 64 * sizeo
 
 int attn_lpr(const l2j_ctx *c) { return c->head_size <= 64 ? 16 : c->head_size <= 128 ? 32 : 64; }
 
-size_t attn_smem(const l2j_ctx *c)
+size_t attn_smem_for(const l2j_ctx *c, int threads)
 {
-    const int nent = (c->attn_threads / 64) * (64 / attn_lpr(c));
-    return (size_t)(2 * nent + nent * c->head_size) * sizeof(float);
+    const int nent = (threads / 64) * (64 / attn_lpr(c));
+    return (size_t)(2 * nent + nent * c->head_size + 1) * sizeof(float);
 }
 
-// Arguments of the phases of layer l (J/Run.java:76-159).
-MatvecPhase matvec_phase(const l2j_ctx *c, int kclass, int l)
+size_t attn_smem(const l2j_ctx *c) { return attn_smem_for(c, c->attn_threads); }
+
+size_t layer_smem(const l2j_ctx *c)
+{
+    return std::max(mv_smem(std::max(c->cfg.dim, c->cfg.hidden_dim)), attn_smem_for(c, c->pk_threads));
+}
+
+static_assert(K_QKV == L2J_K_QKV && K_ATT == L2J_K_ATTENTION && K_WO == L2J_K_WO && K_W13 == L2J_K_W13 && K_W2 == L2J_K_W2 &&
+              K_CLS == L2J_K_CLASSIFIER, "kernel classes of the C ABI and of the device code must agree");
+
+MatvecPhase matvec_phase(const l2j_ctx *c, int kclass, int l) { return matvec_phase_of(c->geom, kclass, l); }
+AttnPhase attn_phase(const l2j_ctx *c, int l) { return attn_phase_of(c->geom, l, c->attn_rows); }
+ClsPhase cls_phase(const l2j_ctx *c) { return cls_phase_of(c->geom, c->pk_grid); }
+
+void build_geom(l2j_ctx *c)
 {
     const l2j_config &g = c->cfg;
-    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim, L = g.n_layers;
-    const uint64_t kvoff = (uint64_t)l * g.seq_len * kvd;
-    MatvecPhase d{};
-    d.emb = c->emb; d.rope = c->rope; d.silu = c->silu; d.st = c->st;
-    d.head_size = c->head_size; d.kv_dim = c->kv_dim; d.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0;
-    switch (kclass) {
-    case L2J_K_QKV:
-        d.n = g.dim; d.from_emb = l == 0; d.xin = c->x; d.rmsw = c->rmsw + (uint64_t)l * dim;
-        d.d0 = g.dim; d.d1 = d.d2 = c->kv_dim;
-        d.m0 = qmat(c, L2J_WQ, l * dim * dim); d.m1 = qmat(c, L2J_WK, l * dim * kvd); d.m2 = qmat(c, L2J_WV, l * dim * kvd);
-        d.out0 = c->q; d.out1 = c->kcache + kvoff; d.out2 = c->vcache + kvoff;
-        break;
-    case L2J_K_WO:
-        d.n = g.dim; d.xin = c->xb; d.d0 = g.dim; d.m0 = qmat(c, L2J_WO, l * dim * dim);
-        d.out0 = c->x; d.res_src = c->x; d.res_emb = l == 0;
-        break;
-    case L2J_K_W13:
-        d.n = g.dim; d.xin = c->x; d.rmsw = c->rmsw + (L + l) * dim; d.d0 = g.hidden_dim;
-        d.m0 = qmat(c, L2J_W1, l * dim * hid); d.m1 = qmat(c, L2J_W3, l * dim * hid); d.out0 = c->hb;
-        break;
-    default:  // L2J_K_W2
-        d.n = g.hidden_dim; d.xin = c->hb; d.d0 = g.dim; d.m0 = qmat(c, L2J_W2, l * dim * hid);
-        d.out0 = c->x; d.res_src = c->x;
-        break;
-    }
-    return d;
+    TokenGeom &t = c->geom;
+    t.dim = g.dim; t.hidden = g.hidden_dim; t.n_layers = g.n_layers; t.n_heads = g.n_heads; t.kv_mul = c->kv_mul;
+    t.head_size = c->head_size; t.kv_dim = c->kv_dim; t.seq_len = g.seq_len; t.vocab = g.vocab_size;
+    t.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0;
+    t.sd = (long)c->sd; t.sh = (long)c->sh;
+    t.emb = c->emb; t.rmsw = c->rmsw; t.silu = c->silu; t.wcls = c->wcls; t.rope = c->rope;
+    t.x = c->x; t.xb = c->xb; t.hb = c->hb; t.q = c->q; t.kcache = c->kcache; t.vcache = c->vcache; t.logits = c->logits;
+    t.wq = qmat(c, L2J_WQ, 0); t.wk = qmat(c, L2J_WK, 0); t.wv = qmat(c, L2J_WV, 0); t.wo = qmat(c, L2J_WO, 0);
+    t.w1 = qmat(c, L2J_W1, 0); t.w2 = qmat(c, L2J_W2, 0); t.w3 = qmat(c, L2J_W3, 0);
+    t.attn_part = c->attn_part; t.attn_counters = c->counters; t.attn_nsplit = c->attn_nsplit;
+    t.sqrt_hs = sqrtf((float)c->head_size);
+    t.st = c->st; t.cls_val = c->cls_val; t.cls_idx = c->cls_idx; t.prompt = c->prompt; t.out_tokens = c->out_tokens;
+    t.bar_ctr = c->bar_ctr; t.nbar = c->nbar; t.fault = c->fault;
 }
 
-AttnPhase attn_phase(const l2j_ctx *c, int l)
+// Every buffer a kernel may touch exists (checked on the host before anything is launched).
+bool geom_complete(const TokenGeom &t)
 {
-    const uint64_t kvoff = (uint64_t)l * c->cfg.seq_len * c->kv_dim;
-    AttnPhase t{};
-    t.q = c->q; t.kc = c->kcache + kvoff; t.vc = c->vcache + kvoff; t.out = c->xb; t.part = c->attn_part;
-    t.counters = c->counters; t.st = c->st; t.n_heads = c->cfg.n_heads; t.kv_mul = c->kv_mul; t.head_size = c->head_size;
-    t.kv_dim = c->kv_dim; t.nsplit = c->attn_nsplit; t.rows_per_split = c->attn_rows;
-    t.sqrt_hs = sqrtf((float)c->head_size);  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
-    return t;
+    const void *ptrs[] = {t.emb, t.rmsw, t.silu, t.wcls, t.rope, t.x, t.xb, t.hb, t.q, t.kcache, t.vcache, t.logits,
+                          t.wq.codes, t.wq.gs, t.wk.codes, t.wk.gs, t.wv.codes, t.wv.gs, t.wo.codes, t.wo.gs,
+                          t.w1.codes, t.w1.gs, t.w2.codes, t.w2.gs, t.w3.codes, t.w3.gs,
+                          t.attn_part, t.attn_counters, t.st, t.cls_val, t.cls_idx, t.prompt, t.out_tokens, t.bar_ctr, t.fault};
+    for (const void *p : ptrs)
+        if (!p) return false;
+    return true;
 }
 
-ClsPhase cls_phase(const l2j_ctx *c)
+// Layers [l0, l1) (and the classifier after the last layer) in one launch of k_token.
+hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s)
 {
-    ClsPhase a{};
-    a.xin = c->x; a.rmsw = c->rmsw + 2ull * c->cfg.n_layers * c->cfg.dim; a.w = c->wcls; a.n = c->cfg.dim; a.vocab = c->cfg.vocab_size;
-    a.logits = c->logits; a.part_val = c->cls_val; a.part_idx = c->cls_idx; a.nparts = c->pk_grid;
-    a.st = c->st; a.prompt = c->prompt; a.out_tokens = c->out_tokens;
-    return a;
+    TokenArgs a{};
+    a.g = c->geom;
+    a.l0 = l0; a.l1 = l1; a.with_cls = l1 == c->cfg.n_layers;
+    a.attn_rows = c->fused_attn_rows;
+    a.maxspin = 20000;
+    const dim3 grid(c->pk_grid), block(c->pk_threads);
+    const size_t smem = layer_smem(c);
+    const int lpr = attn_lpr(c);
+    if (lpr == 16) hipLaunchKernelGGL(k_token<16>, grid, block, smem, s, a);
+    else if (lpr == 32) hipLaunchKernelGGL(k_token<32>, grid, block, smem, s, a);
+    else hipLaunchKernelGGL(k_token<64>, grid, block, smem, s, a);
+    return hipGetLastError();
 }
 
 template <typename K, typename A>
@@ -228,7 +250,7 @@ hipError_t launch_class(const l2j_ctx *c, int kclass, int l, hipStream_t s, hipE
     case L2J_K_WO:
     case L2J_K_W2: {
         const int n = kclass == L2J_K_WO ? c->cfg.dim : c->cfg.hidden_dim;
-        if (n / 16 > 64 * kTU)  // long rows: one row per wave keeps every wave busy
+        if (row_mode(n))  // long rows: one row per wave keeps every wave busy
             return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
         return launch1(k_matvec<PH_RES>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
     }
@@ -256,23 +278,29 @@ hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
 {
     const l2j_config &g = c->cfg;
     hipError_t e;
+    if (c->fused && !taps) {
+        for (int l = 0; l < g.n_layers; l += c->layers_per_launch)
+            if ((e = launch_layers(c, l, std::min(g.n_layers, l + c->layers_per_launch), s)) != hipSuccess) return e;
+        hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, s, cls_phase(c));
+        return hipGetLastError();
+    }
     for (int l = 0; l < g.n_layers; l++) {
         const uint64_t kvoff = (uint64_t)l * g.seq_len * c->kv_dim;
         if ((e = launch_class(c, L2J_K_QKV, l, s)) != hipSuccess) return e;
         if (taps) {  // rows of the caches at the current position; pos is known on the host in this mode
             const uint64_t row = (uint64_t)c->h_st->pos * c->kv_dim;
-            if ((e = tap_copy(c, L2J_B_Q, l, c->q, g.dim, s)) != hipSuccess) return e;
+            if ((e = tap_copy(c, L2J_B_Q, l, c->q + l * c->sd, g.dim, s)) != hipSuccess) return e;
             if ((e = tap_copy(c, L2J_B_K, l, c->kcache + kvoff + row, c->kv_dim, s)) != hipSuccess) return e;
             if ((e = tap_copy(c, L2J_B_V, l, c->vcache + kvoff + row, c->kv_dim, s)) != hipSuccess) return e;
         }
         if ((e = launch_class(c, L2J_K_ATTENTION, l, s)) != hipSuccess) return e;
-        if (taps && (e = tap_copy(c, L2J_B_XB, l, c->xb, g.dim, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_XB, l, c->xb + l * c->sd, g.dim, s)) != hipSuccess) return e;
         if ((e = launch_class(c, L2J_K_WO, l, s)) != hipSuccess) return e;
-        if (taps && (e = tap_copy(c, L2J_B_XB2, l, c->x, g.dim, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_XB2, l, c->x + (2 * l + 1) * c->sd, g.dim, s)) != hipSuccess) return e;
         if ((e = launch_class(c, L2J_K_W13, l, s)) != hipSuccess) return e;
-        if (taps && (e = tap_copy(c, L2J_B_HB, l, c->hb, g.hidden_dim, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_HB, l, c->hb + l * c->sh, g.hidden_dim, s)) != hipSuccess) return e;
         if ((e = launch_class(c, L2J_K_W2, l, s)) != hipSuccess) return e;
-        if (taps && (e = tap_copy(c, L2J_B_X, l, c->x, g.dim, s)) != hipSuccess) return e;
+        if (taps && (e = tap_copy(c, L2J_B_X, l, c->x + (2 * l + 2) * c->sd, g.dim, s)) != hipSuccess) return e;
     }
     if ((e = launch_class(c, L2J_K_CLASSIFIER, 0, s)) != hipSuccess) return e;
     hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, s, cls_phase(c));
@@ -286,7 +314,16 @@ hipError_t launch_one_token(l2j_ctx *c)
     return c->graph_exec ? hipGraphLaunch(c->graph_exec, c->stream) : launch_token(c, c->stream, false);
 }
 
-int check_barrier_error(l2j_ctx *) { return L2J_OK; }
+// After a synchronize: a workgroup whose bounded wait at a grid barrier ran out has set the flag.
+int check_barrier_error(l2j_ctx *c)
+{
+    if (!c->fused) return L2J_OK;
+    HIPCHK(hipMemcpy(c->h_fault, c->fault, sizeof(int), hipMemcpyDeviceToHost));
+    if (*c->h_fault == 0) return L2J_OK;
+    *c->h_fault = 0;
+    HIPCHK(hipMemcpy(c->fault, c->h_fault, sizeof(int), hipMemcpyHostToDevice));
+    return fail(L2J_E_HIP, "a grid barrier of the layer kernel timed out (its workgroups were not all resident)");
+}
 
 int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
 {
@@ -413,10 +450,13 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     if (cfg->shared_weights) c->wcls = c->emb;
     else TRY(dev_alloc(&c->wcls, vd));
     const uint64_t kvn = (uint64_t)cfg->n_layers * cfg->seq_len * c->kv_dim;
-    TRY(dev_alloc(&c->x, cfg->dim));
-    TRY(dev_alloc(&c->xb, cfg->dim));
-    TRY(dev_alloc(&c->hb, cfg->hidden_dim));
-    TRY(dev_alloc(&c->q, cfg->dim));
+    const uint64_t NL = cfg->n_layers;
+    c->sd = ((uint64_t)cfg->dim + 63) / 64 * 64;
+    c->sh = ((uint64_t)cfg->hidden_dim + 63) / 64 * 64;
+    TRY(dev_alloc(&c->x, (2 * NL + 1) * c->sd));
+    TRY(dev_alloc(&c->xb, NL * c->sd));
+    TRY(dev_alloc(&c->hb, NL * c->sh));
+    TRY(dev_alloc(&c->q, NL * c->sd));
     TRY(dev_alloc(&c->logits, cfg->vocab_size));
     TRY(dev_alloc(&c->kcache, kvn));
     TRY(dev_alloc(&c->vcache, kvn));
@@ -465,6 +505,9 @@ void l2j_destroy(l2j_ctx *c)
     (void)hipFree(c->st);
     (void)hipFree(c->prompt);
     (void)hipFree(c->out_tokens);
+    (void)hipFree(c->bar_ctr);
+    (void)hipFree(c->fault);
+    if (c->h_fault) (void)hipHostFree(c->h_fault);
     for (float *t : c->taps) (void)hipFree(t);
     if (c->h_st) (void)hipHostFree(c->h_st);
     if (c->h_tokens) (void)hipHostFree(c->h_tokens);
@@ -666,18 +709,40 @@ int l2j_finalize(l2j_ctx *c)
         c->attn_rows = std::max(1, env_int("L2J_ATTN_ROWS", 32));
         c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
         c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
-        const size_t need = std::max(mv_smem(nmax), attn_smem(c));
+        c->fused_attn_rows = std::max(1, env_int("L2J_FUSED_ATTN_ROWS", 64));
+        const size_t need = std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c));
         if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
         if (need > 64 * 1024) {
             const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
                                 reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
-                                reinterpret_cast<const void *>(k_classifier)};
+                                reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
+                                reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>)};
             for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
         }
         int rc2;
         if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
         if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
         if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
+        c->nbar = 5 * c->cfg.n_layers;
+        if ((rc2 = dev_alloc(&c->bar_ctr, (uint64_t)c->nbar * kBarStride))) return rc2;
+        if ((rc2 = dev_alloc(&c->fault, 1))) return rc2;
+        HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));
+        HIPCHK(hipMemset(c->fault, 0, sizeof(int)));
+        HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&c->h_fault), sizeof(int), hipHostMallocDefault));
+        *c->h_fault = 0;
+        // k_token needs its whole grid resident at once (grid barriers): at most what the occupancy allows.
+        c->fused = env_int("L2J_FUSE", 1) != 0;
+        c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, env_int("L2J_LAYERS_PER_LAUNCH", c->cfg.n_layers)));
+        if (c->fused) {
+            const int lpr = attn_lpr(c);
+            const void *kl = lpr == 16 ? reinterpret_cast<const void *>(k_token<16>)
+                           : lpr == 32 ? reinterpret_cast<const void *>(k_token<32>) : reinterpret_cast<const void *>(k_token<64>);
+            int per_cu = 0;
+            HIPCHK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kl, c->pk_threads, layer_smem(c)));
+            if (per_cu < 1 || c->pk_grid > per_cu * c->n_cu) c->fused = false;
+        }
+        build_geom(c);
+        if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
     }
 
     // capture one token
@@ -833,10 +898,10 @@ int l2j_read(l2j_ctx *c, int which, int layer, uint64_t off, float *dst, uint64_
         src = c->logits; len = g.vocab_size;
     } else if (layer < 0) {
         switch (which) {
-        case L2J_B_X: src = c->x; len = g.dim; break;
-        case L2J_B_XB: src = c->xb; len = g.dim; break;
-        case L2J_B_HB: src = c->hb; len = g.hidden_dim; break;
-        case L2J_B_Q: src = c->q; len = g.dim; break;
+        case L2J_B_X: src = c->x + 2ull * g.n_layers * c->sd; len = g.dim; break;  // the last layer's vectors
+        case L2J_B_XB: src = c->xb + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
+        case L2J_B_HB: src = c->hb + (uint64_t)(g.n_layers - 1) * c->sh; len = g.hidden_dim; break;
+        case L2J_B_Q: src = c->q + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
         default: return fail(L2J_E_ARG, "this buffer only exists as a per-layer tap");
         }
     } else {

@@ -1,18 +1,27 @@
-// The per-token forward pass (J/Run.java:62-169) as a chain of gfx950 kernels, one per phase:
-//   per layer   k_matvec<PH_QKV>   rmsnorm + Wq,Wk,Wv matvec + RoPE + KV-cache store
-//               k_attention        decode attention, split over the sequence, online softmax
-//               k_matvec<PH_RES>   Wo matvec + residual
-//               k_matvec<PH_W13>   rmsnorm + W1,W3 matvec + SwiGLU (the reference's sigmoid table)
-//               k_matvec<PH_RES>   W2 matvec + residual
-//   once        k_classifier       final rmsnorm + fp32 classifier + per-workgroup first-max
-//               k_finish           fold the maxima, step the token loop state
-// captured once in a hipGraph and replayed per token.
+// The per-token forward pass (J/Run.java:62-169) on gfx950.  Per layer there are five phases:
+//   PH_QKV      rmsnorm + Wq,Wk,Wv matvec + RoPE + KV-cache store
+//   attention   decode attention, split over the sequence, online softmax
+//   PH_RES/ROW  Wo matvec + residual
+//   PH_W13      rmsnorm + W1,W3 matvec + SwiGLU (the reference's sigmoid table)
+//   PH_RES/ROW  W2 matvec + residual
+// and once per token k_classifier (final rmsnorm + fp32 classifier + per-workgroup first-max) and k_finish
+// (fold the maxima, step the token loop state).  k_token runs all phases of a range of layers (by default
+// the whole token, classifier included) in one launch, one 1024-thread workgroup per compute unit, with grid
+// barriers between the phases; each phase also exists as a kernel of its own (k_matvec<MODE>, k_attention,
+// k_classifier) for per-layer taps and per-phase timing.  The launches of a token are captured once in a
+// hipGraph and replayed.
 //
-// Every kernel is HBM-bandwidth bound (batch-1 GEMV: no reuse, so no MFMA): int8 codes are streamed
+// Every phase is HBM-bandwidth bound (batch-1 GEMV: no reuse, so no MFMA): int8 codes are streamed
 // with 16-byte nontemporal loads, one wavefront per pair of sub-rows, the activation vector is staged
-// in LDS once per workgroup (one 1024-thread workgroup per compute unit), accumulation is fp32 and the
-// 64-lane reduction uses DPP.  All arguments are passed by value so that every pointer is a kernel
-// argument (global address space, scalar base + 32-bit lane offset addressing).
+// in LDS once per workgroup, accumulation is fp32 and the 64-lane reduction uses DPP.  All arguments are
+// passed by value so that every pointer is a kernel argument (global address space, scalar base + 32-bit
+// lane offset addressing).
+//
+// Activations cross a grid barrier without cache maintenance: producers store them with device-scope
+// relaxed atomics (write-through), every activation vector of a token has a cache-line-aligned address of
+// its own that nothing reads before its producer has finished, and so consumers use plain loads.  The first
+// weights of the next phase are requested between arriving at a barrier and waiting on it, so HBM stays
+// busy while the slowest workgroups finish the phase.
 #pragma once
 
 #include "kernels.hpp"
@@ -24,6 +33,60 @@ __device__ __forceinline__ void st_coh(float *p, float v) { __hip_atomic_store(p
 __device__ __forceinline__ int ld_coh(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coh(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// ---- grid barrier ------------------------------------------------------------------------------------
+// Two levels of relaxed device-scope counters: a workgroup bumps the counter of its group (blockIdx % ngroups),
+// the last of a group bumps the top counter, everybody polls the top counter.  Every barrier instance of a
+// token has counters of its own (zeroed by k_finish), each on its own 256-byte line.  All workgroups of the
+// grid must be resident (one per compute unit).  The wait is bounded: when it runs out *fault is set, the
+// remaining barriers fall through and the host reports the token as failed.
+struct GridBar {
+    unsigned *ctr;   // instance i: top counter at ctr[i * kBarStride], group g at ctr[i * kBarStride + 64 * (1 + g)]
+    int *fault;
+    int ngroups, maxspin;
+};
+constexpr int kBarGroups = 8;
+constexpr int kBarStride = 64 * (1 + kBarGroups);  // unsigned words per barrier instance
+
+// Called when every store of the workgroup that the other workgroups will read has been acknowledged
+// (s_waitcnt vmcnt(0) in the storing waves, then a workgroup barrier if thread 0 is not the only one).
+__device__ __forceinline__ void bar_arrive(const GridBar &b, int inst)
+{
+    if (threadIdx.x == 0) {
+        unsigned *base = b.ctr + (long)inst * kBarStride;
+        const unsigned g = blockIdx.x % (unsigned)b.ngroups;
+        const unsigned gsize = (gridDim.x - g + b.ngroups - 1) / b.ngroups;
+        const unsigned old = __hip_atomic_fetch_add(base + 64 * (1 + g), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old + 1u == gsize) __hip_atomic_fetch_add(base, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+__device__ __forceinline__ void bar_wait(const GridBar &b, int inst)
+{
+    if (threadIdx.x == 0) {
+        const unsigned *top = b.ctr + (long)inst * kBarStride;
+        const unsigned want = min((unsigned)b.ngroups, gridDim.x);
+        int spins = 0;
+        while (__hip_atomic_load(top, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins > b.maxspin || ((spins & 255) == 0 && ld_coh(b.fault) != 0)) {
+                st_coh(b.fault, 1);
+                break;
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// The thread index as the phases see it.  It goes through an empty asm so that, inside k_token's layer loop,
+// the compiler cannot hoist every phase's lane-dependent addresses and predicates out of the loop and keep
+// them all live in vector registers (which spills).
+__device__ __forceinline__ int phase_tid()
+{
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
 
 enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2, PH_ROW = 3 };  // PH_RES: row pairs + residual; PH_ROW: one row per wave + residual
 
@@ -53,7 +116,7 @@ struct MatvecPhase {
 __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
                                              float *sumx, float *red)
 {
-    const int nch = n >> 4, tid = threadIdx.x, T = blockDim.x;
+    const int nch = n >> 4, tid = phase_tid(), T = blockDim.x;
     if (rmsw) {
         float ssq = 0.0f;
         for (int c = tid; c < nch; c += T) {
@@ -105,64 +168,73 @@ __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int 
 
 constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
 
+// One matvec phase of one workgroup: preload() requests the first item's weights (they do not depend on
+// the input vector), run() stages the vector and streams the items.
 template <int MODE>
-__global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
-{
-    extern __shared__ float4 smem4[];
-    const int n = d.n, nch = n >> 4;
-    float4 *xs = smem4;
-    float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
-    float *red = sumx + nch;  // 16 floats
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int W = blockDim.x >> 6, G = gridDim.x;
-    const int token = d.st->token, pos = d.st->pos;
-    const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
+struct MatvecRun {
+    // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
+    static constexpr int kStep = MODE == PH_ROW ? 2 * 64 * kTU : 64 * kTU;
+    static constexpr int kOff1 = MODE == PH_ROW ? 64 * kTU : 0;
 
-    const int nitems = MODE == PH_QKV ? (d.d0 + d.d1 + d.d2) >> 1 : MODE == PH_RES ? (d.d0 + 1) >> 1 : d.d0;
-    const float *res = d.res_emb ? emb_row : d.res_src;
-
+    const MatvecPhase d;
+    int n, nch, lane, W, G, nitems, item;
     // The codes of an item: two sub-rows, each a scalar base pointer + the lane's 16-byte chunk index.
     const uint8_t *cb0 = nullptr, *cb1 = nullptr;  // first code of each sub-row (uniform)
     const float2 *gb0 = nullptr, *gb1 = nullptr;   // scale entry of the group holding that code
     unsigned r0 = 0, r1 = 0;                       // position of that code inside its group
     int which = 0, r = 0;
-    bool has1 = true;
-    auto resolve = [&](int item) {
+    bool has1 = true, first = false;
+    uint4 w0[kTU], w1[kTU];
+    float2 s0[kTU], s1[kTU];
+
+    __device__ __forceinline__ MatvecRun(const MatvecPhase &d_) : d(d_)
+    {
+        const int tid = phase_tid();
+        n = d.n;
+        nch = n >> 4;
+        lane = tid & 63;
+        W = blockDim.x >> 6;
+        G = gridDim.x;
+        nitems = MODE == PH_QKV ? (d.d0 + d.d1 + d.d2) >> 1 : MODE == PH_RES ? (d.d0 + 1) >> 1 : d.d0;
+        // Items are dealt block-minor (item -> workgroup item % G), so every compute unit gets the same
+        // number of rows even when the rows do not fill all waves.
+        item = __builtin_amdgcn_readfirstlane(tid >> 6) * G + blockIdx.x;
+    }
+
+    __device__ __forceinline__ void resolve(int it)
+    {
         long f0, f1;
         QMat m = d.m0, mb = d.m0;
         which = 0;
         has1 = true;
         if (MODE == PH_QKV) {  // rows (2p, 2p+1) of q, k or v: RoPE rotates the pair
-            r = 2 * item;
+            r = 2 * it;
             if (r >= d.d0 + d.d1) { which = 2; r -= d.d0 + d.d1; m = d.m2; }
             else if (r >= d.d0) { which = 1; r -= d.d0; m = d.m1; }
             mb = m;
             f0 = m.off + (long)r * n;
             f1 = f0 + n;
         } else if (MODE == PH_W13) {  // row p of w1 and row p of w3: SwiGLU needs both
-            r = item;
+            r = it;
             mb = d.m1;
             f0 = m.off + (long)r * n;
             f1 = mb.off + (long)r * n;
         } else if (MODE == PH_RES) {  // rows (2p, 2p+1)
-            r = 2 * item;
+            r = 2 * it;
             has1 = r + 1 < d.d0;
             f0 = m.off + (long)r * n;
             f1 = has1 ? f0 + n : f0;
-        } else {  // PH_ROW, long rows: one row per wave so every wave has work; sub-row 1 is the same row, kTU*64 chunks on
-            r = item;
+        } else {  // PH_ROW, long rows: one row per wave so every wave has work
+            r = it;
             f0 = m.off + (long)r * n;
             f1 = f0;
         }
         cb0 = m.codes + f0; gb0 = m.gs + (f0 >> 8); r0 = (unsigned)(f0 & 255);
         cb1 = mb.codes + f1; gb1 = mb.gs + (f1 >> 8); r1 = (unsigned)(f1 & 255);
-    };
-    uint4 w0[kTU], w1[kTU];
-    float2 s0[kTU], s1[kTU];
-    // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
-    constexpr int kStep = MODE == PH_ROW ? 2 * 64 * kTU : 64 * kTU;
-    constexpr int kOff1 = MODE == PH_ROW ? 64 * kTU : 0;
-    auto issue = [&](int base) {
+    }
+
+    __device__ __forceinline__ void issue(int base)
+    {
 #pragma unroll
         for (int u = 0; u < kTU; u++) {
             const int c = base + 64 * u + lane, c1 = c + kOff1;
@@ -173,78 +245,125 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
             s0[u] = gb0[(r0 + 16u * cc) >> 8];
             s1[u] = gb1[(r1 + 16u * cc1) >> 8];
         }
-    };
-
-    // Items are dealt block-minor (item -> workgroup item % G), so every compute unit gets the same
-    // number of rows even when the rows do not fill all waves.
-    int item = wave * G + blockIdx.x;
-    // The weights do not depend on the input vector: the first loads go out before it is staged, so
-    // HBM latency overlaps the rmsnorm prologue.
-    bool first = item < nitems;
-    if (first) {
-        resolve(item);
-        issue(0);
     }
-    stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red);
 
-    for (; item < nitems; item += W * G) {
-        if (!first) resolve(item);
-        float resv0 = 0.0f, resv1 = 0.0f;
-        if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {  // in flight while the row streams
-            resv0 = res[r];
-            if (MODE == PH_RES && has1) resv1 = res[r + 1];
-        }
-        float acc0 = 0.0f, acc1 = 0.0f;
-        for (int base = 0; base < nch; base += kStep) {
-            if (!(first && base == 0)) issue(base);
+    __device__ __forceinline__ void preload()
+    {
+        first = item < nitems;
+        if (first) {
+            resolve(item);
+            issue(0);
+        } else {  // defined on every path: otherwise the registers stay reserved for the whole layer loop of k_token
 #pragma unroll
             for (int u = 0; u < kTU; u++) {
-                const int c = base + 64 * u + lane;
-                const bool ok = c < nch;
-                const int cc = ok ? c : nch - 1;
-                const float4 x0 = xs[cc], x1 = xs[nch + cc], x2 = xs[2 * nch + cc], x3 = xs[3 * nch + cc];
-                const float sx = sumx[cc];
-                // sum (code*rm + min)*x = rm * sum code*x + min * sum x over the chunk
-                const float t0 = fmaf(s0[u].x, dot16(w0[u], x0, x1, x2, x3), s0[u].y * sx);
-                acc0 += ok ? t0 : 0.0f;
-                if (MODE == PH_ROW) {
-                    const int c1 = c + kOff1;
-                    const bool ok1 = c1 < nch;
-                    const int cc1 = ok1 ? c1 : nch - 1;
-                    const float4 y0 = xs[cc1], y1 = xs[nch + cc1], y2 = xs[2 * nch + cc1], y3 = xs[3 * nch + cc1];
-                    const float t1 = fmaf(s1[u].x, dot16(w1[u], y0, y1, y2, y3), s1[u].y * sumx[cc1]);
-                    acc1 += ok1 ? t1 : 0.0f;
-                } else {
-                    const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
-                    acc1 += ok ? t1 : 0.0f;
-                }
-            }
-        }
-        first = false;
-        acc0 = wave_sum(acc0);
-        acc1 = wave_sum(acc1);
-        if (lane == 0) {
-            if (MODE == PH_QKV) {
-                float v0 = acc0, v1 = acc1;
-                if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
-                    const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
-                    v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
-                    v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
-                }
-                float *dst = which == 0 ? d.out0 + r : (which == 1 ? d.out1 : d.out2) + (long)pos * d.kv_dim + r;
-                dst[0] = v0;
-                dst[1] = v1;
-            } else if (MODE == PH_W13) {
-                const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
-                d.out0[r] = __fmul_rn(acc0, __fmul_rn(s, acc1));
-            } else if (MODE == PH_RES) {
-                d.out0[r] = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
-                if (has1) d.out0[r + 1] = __fadd_rn(resv1, acc1);
-            } else {
-                d.out0[r] = __fadd_rn(resv0, acc0 + acc1);
+                w0[u] = w1[u] = make_uint4(0u, 0u, 0u, 0u);
+                s0[u] = s1[u] = make_float2(0.f, 0.f);
             }
         }
     }
+
+    // Destination of the results of an item (second pointer null when the item has one result).
+    __device__ __forceinline__ void dst_of(int it, int pos, float *&p0, float *&p1) const
+    {
+        if (MODE == PH_QKV) {
+            int rr = 2 * it;
+            float *base = d.out0;
+            if (rr >= d.d0 + d.d1) { rr -= d.d0 + d.d1; base = d.out2 + (long)pos * d.kv_dim; }
+            else if (rr >= d.d0) { rr -= d.d0; base = d.out1 + (long)pos * d.kv_dim; }
+            p0 = base + rr;
+            p1 = p0 + 1;
+        } else if (MODE == PH_RES) {
+            p0 = d.out0 + 2 * it;
+            p1 = 2 * it + 1 < d.d0 ? p0 + 1 : nullptr;
+        } else {
+            p0 = d.out0 + it;
+            p1 = nullptr;
+        }
+    }
+
+    // smem: 4*nch float4 (vector), nch floats (chunk sums), 16 floats (reduction)
+    __device__ __forceinline__ void run(float4 *smem4, int token, int pos)
+    {
+        float4 *xs = smem4;
+        float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
+        float *red = sumx + nch;
+        const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
+        const float *res = d.res_emb ? emb_row : d.res_src;
+        stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red);
+
+        for (; item < nitems; item += W * G) {
+            if (!first) resolve(item);
+            float resv0 = 0.0f, resv1 = 0.0f;
+            if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {  // in flight while the row streams
+                resv0 = res[r];
+                if (MODE == PH_RES && has1) resv1 = res[r + 1];
+            }
+            float acc0 = 0.0f, acc1 = 0.0f;
+            for (int base = 0; base < nch; base += kStep) {
+                if (!(first && base == 0)) issue(base);
+#pragma unroll
+                for (int u = 0; u < kTU; u++) {
+                    const int c = base + 64 * u + lane;
+                    const bool ok = c < nch;
+                    const int cc = ok ? c : nch - 1;
+                    const float4 x0 = xs[cc], x1 = xs[nch + cc], x2 = xs[2 * nch + cc], x3 = xs[3 * nch + cc];
+                    const float sx = sumx[cc];
+                    // sum (code*rm + min)*x = rm * sum code*x + min * sum x over the chunk
+                    const float t0 = fmaf(s0[u].x, dot16(w0[u], x0, x1, x2, x3), s0[u].y * sx);
+                    acc0 += ok ? t0 : 0.0f;
+                    if (MODE == PH_ROW) {
+                        const int c1 = c + kOff1;
+                        const bool ok1 = c1 < nch;
+                        const int cc1 = ok1 ? c1 : nch - 1;
+                        const float4 y0 = xs[cc1], y1 = xs[nch + cc1], y2 = xs[2 * nch + cc1], y3 = xs[3 * nch + cc1];
+                        const float t1 = fmaf(s1[u].x, dot16(w1[u], y0, y1, y2, y3), s1[u].y * sumx[cc1]);
+                        acc1 += ok1 ? t1 : 0.0f;
+                    } else {
+                        const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
+                        acc1 += ok ? t1 : 0.0f;
+                    }
+                }
+            }
+            first = false;
+            acc0 = wave_sum(acc0);
+            acc1 = wave_sum(acc1);
+            if (lane == 0) {
+                float v0, v1 = 0.0f;
+                if (MODE == PH_QKV) {
+                    v0 = acc0;
+                    v1 = acc1;
+                    if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
+                        const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
+                        v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
+                        v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
+                    }
+                } else if (MODE == PH_W13) {
+                    const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
+                    v0 = __fmul_rn(acc0, __fmul_rn(s, acc1));
+                } else if (MODE == PH_RES) {
+                    v0 = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
+                    v1 = __fadd_rn(resv1, acc1);
+                } else {
+                    v0 = __fadd_rn(resv0, acc0 + acc1);
+                }
+                float *p0, *p1;
+                dst_of(item, pos, p0, p1);
+                st_coh(p0, v0);
+                if (p1) st_coh(p1, v1);
+            }
+        }
+    }
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
+{
+    extern __shared__ float4 smem4[];
+    MatvecRun<MODE> run(d);
+    // The weights do not depend on the input vector: the first loads go out before it is staged, so
+    // HBM latency overlaps the rmsnorm prologue.
+    run.preload();
+    run.run(smem4, d.st->token, d.st->pos);
 }
 
 // ---- decode attention: workgroup = (head, split); waves share the split's rows; online softmax ----
@@ -264,133 +383,191 @@ struct AttnPhase {
 constexpr int kAU = 2;  // cache rows in flight per lane group (K and V each)
 
 // LPR = lanes per cache row: each lane owns 4 consecutive floats of the head (head_size <= 4*LPR).
+// prefetch() requests the first cache rows of the workgroup's first item; rows of earlier positions do not
+// depend on this token, so in k_layer it runs before the wait for the phase that writes q and the row of
+// this position (that row is fetched in run()).
+template <int LPR>
+struct AttnRun {
+    static constexpr int RPW = 64 / LPR;
+    const AttnPhase a;
+    int hs, W, tid, lane, nent, len, chunk, nact, j, slot, nitems;
+    bool active, early = false;
+    float4 k4[kAU], v4[kAU];
+
+    __device__ __forceinline__ AttnRun(const AttnPhase &a_, int pos) : a(a_)
+    {
+        hs = a.head_size;
+        W = blockDim.x >> 6;
+        tid = phase_tid();
+        lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        nent = W * RPW;
+        len = pos + 1;
+        int nsplit = (len + a.rows_per_split - 1) / a.rows_per_split;  // short contexts: fewer, fuller splits
+        if (nsplit > a.nsplit) nsplit = a.nsplit;
+        chunk = (len + nsplit - 1) / nsplit;
+        nact = (len + chunk - 1) / chunk;
+        j = lane % LPR;
+        slot = wave * RPW + lane / LPR;
+        active = 4 * j < hs;
+        nitems = a.n_heads * nact;
+    }
+
+    // rows tb + u*nent (u < kAU) below t1; `part` 0: all of them, 1: only positions before this token's, 2: only this token's
+    __device__ __forceinline__ void fetch(int h, int tb, int t1, int part)
+    {
+        const long col = (long)(h / a.kv_mul) * hs + 4 * j;
+#pragma unroll
+        for (int u = 0; u < kAU; u++) {
+            const int t = tb + u * nent;
+            const bool want = part == 0 || (part == 1 ? t < len - 1 : t == len - 1);
+            if (t < t1 && active && want) {
+                k4[u] = load_stream(reinterpret_cast<const float4 *>(a.kc + (long)t * a.kv_dim + col));
+                v4[u] = load_stream(reinterpret_cast<const float4 *>(a.vc + (long)t * a.kv_dim + col));
+            }
+        }
+    }
+
+    __device__ __forceinline__ void clear()
+    {
+#pragma unroll
+        for (int u = 0; u < kAU; u++) k4[u] = v4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    __device__ __forceinline__ int store_waves() const { return (hs + 63) >> 6; }  // waves that store the output
+    __device__ __forceinline__ void preload() { prefetch(); }
+
+    __device__ __forceinline__ void prefetch()
+    {
+        clear();
+        early = true;
+        if ((int)blockIdx.x < nitems) {
+            const int s = blockIdx.x / a.n_heads, t0 = s * chunk;
+            fetch(blockIdx.x % a.n_heads, t0 + slot, min(len, t0 + chunk), 1);
+        }
+    }
+
+    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int
+    __device__ __forceinline__ void run(float *smem)
+    {
+        float *sm_m = smem;           // nent
+        float *sm_l = sm_m + nent;    // nent
+        float *sm_acc = sm_l + nent;  // nent * hs
+        int &s_last = *reinterpret_cast<int *>(sm_acc + nent * hs);
+
+        for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
+            const int h = it % a.n_heads, s = it / a.n_heads;
+            const int t0 = s * chunk, t1 = min(len, t0 + chunk);
+            float4 q4 = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (active) q4 = *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
+            float m = -3.402823466e+38f, l = 0.0f;
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int tb = t0 + slot; tb < t1; tb += nent * kAU) {
+                bool ok[kAU];
+#pragma unroll
+                for (int u = 0; u < kAU; u++) ok[u] = tb + u * nent < t1;
+                if (early && it == (int)blockIdx.x && tb == t0 + slot) {
+                    fetch(h, tb, t1, 2);  // only the row of this position is still missing
+                } else {
+                    clear();
+                    fetch(h, tb, t1, 0);
+                }
+                float sc[kAU], mb = m;
+#pragma unroll
+                for (int u = 0; u < kAU; u++) {
+                    // att[t] = (q . k_t) / sqrt(head_size)   (K/AttentionLoop.java:36-48)
+                    sc[u] = __fdiv_rn(group_sum<LPR>(dot4(q4, k4[u])), a.sqrt_hs);
+                    if (ok[u]) mb = fmaxf(mb, sc[u]);
+                }
+                // Online softmax, shifted by the running maximum of the scores.  The reference shifts by a
+                // running maximum of element products (K/AttentionLoop.java:44-51); softmax is shift
+                // invariant, so only rounding differs.
+                const float scale = expf(m - mb);  // 0 on the first batch (m = -FLT_MAX)
+                l *= scale;
+                acc.x *= scale; acc.y *= scale; acc.z *= scale; acc.w *= scale;
+#pragma unroll
+                for (int u = 0; u < kAU; u++) {
+                    const float p = ok[u] ? expf(sc[u] - mb) : 0.0f;
+                    l += p;
+                    acc.x = fmaf(p, v4[u].x, acc.x);  // K/AccumWeightedValue.java:48-62
+                    acc.y = fmaf(p, v4[u].y, acc.y);
+                    acc.z = fmaf(p, v4[u].z, acc.z);
+                    acc.w = fmaf(p, v4[u].w, acc.w);
+                }
+                m = mb;
+            }
+            __syncthreads();  // LDS reuse across items
+            if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
+            if (active) *reinterpret_cast<float4 *>(sm_acc + slot * hs + 4 * j) = acc;
+            __syncthreads();
+            // fold the row slots in a fixed order, so the result does not depend on timing
+            float M = -3.402823466e+38f, L = 0.0f, o = 0.0f;
+            for (int e = 0; e < nent; e++) M = fmaxf(M, sm_m[e]);
+            if (tid < hs) {
+                for (int e = 0; e < nent; e++) {
+                    const float w = expf(sm_m[e] - M);  // empty slots: exp(-huge) = 0
+                    L = fmaf(sm_l[e], w, L);
+                    o = fmaf(sm_acc[e * hs + tid], w, o);
+                }
+            }
+            if (nact == 1) {
+                if (tid < hs) st_coh(a.out + h * hs + tid, __fdiv_rn(o, L));
+                continue;
+            }
+            // Several splits: partials travel through memory with device-scope relaxed atomics (write-through
+            // stores, cache-bypassing loads), which is far cheaper here than a fence that writes back and
+            // invalidates the L2 of every XCD.  The split that arrives last folds them in split order.
+            float *mypart = a.part + ((long)h * a.nsplit + s) * (hs + 2);
+            if (tid < hs) st_coh(mypart + 2 + tid, o);
+            if (tid == 0) { st_coh(mypart, M); st_coh(mypart + 1, L); }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's partial stores have been acknowledged
+            __syncthreads();
+            if (tid == 0) s_last = (__hip_atomic_fetch_add(a.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(nact - 1));
+            __syncthreads();
+            if (!s_last) continue;
+            const float *hp = a.part + (long)h * a.nsplit * (hs + 2);
+            if (tid < hs) {
+                float MM = -3.402823466e+38f, LL = 0.0f, oo = 0.0f;
+                for (int i0 = 0; i0 < nact; i0 += 8) {
+                    float pm[8], pl[8], po[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const float *pp = hp + (long)min(i0 + i, nact - 1) * (hs + 2);
+                        pm[i] = ld_coh(pp);
+                        pl[i] = ld_coh(pp + 1);
+                        po[i] = ld_coh(pp + 2 + tid);
+                    }
+                    float mb = MM;
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        if (i0 + i < nact) mb = fmaxf(mb, pm[i]);
+                    const float scale = expf(MM - mb);
+                    LL *= scale;
+                    oo *= scale;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        if (i0 + i < nact) {
+                            const float w = expf(pm[i] - mb);
+                            LL = fmaf(pl[i], w, LL);
+                            oo = fmaf(po[i], w, oo);
+                        }
+                    }
+                    MM = mb;
+                }
+                st_coh(a.out + h * hs + tid, __fdiv_rn(oo, LL));
+            }
+            if (tid == 0) st_coh(a.counters + h, 0u);
+        }
+    }
+};
+
 template <int LPR>
 __global__ void __launch_bounds__(1024) k_attention(const AttnPhase a)
 {
     extern __shared__ float smem[];
-    constexpr int RPW = 64 / LPR;
-    const int hs = a.head_size, W = blockDim.x >> 6, tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nent = W * RPW;
-    float *sm_m = smem;                 // nent
-    float *sm_l = sm_m + nent;          // nent
-    float *sm_acc = sm_l + nent;        // nent * hs
-    __shared__ int s_last;
-
-    const int len = a.st->pos + 1;
-    int nsplit = (len + a.rows_per_split - 1) / a.rows_per_split;  // short contexts: fewer, fuller splits
-    if (nsplit > a.nsplit) nsplit = a.nsplit;
-    const int chunk = (len + nsplit - 1) / nsplit;
-    const int nact = (len + chunk - 1) / chunk;
-    const int j = lane % LPR, slot = wave * RPW + lane / LPR;
-    const bool active = 4 * j < hs;
-
-    for (int it = blockIdx.x; it < a.n_heads * nact; it += gridDim.x) {
-        const int h = it % a.n_heads, s = it / a.n_heads;
-        const int t0 = s * chunk, t1 = min(len, t0 + chunk);
-        const long col = (long)(h / a.kv_mul) * hs + 4 * j;
-        float4 q4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (active) q4 = *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
-        float m = -3.402823466e+38f, l = 0.0f;
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int tb = t0 + slot; tb < t1; tb += nent * kAU) {
-            float4 k4[kAU], v4[kAU];
-            bool ok[kAU];
-#pragma unroll
-            for (int u = 0; u < kAU; u++) {
-                const int t = tb + u * nent;
-                ok[u] = t < t1;
-                k4[u] = v4[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (ok[u] && active) {
-                    k4[u] = load_stream(reinterpret_cast<const float4 *>(a.kc + (long)t * a.kv_dim + col));
-                    v4[u] = load_stream(reinterpret_cast<const float4 *>(a.vc + (long)t * a.kv_dim + col));
-                }
-            }
-            float sc[kAU], mb = m;
-#pragma unroll
-            for (int u = 0; u < kAU; u++) {
-                // att[t] = (q . k_t) / sqrt(head_size)   (K/AttentionLoop.java:36-48)
-                sc[u] = __fdiv_rn(group_sum<LPR>(dot4(q4, k4[u])), a.sqrt_hs);
-                if (ok[u]) mb = fmaxf(mb, sc[u]);
-            }
-            // Online softmax, shifted by the running maximum of the scores.  The reference shifts by a
-            // running maximum of element products (K/AttentionLoop.java:44-51); softmax is shift
-            // invariant, so only rounding differs.
-            const float scale = expf(m - mb);  // 0 on the first batch (m = -FLT_MAX)
-            l *= scale;
-            acc.x *= scale; acc.y *= scale; acc.z *= scale; acc.w *= scale;
-#pragma unroll
-            for (int u = 0; u < kAU; u++) {
-                const float p = ok[u] ? expf(sc[u] - mb) : 0.0f;
-                l += p;
-                acc.x = fmaf(p, v4[u].x, acc.x);  // K/AccumWeightedValue.java:48-62
-                acc.y = fmaf(p, v4[u].y, acc.y);
-                acc.z = fmaf(p, v4[u].z, acc.z);
-                acc.w = fmaf(p, v4[u].w, acc.w);
-            }
-            m = mb;
-        }
-        __syncthreads();  // LDS reuse across items
-        if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
-        if (active) *reinterpret_cast<float4 *>(sm_acc + slot * hs + 4 * j) = acc;
-        __syncthreads();
-        // fold the row slots in a fixed order, so the result does not depend on timing
-        float M = -3.402823466e+38f, L = 0.0f, o = 0.0f;
-        for (int e = 0; e < nent; e++) M = fmaxf(M, sm_m[e]);
-        if (tid < hs) {
-            for (int e = 0; e < nent; e++) {
-                const float w = expf(sm_m[e] - M);  // empty slots: exp(-huge) = 0
-                L = fmaf(sm_l[e], w, L);
-                o = fmaf(sm_acc[e * hs + tid], w, o);
-            }
-        }
-        if (nact == 1) {
-            if (tid < hs) a.out[h * hs + tid] = __fdiv_rn(o, L);
-            continue;
-        }
-        // Several splits: partials travel through memory with device-scope relaxed atomics (write-through
-        // stores, cache-bypassing loads), which is far cheaper here than a fence that writes back and
-        // invalidates the L2 of every XCD.  The split that arrives last folds them in split order.
-        float *mypart = a.part + ((long)h * a.nsplit + s) * (hs + 2);
-        if (tid < hs) st_coh(mypart + 2 + tid, o);
-        if (tid == 0) { st_coh(mypart, M); st_coh(mypart + 1, L); }
-        __syncthreads();  // the partial stores of every wave have completed
-        if (tid == 0) s_last = (__hip_atomic_fetch_add(a.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(nact - 1));
-        __syncthreads();
-        if (!s_last) continue;
-        const float *hp = a.part + (long)h * a.nsplit * (hs + 2);
-        if (tid < hs) {
-            float MM = -3.402823466e+38f, LL = 0.0f, oo = 0.0f;
-            for (int i0 = 0; i0 < nact; i0 += 8) {
-                float pm[8], pl[8], po[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    const float *pp = hp + (long)min(i0 + i, nact - 1) * (hs + 2);
-                    pm[i] = ld_coh(pp);
-                    pl[i] = ld_coh(pp + 1);
-                    po[i] = ld_coh(pp + 2 + tid);
-                }
-                float mb = MM;
-#pragma unroll
-                for (int i = 0; i < 8; i++)
-                    if (i0 + i < nact) mb = fmaxf(mb, pm[i]);
-                const float scale = expf(MM - mb);
-                LL *= scale;
-                oo *= scale;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    if (i0 + i < nact) {
-                        const float w = expf(pm[i] - mb);
-                        LL = fmaf(pl[i], w, LL);
-                        oo = fmaf(po[i], w, oo);
-                    }
-                }
-                MM = mb;
-            }
-            a.out[h * hs + tid] = __fdiv_rn(oo, LL);
-        }
-        if (tid == 0) st_coh(a.counters + h, 0u);
-    }
+    AttnRun<LPR> run(a, a.st->pos);
+    run.clear();
+    run.run(smem);
 }
 
 // ---- final rmsnorm + fp32 classifier + per-workgroup first-max -----------------------------------
@@ -407,58 +584,283 @@ struct ClsPhase {
     DevState *st;
     const int *prompt;   // seq_len
     int *out_tokens;     // seq_len
+    unsigned *bar_ctr;   // grid barrier counters of the token, zeroed for the next one
+    int nbar;
 };
 
 constexpr int kCU = 8;
 
+struct ClsRun {
+    const ClsPhase a;
+    int n, nch, n4, lane, wave, W, G, row;
+    bool first = false;
+    float4 pre[kCU];
+
+    __device__ __forceinline__ ClsRun(const ClsPhase &a_) : a(a_)
+    {
+        n = a.n;
+        nch = n >> 4;
+        n4 = n >> 2;
+        const int tid = phase_tid();
+        lane = tid & 63;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        W = blockDim.x >> 6;
+        G = gridDim.x;
+        row = wave * G + blockIdx.x;
+    }
+
+    __device__ __forceinline__ void issue(int r, int base)
+    {
+        const float4 *wr = reinterpret_cast<const float4 *>(a.w + (long)r * n);
+#pragma unroll
+        for (int u = 0; u < kCU; u++) {
+            const int c = base + 64 * u + lane;
+            pre[u] = load_stream(wr + (c < n4 ? c : n4 - 1));
+        }
+    }
+
+    __device__ __forceinline__ void preload()
+    {
+        first = row < a.vocab;
+        if (first) {
+            issue(row, 0);
+        } else {
+#pragma unroll
+            for (int u = 0; u < kCU; u++) pre[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+
+    // smem: as for a matvec phase, then 16 floats and 16 ints for the per-wave maxima
+    __device__ __forceinline__ void run(float4 *smem4)
+    {
+        float4 *xs = smem4;
+        float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
+        float *red = sumx + nch;
+        float *bval = red + 16;
+        int *bidx = reinterpret_cast<int *>(red + 32);
+        stage_vector(a.xin, n, a.rmsw, xs, sumx, red);
+
+        float best_v = -__builtin_inff();
+        int best_i = 0x7fffffff;
+        for (; row < a.vocab; row += W * G) {
+            float acc = 0.0f;
+            for (int base = 0; base < n4; base += 64 * kCU) {
+                if (!(first && base == 0)) issue(row, base);
+#pragma unroll
+                for (int u = 0; u < kCU; u++) {
+                    const int c = base + 64 * u + lane;
+                    const bool ok = c < n4;
+                    const int cc = ok ? c : n4 - 1;
+                    const float t = dot4(pre[u], xs[(cc & 3) * nch + (cc >> 2)]);
+                    acc += ok ? t : 0.0f;
+                }
+            }
+            first = false;
+            acc = wave_sum(acc);
+            if (lane == 0) {
+                a.logits[row] = acc;
+                if (better(acc, row, best_v, best_i)) { best_v = acc; best_i = row; }
+            }
+        }
+        if (lane == 0) { bval[wave] = best_v; bidx[wave] = best_i; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < W; w++)
+                if (better(bval[w], bidx[w], best_v, best_i)) { best_v = bval[w]; best_i = bidx[w]; }
+            a.part_val[blockIdx.x] = best_v;
+            a.part_idx[blockIdx.x] = best_i;
+        }
+    }
+};
+
 __global__ void __launch_bounds__(1024) k_classifier(const ClsPhase a)
 {
     extern __shared__ float4 smem4[];
-    const int n = a.n, nch = n >> 4, n4 = n >> 2;
-    float4 *xs = smem4;
-    float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
-    float *red = sumx + nch;
-    float *bval = red + 16;
-    int *bidx = reinterpret_cast<int *>(red + 32);
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int W = blockDim.x >> 6, G = gridDim.x;
+    ClsRun run(a);
+    run.preload();
+    run.run(smem4);
+}
 
-    stage_vector(a.xin, n, a.rmsw, xs, sumx, red);
+// ---- layers [l0, l1) and optionally the classifier in one launch ------------------------------------
+// Grid: one workgroup per compute unit, all resident.  Barrier instance 5*l + k follows phase k of layer l.
 
-    float best_v = -__builtin_inff();
-    int best_i = 0x7fffffff;
-    for (int row = wave * G + blockIdx.x; row < a.vocab; row += W * G) {
-        const float4 *wr = reinterpret_cast<const float4 *>(a.w + (long)row * n);
-        float acc = 0.0f;
-        for (int base = 0; base < n4; base += 64 * kCU) {
-            float4 pre[kCU];
-#pragma unroll
-            for (int u = 0; u < kCU; u++) {
-                const int c = base + 64 * u + lane;
-                pre[u] = load_stream(wr + (c < n4 ? c : n4 - 1));
-            }
-#pragma unroll
-            for (int u = 0; u < kCU; u++) {
-                const int c = base + 64 * u + lane;
-                const bool ok = c < n4;
-                const int cc = ok ? c : n4 - 1;
-                const float t = dot4(pre[u], xs[(cc & 3) * nch + (cc >> 2)]);
-                acc += ok ? t : 0.0f;
-            }
-        }
-        acc = wave_sum(acc);
-        if (lane == 0) {
-            a.logits[row] = acc;
-            if (better(acc, row, best_v, best_i)) { best_v = acc; best_i = row; }
-        }
+enum { K_QKV = 0, K_ATT = 1, K_WO = 2, K_W13 = 3, K_W2 = 4, K_CLS = 5 };
+
+// Everything the phases of a token are built from.  The phase arguments of layer l are derived from it on
+// the host (one launch per phase) and on the device (k_token) by the same functions.
+struct TokenGeom {
+    int dim, hidden, n_layers, n_heads, kv_mul, head_size, kv_dim, seq_len, vocab, exact_silu;
+    long sd, sh;  // strides of dim-long and hidden-long activation vectors, in floats
+    const float *emb, *rmsw, *silu, *wcls;
+    const float2 *rope;
+    float *x, *xb, *hb, *q, *kcache, *vcache, *logits;
+    QMat wq, wk, wv, wo, w1, w2, w3;  // off = 0: layer 0
+    float *attn_part;
+    unsigned *attn_counters;
+    int attn_nsplit;
+    float sqrt_hs;
+    DevState *st;
+    float *cls_val;
+    int *cls_idx;
+    const int *prompt;
+    int *out_tokens;
+    unsigned *bar_ctr;
+    int nbar;
+    int *fault;
+};
+
+// The builders below are templates on the geometry's type so that the device can read it straight from the
+// kernel-argument segment (constant address space, scalar loads) instead of from a copy in registers.
+template <class M>
+__host__ __device__ inline QMat at_layer(const M &m, long floats_per_layer, int l)
+{
+    QMat r;
+    r.codes = m.codes;
+    r.gs = m.gs;
+    r.off = m.off + floats_per_layer * l;
+    return r;
+}
+
+// Arguments of the phases of layer l (J/Run.java:76-159).
+template <class G>
+__host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, int l)
+{
+    const long dim = g.dim, hid = g.hidden, kvd = g.kv_dim;
+    const long kvoff = (long)l * g.seq_len * kvd;
+    MatvecPhase d{};
+    d.emb = g.emb; d.rope = g.rope; d.silu = g.silu; d.st = g.st;
+    d.head_size = g.head_size; d.kv_dim = g.kv_dim; d.exact_silu = g.exact_silu;
+    switch (kclass) {
+    case K_QKV:
+        d.n = g.dim; d.from_emb = l == 0; d.xin = g.x + 2 * l * g.sd; d.rmsw = g.rmsw + l * dim;
+        d.d0 = g.dim; d.d1 = d.d2 = g.kv_dim;
+        d.m0 = at_layer(g.wq, dim * dim, l); d.m1 = at_layer(g.wk, dim * kvd, l); d.m2 = at_layer(g.wv, dim * kvd, l);
+        d.out0 = g.q + l * g.sd; d.out1 = g.kcache + kvoff; d.out2 = g.vcache + kvoff;
+        break;
+    case K_WO:
+        d.n = g.dim; d.xin = g.xb + l * g.sd; d.d0 = g.dim; d.m0 = at_layer(g.wo, dim * dim, l);
+        d.out0 = g.x + (2 * l + 1) * g.sd; d.res_src = g.x + 2 * l * g.sd; d.res_emb = l == 0;
+        break;
+    case K_W13:
+        d.n = g.dim; d.xin = g.x + (2 * l + 1) * g.sd; d.rmsw = g.rmsw + (g.n_layers + l) * dim; d.d0 = g.hidden;
+        d.m0 = at_layer(g.w1, dim * hid, l); d.m1 = at_layer(g.w3, dim * hid, l); d.out0 = g.hb + l * g.sh;
+        break;
+    default:  // K_W2
+        d.n = g.hidden; d.xin = g.hb + l * g.sh; d.d0 = g.dim; d.m0 = at_layer(g.w2, dim * hid, l);
+        d.out0 = g.x + (2 * l + 2) * g.sd; d.res_src = g.x + (2 * l + 1) * g.sd;
+        break;
     }
-    if (lane == 0) { bval[wave] = best_v; bidx[wave] = best_i; }
+    return d;
+}
+
+template <class G>
+__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split)
+{
+    const long kvoff = (long)l * g.seq_len * g.kv_dim;
+    AttnPhase t{};
+    t.q = g.q + l * g.sd; t.kc = g.kcache + kvoff; t.vc = g.vcache + kvoff; t.out = g.xb + l * g.sd;
+    t.part = g.attn_part; t.counters = g.attn_counters; t.st = g.st;
+    t.n_heads = g.n_heads; t.kv_mul = g.kv_mul; t.head_size = g.head_size; t.kv_dim = g.kv_dim;
+    t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split;
+    t.sqrt_hs = g.sqrt_hs;  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
+    return t;
+}
+
+template <class G>
+__host__ __device__ inline ClsPhase cls_phase_of(const G &g, int nparts)
+{
+    ClsPhase a{};
+    a.xin = g.x + 2L * g.n_layers * g.sd; a.rmsw = g.rmsw + 2L * g.n_layers * g.dim; a.w = g.wcls;
+    a.n = g.dim; a.vocab = g.vocab; a.logits = g.logits; a.part_val = g.cls_val; a.part_idx = g.cls_idx; a.nparts = nparts;
+    a.st = g.st; a.prompt = g.prompt; a.out_tokens = g.out_tokens; a.bar_ctr = g.bar_ctr; a.nbar = g.nbar;
+    return a;
+}
+
+// Long rows are streamed one row per wave (PH_ROW) so every wave has work; shorter ones as row pairs (PH_RES).
+__host__ __device__ inline bool row_mode(int n) { return n / 16 > 64 * kTU; }
+
+struct TokenArgs {
+    TokenGeom g;
+    int l0, l1, with_cls;   // layers [l0, l1), then the classifier when with_cls
+    int attn_rows;          // cache rows per attention split in this kernel
+    int maxspin;
+};
+
+// Between two phases: every wave waits for its own stores to be acknowledged, the workgroup arrives at the
+// barrier, requests the first weights of the next phase, and only then waits for the other workgroups.
+template <class Next>
+__device__ __forceinline__ void handoff(const GridBar &b, int inst, Next &nx)
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < W; w++)
-            if (better(bval[w], bidx[w], best_v, best_i)) { best_v = bval[w]; best_i = bidx[w]; }
-        a.part_val[blockIdx.x] = best_v;
-        a.part_idx[blockIdx.x] = best_i;
+    bar_arrive(b, inst);
+    nx.preload();
+    bar_wait(b, inst);
+}
+
+// The kernel arguments, re-read from the kernel-argument segment by every phase: the pointer goes through an
+// empty asm so the compiler cannot keep all ~100 argument words live in scalar registers across the layer
+// loop (which spills), and each phase loads just the words it uses.
+typedef const __attribute__((address_space(4))) TokenArgs *TokenArgsPtr;
+__device__ __forceinline__ TokenArgsPtr token_args()
+{
+    TokenArgsPtr p = (TokenArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return p;
+}
+
+template <int W2_MODE>
+__device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4, int token, int pos)
+{
+    MatvecRun<W2_MODE> w2(matvec_phase_of(token_args()->g, K_W2, l));
+    handoff(b, 5 * l + 3, w2);
+    w2.run(smem4, token, pos);
+}
+
+template <int WO_MODE>
+__device__ __forceinline__ void token_wo(const GridBar &b, int l, float4 *smem4, int token, int pos)
+{
+    MatvecRun<WO_MODE> wo(matvec_phase_of(token_args()->g, K_WO, l));
+    handoff(b, 5 * l + 1, wo);
+    wo.run(smem4, token, pos);
+}
+
+template <int LPR>
+__global__ void __launch_bounds__(1024) k_token(const TokenArgs)
+{
+    extern __shared__ float4 smem4[];
+    TokenArgsPtr t = token_args();
+    const int token = t->g.st->token, pos = t->g.st->pos;
+    const int l0 = t->l0, l1 = t->l1;
+    const bool wo_row = row_mode(t->g.dim), w2_row = row_mode(t->g.hidden);
+    GridBar b;
+    b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = kBarGroups; b.maxspin = t->maxspin;
+    for (int l = l0; l < l1; l++) {
+        {
+            MatvecRun<PH_QKV> qkv(matvec_phase_of(token_args()->g, K_QKV, l));
+            if (l == l0) qkv.preload();             // launch order guarantees the input
+            else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
+            qkv.run(smem4, token, pos);
+        }
+        {
+            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows), pos);
+            handoff(b, 5 * l, att);
+            att.run(reinterpret_cast<float *>(smem4));
+        }
+        if (wo_row) token_wo<PH_ROW>(b, l, smem4, token, pos);
+        else token_wo<PH_RES>(b, l, smem4, token, pos);
+        {
+            MatvecRun<PH_W13> w13(matvec_phase_of(token_args()->g, K_W13, l));
+            handoff(b, 5 * l + 2, w13);
+            w13.run(smem4, token, pos);
+        }
+        if (w2_row) token_w2<PH_ROW>(b, l, smem4, token, pos);
+        else token_w2<PH_RES>(b, l, smem4, token, pos);
+    }
+    if (token_args()->with_cls) {
+        ClsRun cls(cls_phase_of(token_args()->g, gridDim.x));
+        handoff(b, 5 * (l1 - 1) + 4, cls);
+        cls.run(smem4);
     }
 }
 
@@ -470,6 +872,8 @@ __global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
     __shared__ int bidx[16];
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < a.nbar * (1 + kBarGroups); i += blockDim.x)
+        st_coh(a.bar_ctr + (long)(i / (1 + kBarGroups)) * kBarStride + 64 * (i % (1 + kBarGroups)), 0u);
     for (int b = threadIdx.x; b < a.nparts; b += blockDim.x) {
         const float v = a.part_val[b];
         const int i = a.part_idx[b];

@@ -166,6 +166,25 @@ def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
         assert nxt == int(np.argmax(outs[0][p]))
 
 
+def test_split_attention_in_both_launch_modes(orc):
+    # contexts long enough that attention is split over several workgroups (whole-token launch: beyond 64
+    # positions; kernel-by-kernel: beyond 32) and folded by the last arriver; multiquery, head 16
+    shape = (64, 96, 2, 4, 2, 40, 200, 1)
+    m, g = make_pair(orc, shape, seed=33, realistic=True)
+    rng = np.random.default_rng(5)
+    toks = rng.integers(0, shape[5], size=shape[6])
+    fused = []
+    for pos, tok in enumerate(toks):
+        want = m.forward(int(tok), pos)
+        got = g.forward(int(tok), pos)
+        assert rel_err(got, want) < 1e-4, pos
+        fused.append(got.copy())
+    g.reset()
+    for pos, tok in enumerate(toks):
+        got = g.forward_taps(int(tok), pos)
+        assert rel_err(got, fused[pos]) < 1e-5, pos
+
+
 def test_argmax_first_max_tie_rule(orc):
     # identical classifier rows give exactly equal logits: the lowest index must win (J/Sampler.java:51)
     shape = (64, 256, 1, 4, 4, 1000, 4, 0)
@@ -392,6 +411,7 @@ def test_config4_long_context_attention(orc):
             a, b = g.read(BUFFER.XB, layer=l), m.tap(orc.TAP_ATT_OUT, l)
             assert np.abs(a - b).max() <= 2e-5 * max(1.0, float(np.abs(b).max())), (pos, l)
         assert rel_err(got, want) < LOGIT_TOL, pos
+        assert rel_err(g.forward(17, pos), want) < LOGIT_TOL, pos  # the whole-token launch at the same position
     # round trip of the cache taps
     np.testing.assert_array_equal(g.read(BUFFER.VCACHE, layer=1, off=5 * kvd, n=kvd), vc[1, 5])
 
