@@ -29,8 +29,8 @@ class BUFFER:
 
 
 class KERNEL:
-    QKV, ATTENTION, WO, W13, W2, CLASSIFIER = range(6)
-    NAMES = ("qkv", "attention", "wo", "w13", "w2", "classifier")
+    QKV, ATTENTION, WO, W13, W2, CLASSIFIER, TOKEN = range(7)
+    NAMES = ("qkv", "attention", "wo", "w13", "w2", "classifier", "token")
 
 
 class L2JError(RuntimeError):

@@ -213,7 +213,7 @@ bool geom_complete(const TokenGeom &t)
 }
 
 // Layers [l0, l1) (and the classifier after the last layer) in one launch of k_token.
-hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s)
+hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
 {
     TokenArgs a{};
     a.g = c->geom;
@@ -223,9 +223,15 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s)
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
     const int lpr = attn_lpr(c);
-    if (lpr == 16) hipLaunchKernelGGL(k_token<16>, grid, block, smem, s, a);
-    else if (lpr == 32) hipLaunchKernelGGL(k_token<32>, grid, block, smem, s, a);
-    else hipLaunchKernelGGL(k_token<64>, grid, block, smem, s, a);
+    if (e0) {
+        if (lpr == 16) hipExtLaunchKernelGGL(k_token<16>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
+        else if (lpr == 32) hipExtLaunchKernelGGL(k_token<32>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
+        else hipExtLaunchKernelGGL(k_token<64>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
+    } else {
+        if (lpr == 16) hipLaunchKernelGGL(k_token<16>, grid, block, smem, s, a);
+        else if (lpr == 32) hipLaunchKernelGGL(k_token<32>, grid, block, smem, s, a);
+        else hipLaunchKernelGGL(k_token<64>, grid, block, smem, s, a);
+    }
     return hipGetLastError();
 }
 
@@ -975,8 +981,32 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
     case L2J_K_W13: b = quant_bytes_of(2 * dim * hid) + quant_bytes_of(dim); break;
     case L2J_K_W2: b = quant_bytes_of(dim * hid); break;
     case L2J_K_CLASSIFIER: b = (uint64_t)g.vocab_size * dim * 4 + quant_bytes_of(dim); break;
+    case L2J_K_TOKEN: b = l2j_bytes_per_token(&g, pos); break;
     }
     if (bytes) *bytes = b;
+    if (kclass == L2J_K_TOKEN) {  // the whole-token kernel, then k_finish (untimed) to reset the barrier counters
+        if (!c->fused) return fail(L2J_E_STATE, "the whole-token kernel is switched off or does not fit this shape");
+        while ((int)c->events.size() < 35) {
+            hipEvent_t ev;
+            HIPCHK(hipEventCreate(&ev));
+            c->events.push_back(ev);
+        }
+        double total = 0.0;
+        for (int r = 0; r < rounds; r++) {
+            if ((rc = set_state(c, 1, pos, 0))) return rc;
+            hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33], c->events[34]);
+            if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
+            hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));
+            HIPCHK(hipGetLastError());
+            HIPCHK(hipStreamSynchronize(c->stream));
+            if ((rc = check_barrier_error(c))) return rc;
+            float ms = 0.f;
+            HIPCHK(hipEventElapsedTime(&ms, c->events[33], c->events[34]));
+            total += ms;
+        }
+        *mean_us = total * 1e3 / rounds;
+        return L2J_OK;
+    }
     const int per_round = kclass == L2J_K_CLASSIFIER ? 1 : g.n_layers;
     while ((int)c->events.size() < 2 * per_round + 33) {
         hipEvent_t ev;

@@ -185,6 +185,24 @@ def test_split_attention_in_both_launch_modes(orc):
         assert rel_err(got, fused[pos]) < 1e-5, pos
 
 
+def test_kernel_timing_entry_point(orc):
+    # every kernel class launches and reports a time, deep enough in the context that attention is split;
+    # the measurement leaves the context usable (same tokens before and after)
+    shape = (64, 96, 2, 4, 2, 40, 200, 1)
+    m, g = make_pair(orc, shape, seed=34, realistic=True)
+    prompt = orc.synth_prompt(34, 4, shape[5])
+    before, _ = g.decode_greedy(prompt, 160)
+    for k in range(7):
+        us, nbytes = g.time_kernel(k, 150, rounds=2)
+        assert us > 0.0 and nbytes > 0, k
+    assert g.time_kernel(l2j.KERNEL.TOKEN, 150, rounds=1)[1] == g.bytes_per_token(150)
+    g.reset()
+    after, _ = g.decode_greedy(prompt, 160)
+    np.testing.assert_array_equal(before, after)
+    want, _, _ = m.generate_greedy(prompt, 160)
+    np.testing.assert_array_equal(after, want)
+
+
 def test_argmax_first_max_tie_rule(orc):
     # identical classifier rows give exactly equal logits: the lowest index must win (J/Sampler.java:51)
     shape = (64, 256, 1, 4, 4, 1000, 4, 0)
