@@ -92,10 +92,10 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
-// Block-wide sum / max through LDS; `red` holds one float per wave.  All threads get the result.
-__device__ __forceinline__ float block_sum(float v, float *red)
+// Block-wide sum / max through LDS; `red` holds one float per wave (nw waves).  All threads get the result.
+__device__ __forceinline__ float block_sum(float v, float *red, int nw)
 {
-    const int wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int wave = threadIdx.x >> 6;
     v = wave_sum(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[wave] = v;

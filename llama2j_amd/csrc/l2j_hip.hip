@@ -179,7 +179,7 @@ static_assert(K_QKV == L2J_K_QKV && K_ATT == L2J_K_ATTENTION && K_WO == L2J_K_WO
               K_CLS == L2J_K_CLASSIFIER, "kernel classes of the C ABI and of the device code must agree");
 
 MatvecPhase matvec_phase(const l2j_ctx *c, int kclass, int l) { return matvec_phase_of(c->geom, kclass, l); }
-AttnPhase attn_phase(const l2j_ctx *c, int l) { return attn_phase_of(c->geom, l, c->attn_rows); }
+AttnPhase attn_phase(const l2j_ctx *c, int l) { return attn_phase_of(c->geom, l, c->attn_rows, c->attn_threads); }
 ClsPhase cls_phase(const l2j_ctx *c) { return cls_phase_of(c->geom, c->pk_grid); }
 
 void build_geom(l2j_ctx *c)
@@ -189,6 +189,7 @@ void build_geom(l2j_ctx *c)
     t.dim = g.dim; t.hidden = g.hidden_dim; t.n_layers = g.n_layers; t.n_heads = g.n_heads; t.kv_mul = c->kv_mul;
     t.head_size = c->head_size; t.kv_dim = c->kv_dim; t.seq_len = g.seq_len; t.vocab = g.vocab_size;
     t.exact_silu = (g.flags & L2J_F_EXACT_SILU) ? 1 : 0;
+    t.threads = c->pk_threads;
     t.sd = (long)c->sd; t.sh = (long)c->sh;
     t.emb = c->emb; t.rmsw = c->rmsw; t.silu = c->silu; t.wcls = c->wcls; t.rope = c->rope;
     t.x = c->x; t.xb = c->xb; t.hb = c->hb; t.q = c->q; t.kcache = c->kcache; t.vcache = c->vcache; t.logits = c->logits;

@@ -45,7 +45,7 @@ struct GridBar {
     int *fault;
     int ngroups, maxspin;
 };
-constexpr int kBarGroups = 8;
+constexpr int kBarGroups = 4;   // measured: 4 groups of 64 beat 8 of 32 and 2 of 128 at 256 workgroups
 constexpr int kBarStride = 64 * (1 + kBarGroups);  // unsigned words per barrier instance
 
 // Called when every store of the workgroup that the other workgroups will read has been acknowledged
@@ -106,6 +106,7 @@ struct MatvecPhase {
     const float *silu;          // sigmoid table
     const DevState *st;
     int head_size, kv_dim, exact_silu;
+    int threads;    // workgroup size (a kernel argument: reading it from the dispatch costs a vector load per phase)
 };
 
 // ---- activation vector -> LDS ------------------------------------------------------------------
@@ -114,9 +115,9 @@ struct MatvecPhase {
 // sumx[c] = sum of the 16 activations of chunk c (for the group-minimum term of the dequantization).
 
 __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
-                                             float *sumx, float *red)
+                                             float *sumx, float *red, int T)
 {
-    const int nch = n >> 4, tid = phase_tid(), T = blockDim.x;
+    const int nch = n >> 4, tid = phase_tid();
     if (rmsw) {
         float ssq = 0.0f;
         for (int c = tid; c < nch; c += T) {
@@ -129,7 +130,7 @@ __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int 
             ssq += (a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w) + (b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w) +
                    (cc.x * cc.x + cc.y * cc.y + cc.z * cc.z + cc.w * cc.w) + (d.x * d.x + d.y * d.y + d.z * d.z + d.w * d.w);
         }
-        ssq = block_sum(ssq, red);
+        ssq = block_sum(ssq, red, T >> 6);
         // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
         const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
         for (int c = tid; c < nch; c += T) {
@@ -193,7 +194,7 @@ struct MatvecRun {
         n = d.n;
         nch = n >> 4;
         lane = tid & 63;
-        W = blockDim.x >> 6;
+        W = d.threads >> 6;
         G = gridDim.x;
         nitems = MODE == PH_QKV ? (d.d0 + d.d1 + d.d2) >> 1 : MODE == PH_RES ? (d.d0 + 1) >> 1 : d.d0;
         // Items are dealt block-minor (item -> workgroup item % G), so every compute unit gets the same
@@ -289,7 +290,7 @@ struct MatvecRun {
         float *red = sumx + nch;
         const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
         const float *res = d.res_emb ? emb_row : d.res_src;
-        stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red);
+        stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
 
         for (; item < nitems; item += W * G) {
             if (!first) resolve(item);
@@ -378,6 +379,7 @@ struct AttnPhase {
     const DevState *st;
     int n_heads, kv_mul, head_size, kv_dim, nsplit, rows_per_split;
     float sqrt_hs;
+    int threads;           // workgroup size
 };
 
 constexpr int kAU = 2;  // cache rows in flight per lane group (K and V each)
@@ -397,7 +399,7 @@ struct AttnRun {
     __device__ __forceinline__ AttnRun(const AttnPhase &a_, int pos) : a(a_)
     {
         hs = a.head_size;
-        W = blockDim.x >> 6;
+        W = a.threads >> 6;
         tid = phase_tid();
         lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -586,6 +588,7 @@ struct ClsPhase {
     int *out_tokens;     // seq_len
     unsigned *bar_ctr;   // grid barrier counters of the token, zeroed for the next one
     int nbar;
+    int threads;         // workgroup size of the classifier
 };
 
 constexpr int kCU = 8;
@@ -604,7 +607,7 @@ struct ClsRun {
         const int tid = phase_tid();
         lane = tid & 63;
         wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        W = blockDim.x >> 6;
+        W = a.threads >> 6;
         G = gridDim.x;
         row = wave * G + blockIdx.x;
     }
@@ -638,7 +641,7 @@ struct ClsRun {
         float *red = sumx + nch;
         float *bval = red + 16;
         int *bidx = reinterpret_cast<int *>(red + 32);
-        stage_vector(a.xin, n, a.rmsw, xs, sumx, red);
+        stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
 
         float best_v = -__builtin_inff();
         int best_i = 0x7fffffff;
@@ -690,6 +693,7 @@ enum { K_QKV = 0, K_ATT = 1, K_WO = 2, K_W13 = 3, K_W2 = 4, K_CLS = 5 };
 // the host (one launch per phase) and on the device (k_token) by the same functions.
 struct TokenGeom {
     int dim, hidden, n_layers, n_heads, kv_mul, head_size, kv_dim, seq_len, vocab, exact_silu;
+    int threads;  // workgroup size of the matvec phases, the classifier and k_token
     long sd, sh;  // strides of dim-long and hidden-long activation vectors, in floats
     const float *emb, *rmsw, *silu, *wcls;
     const float2 *rope;
@@ -729,7 +733,7 @@ __host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, i
     const long kvoff = (long)l * g.seq_len * kvd;
     MatvecPhase d{};
     d.emb = g.emb; d.rope = g.rope; d.silu = g.silu; d.st = g.st;
-    d.head_size = g.head_size; d.kv_dim = g.kv_dim; d.exact_silu = g.exact_silu;
+    d.head_size = g.head_size; d.kv_dim = g.kv_dim; d.exact_silu = g.exact_silu; d.threads = g.threads;
     switch (kclass) {
     case K_QKV:
         d.n = g.dim; d.from_emb = l == 0; d.xin = g.x + 2 * l * g.sd; d.rmsw = g.rmsw + l * dim;
@@ -754,14 +758,14 @@ __host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, i
 }
 
 template <class G>
-__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split)
+__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split, int threads)
 {
     const long kvoff = (long)l * g.seq_len * g.kv_dim;
     AttnPhase t{};
     t.q = g.q + l * g.sd; t.kc = g.kcache + kvoff; t.vc = g.vcache + kvoff; t.out = g.xb + l * g.sd;
     t.part = g.attn_part; t.counters = g.attn_counters; t.st = g.st;
     t.n_heads = g.n_heads; t.kv_mul = g.kv_mul; t.head_size = g.head_size; t.kv_dim = g.kv_dim;
-    t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split;
+    t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split; t.threads = threads;
     t.sqrt_hs = g.sqrt_hs;  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
     return t;
 }
@@ -772,7 +776,7 @@ __host__ __device__ inline ClsPhase cls_phase_of(const G &g, int nparts)
     ClsPhase a{};
     a.xin = g.x + 2L * g.n_layers * g.sd; a.rmsw = g.rmsw + 2L * g.n_layers * g.dim; a.w = g.wcls;
     a.n = g.dim; a.vocab = g.vocab; a.logits = g.logits; a.part_val = g.cls_val; a.part_idx = g.cls_idx; a.nparts = nparts;
-    a.st = g.st; a.prompt = g.prompt; a.out_tokens = g.out_tokens; a.bar_ctr = g.bar_ctr; a.nbar = g.nbar;
+    a.st = g.st; a.prompt = g.prompt; a.out_tokens = g.out_tokens; a.bar_ctr = g.bar_ctr; a.nbar = g.nbar; a.threads = g.threads;
     return a;
 }
 
@@ -843,7 +847,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             qkv.run(smem4, token, pos);
         }
         {
-            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows), pos);
+            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads), pos);
             handoff(b, 5 * l, att);
             att.run(reinterpret_cast<float *>(smem4));
         }
