@@ -2,8 +2,8 @@
  * libllama2j_hip.so - C ABI of the MI355X (gfx950) mode of llama2j's per-token forward pass.
  *
  * The library owns every device buffer (weights, activations, KV cache), takes llama2j's own
- * weight formats, and replays the whole token (a chain of hand-written gfx950 kernels) as one captured
- * hipGraph on one GPU.  It is the
+ * weight formats, and runs the whole token as one hand-written gfx950 kernel (plus a one-workgroup
+ * argmax/step kernel), captured in a hipGraph and replayed on one GPU.  It is the
  * seam a `Mode.HIP` plugs into beside the reference's CPU and CUDA modes: each entry point
  * names the reference interface it replaces (paths relative to the reference root,
  * J/ = src/main/java/com/lastbot/llama2j/, K/ = J/kernel/).

@@ -2,7 +2,7 @@
 //
 // Shared device helpers (wavefront reductions, streaming loads, the code/activation dot product,
 // the reference's sigmoid table) and the kernels of the load path (format conversion, the group-int8
-// encoder, seeded tensors).  The forward pass itself is in token_kernel.hpp.
+// encoder, seeded tensors).  The forward pass itself is in phase_kernels.hpp.
 //
 // Reference semantics (paths relative to the reference root, J/ = src/main/java/com/lastbot/llama2j/,
 // K/ = J/kernel/):
