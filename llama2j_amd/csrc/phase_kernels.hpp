@@ -282,7 +282,10 @@ struct MatvecRun {
         }
     }
 
-    // smem: 4*nch float4 (vector), nch floats (chunk sums), 16 floats (reduction)
+    // smem: 4*nch float4 (vector), nch floats (chunk sums), 16 floats (reduction).
+    // COH: results are written through to memory for consumers in the same launch (k_token); a kernel of its
+    // own leaves them to the end-of-kernel write-back.
+    template <bool COH>
     __device__ __forceinline__ void run(float4 *smem4, int token, int pos)
     {
         float4 *xs = smem4;
@@ -349,8 +352,13 @@ struct MatvecRun {
                 }
                 float *p0, *p1;
                 dst_of(item, pos, p0, p1);
-                st_coh(p0, v0);
-                if (p1) st_coh(p1, v1);
+                if (COH) {
+                    st_coh(p0, v0);
+                    if (p1) st_coh(p1, v1);
+                } else {
+                    *p0 = v0;
+                    if (p1) *p1 = v1;
+                }
             }
         }
     }
@@ -364,7 +372,7 @@ __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
     // The weights do not depend on the input vector: the first loads go out before it is staged, so
     // HBM latency overlaps the rmsnorm prologue.
     run.preload();
-    run.run(smem4, d.st->token, d.st->pos);
+    run.template run<false>(smem4, d.st->token, d.st->pos);
 }
 
 // ---- decode attention: workgroup = (head, split); waves share the split's rows; online softmax ----
@@ -449,7 +457,9 @@ struct AttnRun {
         }
     }
 
-    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int
+    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int.  COH as for the matvec phases (the partials of
+    // a split always travel write-through: other workgroups of the same launch read them).
+    template <bool COH>
     __device__ __forceinline__ void run(float *smem)
     {
         float *sm_m = smem;           // nent
@@ -513,7 +523,10 @@ struct AttnRun {
                 }
             }
             if (nact == 1) {
-                if (tid < hs) st_coh(a.out + h * hs + tid, __fdiv_rn(o, L));
+                if (tid < hs) {
+                    if (COH) st_coh(a.out + h * hs + tid, __fdiv_rn(o, L));
+                    else a.out[h * hs + tid] = __fdiv_rn(o, L);
+                }
                 continue;
             }
             // Several splits: partials travel through memory with device-scope relaxed atomics (write-through
@@ -556,7 +569,8 @@ struct AttnRun {
                     }
                     MM = mb;
                 }
-                st_coh(a.out + h * hs + tid, __fdiv_rn(oo, LL));
+                if (COH) st_coh(a.out + h * hs + tid, __fdiv_rn(oo, LL));
+                else a.out[h * hs + tid] = __fdiv_rn(oo, LL);
             }
             if (tid == 0) st_coh(a.counters + h, 0u);
         }
@@ -569,7 +583,7 @@ __global__ void __launch_bounds__(1024) k_attention(const AttnPhase a)
     extern __shared__ float smem[];
     AttnRun<LPR> run(a, a.st->pos);
     run.clear();
-    run.run(smem);
+    run.template run<false>(smem);
 }
 
 // ---- final rmsnorm + fp32 classifier + per-workgroup first-max -----------------------------------
@@ -818,7 +832,7 @@ __device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4,
 {
     MatvecRun<W2_MODE> w2(matvec_phase_of(token_args()->g, K_W2, l));
     handoff(b, 5 * l + 3, w2);
-    w2.run(smem4, token, pos);
+    w2.template run<true>(smem4, token, pos);
 }
 
 template <int WO_MODE>
@@ -826,7 +840,7 @@ __device__ __forceinline__ void token_wo(const GridBar &b, int l, float4 *smem4,
 {
     MatvecRun<WO_MODE> wo(matvec_phase_of(token_args()->g, K_WO, l));
     handoff(b, 5 * l + 1, wo);
-    wo.run(smem4, token, pos);
+    wo.template run<true>(smem4, token, pos);
 }
 
 template <int LPR>
@@ -844,19 +858,19 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             MatvecRun<PH_QKV> qkv(matvec_phase_of(token_args()->g, K_QKV, l));
             if (l == l0) qkv.preload();             // launch order guarantees the input
             else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
-            qkv.run(smem4, token, pos);
+            qkv.template run<true>(smem4, token, pos);
         }
         {
             AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads), pos);
             handoff(b, 5 * l, att);
-            att.run(reinterpret_cast<float *>(smem4));
+            att.template run<true>(reinterpret_cast<float *>(smem4));
         }
         if (wo_row) token_wo<PH_ROW>(b, l, smem4, token, pos);
         else token_wo<PH_RES>(b, l, smem4, token, pos);
         {
             MatvecRun<PH_W13> w13(matvec_phase_of(token_args()->g, K_W13, l));
             handoff(b, 5 * l + 2, w13);
-            w13.run(smem4, token, pos);
+            w13.template run<true>(smem4, token, pos);
         }
         if (w2_row) token_w2<PH_ROW>(b, l, smem4, token, pos);
         else token_w2<PH_RES>(b, l, smem4, token, pos);

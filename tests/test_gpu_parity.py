@@ -24,6 +24,14 @@ QT = [TENSOR.RMS_ATT, TENSOR.WQ, TENSOR.WK, TENSOR.WV, TENSOR.WO, TENSOR.RMS_FFN
       TENSOR.W3, TENSOR.RMS_FINAL]
 
 
+@pytest.fixture(params=["token", "phase"])
+def launch_mode(request, monkeypatch):
+    """The forward pass as one whole-token launch (the default for large models) or as one launch per phase
+    (the default for small ones); the library reads the switch when a transformer is finalized."""
+    monkeypatch.setenv("L2J_FUSE", "1" if request.param == "token" else "0")
+    return request.param
+
+
 def say(*a):
     print(*a, flush=True)
     sys.stdout.flush()
@@ -144,7 +152,7 @@ def test_per_layer_taps_match_oracle(orc, shape):
     np.testing.assert_array_equal(g.read(BUFFER.XB, layer=0), g.read(BUFFER.V, layer=0)[i // hs // kv_mul * hs + i % hs])
 
 
-def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
+def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc, launch_mode):
     m, g = make_pair(orc, TINY[1], seed=31, realistic=True)
     outs = []
     for rep in range(3):
@@ -166,7 +174,7 @@ def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc):
         assert nxt == int(np.argmax(outs[0][p]))
 
 
-def test_split_attention_in_both_launch_modes(orc):
+def test_split_attention_in_both_launch_modes(orc, launch_mode):
     # contexts long enough that attention is split over several workgroups (whole-token launch: beyond 64
     # positions; kernel-by-kernel: beyond 32) and folded by the last arriver; multiquery, head 16
     shape = (64, 96, 2, 4, 2, 40, 200, 1)
@@ -185,17 +193,23 @@ def test_split_attention_in_both_launch_modes(orc):
         assert rel_err(got, fused[pos]) < 1e-5, pos
 
 
-def test_kernel_timing_entry_point(orc):
+def test_kernel_timing_entry_point(orc, launch_mode):
     # every kernel class launches and reports a time, deep enough in the context that attention is split;
     # the measurement leaves the context usable (same tokens before and after)
     shape = (64, 96, 2, 4, 2, 40, 200, 1)
     m, g = make_pair(orc, shape, seed=34, realistic=True)
     prompt = orc.synth_prompt(34, 4, shape[5])
     before, _ = g.decode_greedy(prompt, 160)
-    for k in range(7):
+    for k in range(6):
         us, nbytes = g.time_kernel(k, 150, rounds=2)
         assert us > 0.0 and nbytes > 0, k
-    assert g.time_kernel(l2j.KERNEL.TOKEN, 150, rounds=1)[1] == g.bytes_per_token(150)
+    if launch_mode == "token":
+        us, nbytes = g.time_kernel(l2j.KERNEL.TOKEN, 150, rounds=2)
+        assert us > 0.0 and nbytes == g.bytes_per_token(150)
+    else:  # no whole-token kernel in this mode
+        with pytest.raises(l2j.L2JError) as e:
+            g.time_kernel(l2j.KERNEL.TOKEN, 150, rounds=1)
+        assert e.value.code == -3
     g.reset()
     after, _ = g.decode_greedy(prompt, 160)
     np.testing.assert_array_equal(before, after)
@@ -203,7 +217,7 @@ def test_kernel_timing_entry_point(orc):
     np.testing.assert_array_equal(after, want)
 
 
-def test_argmax_first_max_tie_rule(orc):
+def test_argmax_first_max_tie_rule(orc, launch_mode):
     # identical classifier rows give exactly equal logits: the lowest index must win (J/Sampler.java:51)
     shape = (64, 256, 1, 4, 4, 1000, 4, 0)
     m, g0 = make_pair(orc, shape, seed=41)
@@ -227,7 +241,7 @@ def test_argmax_first_max_tie_rule(orc):
 
 # ------------------------------------------------------------------ token loop
 
-def test_decode_greedy_loop_semantics(orc):
+def test_decode_greedy_loop_semantics(orc, launch_mode):
     m, g = make_pair(orc, TINY[0], seed=51, realistic=True)
     prompt = np.array([5, 9, 11], np.int32)
     want, _, _ = m.generate_greedy(prompt, 10)
@@ -392,12 +406,12 @@ def run_config(orc, name, shape, seed, n_prompt, n_steps, n_logit_steps):
     m.close(); g.close()
 
 
-def test_config1_stories15m_shape(orc):
+def test_config1_stories15m_shape(orc, launch_mode):
     # dim 288: quantization groups straddle rows and layers, head 48; 8 prompt ids + 248 greedy
     run_config(orc, "15M", (288, 768, 6, 6, 6, 32000, 256, 1), seed=101, n_prompt=8, n_steps=256, n_logit_steps=256)
 
 
-def test_config2_stories110m_shape(orc):
+def test_config2_stories110m_shape(orc, launch_mode):
     run_config(orc, "110M", (768, 2048, 12, 12, 12, 32000, 1024, 1), seed=102, n_prompt=16, n_steps=16 + 128,
                n_logit_steps=16 + 128)
 
