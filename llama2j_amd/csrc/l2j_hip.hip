@@ -179,7 +179,7 @@ static_assert(K_QKV == L2J_K_QKV && K_ATT == L2J_K_ATTENTION && K_WO == L2J_K_WO
               K_CLS == L2J_K_CLASSIFIER, "kernel classes of the C ABI and of the device code must agree");
 
 MatvecPhase matvec_phase(const l2j_ctx *c, int kclass, int l) { return matvec_phase_of(c->geom, kclass, l); }
-AttnPhase attn_phase(const l2j_ctx *c, int l) { return attn_phase_of(c->geom, l, c->attn_rows, c->attn_threads); }
+AttnPhase attn_phase(const l2j_ctx *c, int l) { return attn_phase_of(c->geom, l, c->attn_rows, c->attn_threads, c->attn_nsplit); }
 ClsPhase cls_phase(const l2j_ctx *c) { return cls_phase_of(c->geom, c->pk_grid); }
 
 void build_geom(l2j_ctx *c)
@@ -220,6 +220,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.g = c->geom;
     a.l0 = l0; a.l1 = l1; a.with_cls = l1 == c->cfg.n_layers;
     a.attn_rows = c->fused_attn_rows;
+    a.attn_splits = std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
     a.maxspin = 20000;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);

@@ -388,6 +388,7 @@ struct AttnPhase {
     int n_heads, kv_mul, head_size, kv_dim, nsplit, rows_per_split;
     float sqrt_hs;
     int threads;           // workgroup size
+    int max_splits;        // at most this many splits per head (<= nsplit, the stride of `part`)
 };
 
 constexpr int kAU = 2;  // cache rows in flight per lane group (K and V each)
@@ -414,7 +415,7 @@ struct AttnRun {
         nent = W * RPW;
         len = pos + 1;
         int nsplit = (len + a.rows_per_split - 1) / a.rows_per_split;  // short contexts: fewer, fuller splits
-        if (nsplit > a.nsplit) nsplit = a.nsplit;
+        if (nsplit > a.max_splits) nsplit = a.max_splits;
         chunk = (len + nsplit - 1) / nsplit;
         nact = (len + chunk - 1) / chunk;
         j = lane % LPR;
@@ -772,7 +773,7 @@ __host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, i
 }
 
 template <class G>
-__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split, int threads)
+__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split, int threads, int max_splits)
 {
     const long kvoff = (long)l * g.seq_len * g.kv_dim;
     AttnPhase t{};
@@ -780,6 +781,7 @@ __host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_p
     t.part = g.attn_part; t.counters = g.attn_counters; t.st = g.st;
     t.n_heads = g.n_heads; t.kv_mul = g.kv_mul; t.head_size = g.head_size; t.kv_dim = g.kv_dim;
     t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split; t.threads = threads;
+    t.max_splits = max_splits < g.attn_nsplit ? max_splits : g.attn_nsplit;
     t.sqrt_hs = g.sqrt_hs;  // (float) Math.sqrt(head_size), K/AttentionLoop.java:48
     return t;
 }
@@ -800,7 +802,8 @@ __host__ __device__ inline bool row_mode(int n) { return n / 16 > 64 * kTU; }
 struct TokenArgs {
     TokenGeom g;
     int l0, l1, with_cls;   // layers [l0, l1), then the classifier when with_cls
-    int attn_rows;          // cache rows per attention split in this kernel
+    int attn_rows;          // cache rows per attention split in this kernel (more when the splits run out)
+    int attn_splits;        // at most this many splits per head: one (head, split) item per workgroup
     int maxspin;
 };
 
@@ -861,7 +864,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             qkv.template run<true>(smem4, token, pos);
         }
         {
-            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads), pos);
+            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads, token_args()->attn_splits), pos);
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
