@@ -10,8 +10,9 @@
  *
  * Conventions: plain C, no exceptions cross the boundary, 0 = success and negative = error
  * (the text is in l2j_last_error(), thread local).  Entry points that run the forward pass are
- * not re-entrant per context; uploads are thread safe (the reference uploads from ten threads,
- * J/TransformerWeights.java:52,204).  There is no CPU fallback: without a GPU l2j_create fails.
+ * not re-entrant per context, and forwards of different contexts of one process take turns (the
+ * whole-token kernel occupies every compute unit); uploads are thread safe (the reference uploads from
+ * ten threads, J/TransformerWeights.java:52,204).  There is no CPU fallback: without a GPU l2j_create fails.
  */
 #ifndef LLAMA2J_HIP_H
 #define LLAMA2J_HIP_H

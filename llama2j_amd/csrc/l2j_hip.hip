@@ -322,6 +322,10 @@ hipError_t launch_one_token(l2j_ctx *c)
     return c->graph_exec ? hipGraphLaunch(c->graph_exec, c->stream) : launch_token(c, c->stream, false);
 }
 
+// The whole-token kernel needs every compute unit of the device for itself, so forwards of different contexts
+// of this process take turns (each entry point synchronizes before it returns).
+std::mutex g_forward_mu;
+
 // After a synchronize: a workgroup whose bounded wait at a grid barrier ran out has set the flag.
 int check_barrier_error(l2j_ctx *c)
 {
@@ -330,7 +334,8 @@ int check_barrier_error(l2j_ctx *c)
     if (*c->h_fault == 0) return L2J_OK;
     *c->h_fault = 0;
     HIPCHK(hipMemcpy(c->fault, c->h_fault, sizeof(int), hipMemcpyHostToDevice));
-    return fail(L2J_E_HIP, "a grid barrier of the layer kernel timed out (its workgroups were not all resident)");
+    HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));  // leave the context usable
+    return fail(L2J_E_HIP, "a grid barrier of the whole-token kernel timed out (its workgroups were not all resident)");
 }
 
 int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
@@ -794,6 +799,7 @@ int l2j_sync(l2j_ctx *c)
 
 int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 {
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     int rc = check_forward_args(c, token, pos);
     if (rc) return rc;
     if ((rc = set_state(c, token, pos, 0))) return rc;
@@ -805,6 +811,7 @@ int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 
 int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
 {
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     if (!next) return fail(L2J_E_ARG, "null argument");
     int rc = check_forward_args(c, token, pos);
     if (rc) return rc;
@@ -818,6 +825,7 @@ int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
 
 int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 {
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     int rc = check_forward_args(c, token, pos);
     if (rc) return rc;
     const uint64_t L = c->cfg.n_layers;
@@ -838,6 +846,7 @@ int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, int32_t *out_tokens, int32_t *n_out,
                       double *seconds)
 {
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     if (!c || !out_tokens || !n_out || (n_prompt > 0 && !prompt) || n_prompt < 0) return fail(L2J_E_ARG, "bad argument");
     if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
     HIPCHK(hipSetDevice(c->cfg.device));
@@ -972,6 +981,7 @@ uint64_t l2j_bytes_per_token(const l2j_config *g, int32_t pos)
 
 int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double *mean_us, uint64_t *bytes)
 {
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     if (!c || !mean_us) return fail(L2J_E_ARG, "null argument");
     if (kclass < 0 || kclass >= L2J_K_COUNT || rounds <= 0) return fail(L2J_E_ARG, "bad kernel class or rounds");
     int rc = check_forward_args(c, 1, pos);

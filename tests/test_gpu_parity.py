@@ -217,6 +217,32 @@ def test_kernel_timing_entry_point(orc, launch_mode):
     np.testing.assert_array_equal(after, want)
 
 
+def test_two_contexts_decode_from_two_threads(orc, launch_mode):
+    # forwards of different contexts take turns on the device: concurrent decodes give the sequential answers
+    import threading
+    shape = (64, 96, 2, 4, 2, 40, 96, 1)
+    pairs = [make_pair(orc, shape, seed=40 + i, realistic=True) for i in range(2)]
+    prompts = [orc.synth_prompt(40 + i, 3, shape[5]) for i in range(2)]
+    want = [g.decode_greedy(p, 90)[0].copy() for (m, g), p in zip(pairs, prompts)]
+    for m, g in pairs:
+        g.reset()
+    got = [None, None]
+
+    def work(i):
+        for rep in range(3):
+            pairs[i][1].reset()
+            got[i] = pairs[i][1].decode_greedy(prompts[i], 90)[0].copy()
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    for i in range(2):
+        np.testing.assert_array_equal(got[i], want[i])
+        np.testing.assert_array_equal(got[i], pairs[i][0].generate_greedy(prompts[i], 90)[0])
+
+
 def test_argmax_first_max_tie_rule(orc, launch_mode):
     # identical classifier rows give exactly equal logits: the lowest index must win (J/Sampler.java:51)
     shape = (64, 256, 1, 4, 4, 1000, 4, 0)
