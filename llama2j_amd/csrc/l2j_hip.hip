@@ -99,6 +99,7 @@ struct l2j_ctx {
     int *fault = nullptr;         // set by a kernel whose barrier wait ran out
     int *h_fault = nullptr;       // pinned
     int fused_attn_rows = 64;
+    int barrier_spins = 20000;    // polls of a grid barrier before it gives up (each poll is a memory round trip, >= 1 us)
     TokenGeom geom{};             // set by l2j_finalize
 
     hipGraph_t graph = nullptr;
@@ -221,7 +222,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.l0 = l0; a.l1 = l1; a.with_cls = l1 == c->cfg.n_layers;
     a.attn_rows = c->fused_attn_rows;
     a.attn_splits = std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
-    a.maxspin = 20000;
+    a.maxspin = c->barrier_spins;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
     const int lpr = attn_lpr(c);
@@ -723,6 +724,7 @@ int l2j_finalize(l2j_ctx *c)
         c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
         c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
         c->fused_attn_rows = std::max(1, env_int("L2J_FUSED_ATTN_ROWS", 64));
+        c->barrier_spins = std::max(0, env_int("L2J_BARRIER_SPINS", 20000));
         const size_t need = std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c));
         if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
         if (need > 64 * 1024) {

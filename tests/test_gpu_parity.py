@@ -217,6 +217,29 @@ def test_kernel_timing_entry_point(orc, launch_mode):
     np.testing.assert_array_equal(after, want)
 
 
+def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
+    # a spin limit of zero makes the bounded waits of the whole-token kernel give up at once: every kernel still
+    # runs to its end, the call reports the failure, and a context with the normal limit is unaffected
+    shape = (64, 96, 2, 4, 2, 40, 32, 1)
+    monkeypatch.setenv("L2J_FUSE", "1")
+    monkeypatch.setenv("L2J_BARRIER_SPINS", "0")
+    m, bad = make_pair(orc, shape, seed=50)
+    failures = 0
+    for pos in range(8):
+        try:
+            bad.forward(3, pos)
+        except l2j.L2JError as e:
+            assert e.code == -4 and "barrier" in str(e)
+            failures += 1
+    assert failures > 0
+    monkeypatch.setenv("L2J_BARRIER_SPINS", "20000")
+    m2, good = make_pair(orc, shape, seed=50)
+    for pos in range(8):
+        assert rel_err(good.forward(3, pos), m2.forward(3, pos)) < 1e-4
+    # the context whose waits expired works again once the stale state is gone
+    bad.close()
+
+
 def test_two_contexts_decode_from_two_threads(orc, launch_mode):
     # forwards of different contexts take turns on the device: concurrent decodes give the sequential answers
     import threading
