@@ -99,6 +99,9 @@ struct l2j_ctx {
     int *fault = nullptr;         // set by a kernel whose barrier wait ran out
     int *h_fault = nullptr;       // pinned
     int fused_attn_rows = 64;
+    bool by_value = false;        // k_token hands activations over by value (no grid barriers)
+    float *knew = nullptr, *vnew = nullptr;  // this token's k and v rows per layer
+    uint64_t skv = 0;
     int barrier_spins = 20000;    // polls of a grid barrier before it gives up (each poll is a memory round trip, >= 1 us)
     TokenGeom geom{};             // set by l2j_finalize
 
@@ -196,6 +199,7 @@ void build_geom(l2j_ctx *c)
     t.x = c->x; t.xb = c->xb; t.hb = c->hb; t.q = c->q; t.kcache = c->kcache; t.vcache = c->vcache; t.logits = c->logits;
     t.wq = qmat(c, L2J_WQ, 0); t.wk = qmat(c, L2J_WK, 0); t.wv = qmat(c, L2J_WV, 0); t.wo = qmat(c, L2J_WO, 0);
     t.w1 = qmat(c, L2J_W1, 0); t.w2 = qmat(c, L2J_W2, 0); t.w3 = qmat(c, L2J_W3, 0);
+    t.knew = c->knew; t.vnew = c->vnew; t.skv = (long)c->skv;
     t.attn_part = c->attn_part; t.attn_counters = c->counters; t.attn_nsplit = c->attn_nsplit;
     t.sqrt_hs = sqrtf((float)c->head_size);
     t.st = c->st; t.cls_val = c->cls_val; t.cls_idx = c->cls_idx; t.prompt = c->prompt; t.out_tokens = c->out_tokens;
@@ -208,10 +212,22 @@ bool geom_complete(const TokenGeom &t)
     const void *ptrs[] = {t.emb, t.rmsw, t.silu, t.wcls, t.rope, t.x, t.xb, t.hb, t.q, t.kcache, t.vcache, t.logits,
                           t.wq.codes, t.wq.gs, t.wk.codes, t.wk.gs, t.wv.codes, t.wv.gs, t.wo.codes, t.wo.gs,
                           t.w1.codes, t.w1.gs, t.w2.codes, t.w2.gs, t.w3.codes, t.w3.gs,
-                          t.attn_part, t.attn_counters, t.st, t.cls_val, t.cls_idx, t.prompt, t.out_tokens, t.bar_ctr, t.fault};
+                          t.knew, t.vnew, t.attn_part, t.attn_counters, t.st, t.cls_val, t.cls_idx, t.prompt, t.out_tokens, t.bar_ctr, t.fault};
     for (const void *p : ptrs)
         if (!p) return false;
     return true;
+}
+
+// Marks every activation vector of a token unwritten (before a k_token that hands over by value).
+hipError_t launch_fill_unset(const l2j_ctx *c, hipStream_t s)
+{
+    const uint64_t L = c->cfg.n_layers;
+    FillArgs f{};
+    float *p[6] = {c->x, c->xb, c->hb, c->q, c->knew, c->vnew};
+    const uint64_t n[6] = {(2 * L + 1) * c->sd, L * c->sd, L * c->sh, L * c->sd, L * c->skv, L * c->skv};
+    for (int i = 0; i < 6; i++) { f.p[i] = p[i]; f.n[i] = (long)n[i]; }
+    hipLaunchKernelGGL(k_fill_unset, dim3(c->n_cu), dim3(1024), 0, s, f);
+    return hipGetLastError();
 }
 
 // Layers [l0, l1) (and the classifier after the last layer) in one launch of k_token.
@@ -223,6 +239,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.attn_rows = c->fused_attn_rows;
     a.attn_splits = std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
     a.maxspin = c->barrier_spins;
+    a.by_value = c->by_value ? 1 : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
     const int lpr = attn_lpr(c);
@@ -288,6 +305,7 @@ hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
     const l2j_config &g = c->cfg;
     hipError_t e;
     if (c->fused && !taps) {
+        if (c->by_value && (e = launch_fill_unset(c, s)) != hipSuccess) return e;
         for (int l = 0; l < g.n_layers; l += c->layers_per_launch)
             if ((e = launch_layers(c, l, std::min(g.n_layers, l + c->layers_per_launch), s)) != hipSuccess) return e;
         hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, s, cls_phase(c));
@@ -336,7 +354,7 @@ int check_barrier_error(l2j_ctx *c)
     *c->h_fault = 0;
     HIPCHK(hipMemcpy(c->fault, c->h_fault, sizeof(int), hipMemcpyHostToDevice));
     HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));  // leave the context usable
-    return fail(L2J_E_HIP, "a grid barrier of the whole-token kernel timed out (its workgroups were not all resident)");
+    return fail(L2J_E_HIP, "a bounded wait of the whole-token kernel ran out (barrier or input vector; its workgroups were not all resident)");
 }
 
 int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
@@ -476,13 +494,16 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     TRY(dev_alloc(&c->vcache, kvn));
     TRY(dev_alloc(&c->rope, (uint64_t)cfg->seq_len * (c->head_size / 2)));
     TRY(dev_alloc(&c->silu, kSiluTable));
-    TRY(dev_alloc(&c->counters, cfg->n_heads + 1));
+    TRY(dev_alloc(&c->counters, NL * cfg->n_heads + 1));
+    c->skv = ((uint64_t)c->kv_dim + 63) / 64 * 64;
+    TRY(dev_alloc(&c->knew, NL * c->skv));
+    TRY(dev_alloc(&c->vnew, NL * c->skv));
     TRY(dev_alloc(&c->st, 1));
     TRY(dev_alloc(&c->prompt, cfg->seq_len));
     TRY(dev_alloc(&c->out_tokens, cfg->seq_len));
     TRYHIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_st), sizeof(DevState), hipHostMallocDefault));
     TRYHIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_tokens), (size_t)cfg->seq_len * sizeof(int), hipHostMallocDefault));
-    TRYHIP(hipMemset(c->counters, 0, (cfg->n_heads + 1) * sizeof(unsigned)));
+    TRYHIP(hipMemset(c->counters, 0, (NL * cfg->n_heads + 1) * sizeof(unsigned)));
     TRYHIP(hipMemset(c->prompt, 0, (size_t)cfg->seq_len * sizeof(int)));
     TRYHIP(hipMemset(c->out_tokens, 0, (size_t)cfg->seq_len * sizeof(int)));
     TRYHIP(hipMemset(c->st, 0, sizeof(DevState)));
@@ -516,6 +537,8 @@ void l2j_destroy(l2j_ctx *c)
     (void)hipFree(c->attn_part);
     (void)hipFree(c->rmsw);
     (void)hipFree(c->counters);
+    (void)hipFree(c->knew);
+    (void)hipFree(c->vnew);
     (void)hipFree(c->st);
     (void)hipFree(c->prompt);
     (void)hipFree(c->out_tokens);
@@ -737,7 +760,7 @@ int l2j_finalize(l2j_ctx *c)
         int rc2;
         if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
         if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
-        if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
+        if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_layers * c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
         c->nbar = 5 * c->cfg.n_layers;
         if ((rc2 = dev_alloc(&c->bar_ctr, (uint64_t)c->nbar * kBarStride))) return rc2;
         if ((rc2 = dev_alloc(&c->fault, 1))) return rc2;
@@ -759,6 +782,8 @@ int l2j_finalize(l2j_ctx *c)
             HIPCHK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kl, c->pk_threads, layer_smem(c)));
             if (per_cu < 1 || c->pk_grid > per_cu * c->n_cu) c->fused = false;
         }
+        c->by_value = c->fused && c->layers_per_launch == c->cfg.n_layers && env_int("L2J_BY_VALUE", 1) != 0 &&
+                      std::max(c->cfg.dim, c->cfg.hidden_dim) <= 4 * kPollWords * c->pk_threads;
         build_geom(c);
         if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
     }
@@ -1011,6 +1036,10 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
         double total = 0.0;
         for (int r = 0; r < rounds; r++) {
             if ((rc = set_state(c, 1, pos, 0))) return rc;
+            if (c->by_value) {
+                hipError_t ef = launch_fill_unset(c, c->stream);
+                if (ef != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(ef));
+            }
             hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33], c->events[34]);
             if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
             hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));

@@ -34,6 +34,58 @@ __device__ __forceinline__ int ld_coh(const int *p) { return __hip_atomic_load(p
 __device__ __forceinline__ void st_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coh(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// ---- hand-over by value ---------------------------------------------------------------------------------
+// Instead of a barrier, a consumer can wait for the data itself: before a token every activation vector is
+// filled with kUnset (a NaN bit pattern no computation produces), producers overwrite it with write-through
+// stores, and consumers re-read their part of the vector with device-coherent 16-byte loads until no kUnset
+// word is left.  The wait is bounded like the barrier's.
+constexpr unsigned kUnset = 0x7FC0DEADu;
+
+__device__ __forceinline__ float4 ld_coh16(const float *p)
+{
+    float4 v;
+    // (the wait is part of the statement: the compiler does not count this load)
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+
+__device__ __forceinline__ bool all_set(const float4 &v)
+{
+    return __float_as_uint(v.x) != kUnset && __float_as_uint(v.y) != kUnset && __float_as_uint(v.z) != kUnset &&
+           __float_as_uint(v.w) != kUnset;
+}
+
+struct Poll {
+    int on;       // 1: wait for the data itself (k_token without barriers); 0: plain loads
+    int maxspin;
+    int *fault;
+};
+
+// The 16-byte word at p once its producers have written all of it.
+__device__ __forceinline__ float4 wait_word(const float *p, const Poll &pl)
+{
+    float4 v = ld_coh16(p);
+    int spins = 0;
+    while (!all_set(v)) {
+        if (++spins > pl.maxspin || ((spins & 63) == 0 && ld_coh(pl.fault) != 0)) { st_coh(pl.fault, 1); break; }
+        __builtin_amdgcn_s_sleep(4);
+        v = ld_coh16(p);
+    }
+    return v;
+}
+
+__device__ __forceinline__ float wait_float(const float *p, const Poll &pl)
+{
+    float v = ld_coh(p);
+    int spins = 0;
+    while (__float_as_uint(v) == kUnset) {
+        if (++spins > pl.maxspin || ((spins & 63) == 0 && ld_coh(pl.fault) != 0)) { st_coh(pl.fault, 1); break; }
+        __builtin_amdgcn_s_sleep(4);
+        v = ld_coh(p);
+    }
+    return v;
+}
+
 // ---- grid barrier ------------------------------------------------------------------------------------
 // Two levels of relaxed device-scope counters: a workgroup bumps the counter of its group (blockIdx % ngroups),
 // the last of a group bumps the top counter, everybody polls the top counter.  Every barrier instance of a
@@ -107,6 +159,8 @@ struct MatvecPhase {
     const DevState *st;
     int head_size, kv_dim, exact_silu;
     int threads;    // workgroup size (a kernel argument: reading it from the dispatch costs a vector load per phase)
+    Poll poll;      // how the input vector and the residual are read
+    float *knew, *vnew;  // QKV with poll.on: this token's k and v rows once more, where attention waits for them
 };
 
 // ---- activation vector -> LDS ------------------------------------------------------------------
@@ -165,6 +219,55 @@ __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int 
     __syncthreads();
 }
 
+// The same with the vector read word by word as soon as its producers have written it (hand-over by value).
+// Thread t takes the 16-byte words t, t+T, ...; the four lanes of a quad hold the four words of a chunk.
+// (Letting a few waves stage the vector and request their weights afterwards, so that the vector is not queued
+// behind them, was slower: 1.96 against 1.76 ms per 7B token.)
+constexpr int kPollWords = 4;  // words per thread: n <= 16 * T (8 words per thread spill registers)
+
+__device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
+                                                  float *sumx, float *red, int T, const Poll &pl)
+{
+    const int nch = n >> 4, nq = n >> 2, tid = phase_tid();
+    const int S = T;  // n <= 4 * kPollWords * T is checked on the host
+    float4 v[kPollWords], w[kPollWords];
+    float ssq = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kPollWords; k++) {
+        v[k] = w[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int i = tid + k * S;
+        if (i < nq) {
+            if (rmsw) w[k] = reinterpret_cast<const float4 *>(rmsw)[i];
+            v[k] = wait_word(xin + 4 * i, pl);
+        }
+        ssq += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+    }
+    float ss = 1.0f;
+    if (rmsw) {
+        ssq = block_sum(ssq, red, T >> 6);
+        // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
+        ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
+    }
+#pragma unroll
+    for (int k = 0; k < kPollWords; k++) {
+        const int i = tid + k * S;
+        float4 xv = v[k];
+        if (rmsw) {  // out = weight * (ss * x)   (K/WeightNormalizeAndScale.java:73)
+            xv.x = __fmul_rn(w[k].x, __fmul_rn(ss, xv.x));
+            xv.y = __fmul_rn(w[k].y, __fmul_rn(ss, xv.y));
+            xv.z = __fmul_rn(w[k].z, __fmul_rn(ss, xv.z));
+            xv.w = __fmul_rn(w[k].w, __fmul_rn(ss, xv.w));
+        }
+        const float s0 = (xv.x + xv.y) + (xv.z + xv.w);
+        const float s1 = dpp_f<0x55>(s0), s2 = dpp_f<0xAA>(s0), s3 = dpp_f<0xFF>(s0);  // quad lanes 1, 2, 3
+        if (i < nq) {
+            xs[(i & 3) * nch + (i >> 2)] = xv;
+            if ((i & 3) == 0) sumx[i >> 2] = ((s0 + s1) + s2) + s3;
+        }
+    }
+    __syncthreads();
+}
+
 // ---- W8A32 matvec: an item is a pair of rows, one wavefront per item ---------------------------------
 
 constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
@@ -185,6 +288,7 @@ struct MatvecRun {
     unsigned r0 = 0, r1 = 0;                       // position of that code inside its group
     int which = 0, r = 0;
     bool has1 = true, first = false;
+    int wave = 0;
     uint4 w0[kTU], w1[kTU];
     float2 s0[kTU], s1[kTU];
 
@@ -199,7 +303,8 @@ struct MatvecRun {
         nitems = MODE == PH_QKV ? (d.d0 + d.d1 + d.d2) >> 1 : MODE == PH_RES ? (d.d0 + 1) >> 1 : d.d0;
         // Items are dealt block-minor (item -> workgroup item % G), so every compute unit gets the same
         // number of rows even when the rows do not fill all waves.
-        item = __builtin_amdgcn_readfirstlane(tid >> 6) * G + blockIdx.x;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        item = wave * G + blockIdx.x;
     }
 
     __device__ __forceinline__ void resolve(int it)
@@ -293,14 +398,23 @@ struct MatvecRun {
         float *red = sumx + nch;
         const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
         const float *res = d.res_emb ? emb_row : d.res_src;
-        stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
+        if (d.poll.on && !d.from_emb) {
+            stage_vector_poll(d.xin, n, d.rmsw, xs, sumx, red, d.threads, d.poll);
+        } else {
+            stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
+        }
 
         for (; item < nitems; item += W * G) {
             if (!first) resolve(item);
             float resv0 = 0.0f, resv1 = 0.0f;
             if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {  // in flight while the row streams
-                resv0 = res[r];
-                if (MODE == PH_RES && has1) resv1 = res[r + 1];
+                if (d.poll.on && !d.res_emb) {  // a line of the vector may have been cached while it was half written
+                    resv0 = wait_float(res + r, d.poll);
+                    if (MODE == PH_RES && has1) resv1 = wait_float(res + r + 1, d.poll);
+                } else {
+                    resv0 = res[r];
+                    if (MODE == PH_RES && has1) resv1 = res[r + 1];
+                }
             }
             float acc0 = 0.0f, acc1 = 0.0f;
             for (int base = 0; base < nch; base += kStep) {
@@ -355,6 +469,11 @@ struct MatvecRun {
                 if (COH) {
                     st_coh(p0, v0);
                     if (p1) st_coh(p1, v1);
+                    if (MODE == PH_QKV && d.knew && which > 0) {  // where attention waits for this token's rows
+                        float *p = (which == 1 ? d.knew : d.vnew) + r;
+                        st_coh(p, v0);
+                        st_coh(p + 1, v1);
+                    }
                 } else {
                     *p0 = v0;
                     if (p1) *p1 = v1;
@@ -389,6 +508,8 @@ struct AttnPhase {
     float sqrt_hs;
     int threads;           // workgroup size
     int max_splits;        // at most this many splits per head (<= nsplit, the stride of `part`)
+    Poll poll;             // how q and this token's k, v rows are read
+    const float *knew, *vnew;  // with poll.on: this token's k and v rows (kv_dim each)
 };
 
 constexpr int kAU = 2;  // cache rows in flight per lane group (K and V each)
@@ -433,8 +554,13 @@ struct AttnRun {
             const int t = tb + u * nent;
             const bool want = part == 0 || (part == 1 ? t < len - 1 : t == len - 1);
             if (t < t1 && active && want) {
-                k4[u] = load_stream(reinterpret_cast<const float4 *>(a.kc + (long)t * a.kv_dim + col));
-                v4[u] = load_stream(reinterpret_cast<const float4 *>(a.vc + (long)t * a.kv_dim + col));
+                if (a.poll.on && t == len - 1) {  // written in this launch: wait for it where its producer parks it
+                    k4[u] = wait_word(a.knew + col, a.poll);
+                    v4[u] = wait_word(a.vnew + col, a.poll);
+                } else {
+                    k4[u] = load_stream(reinterpret_cast<const float4 *>(a.kc + (long)t * a.kv_dim + col));
+                    v4[u] = load_stream(reinterpret_cast<const float4 *>(a.vc + (long)t * a.kv_dim + col));
+                }
             }
         }
     }
@@ -472,7 +598,7 @@ struct AttnRun {
             const int h = it % a.n_heads, s = it / a.n_heads;
             const int t0 = s * chunk, t1 = min(len, t0 + chunk);
             float4 q4 = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (active) q4 = *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
+            if (active) q4 = a.poll.on ? wait_word(a.q + h * hs + 4 * j, a.poll) : *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
             float m = -3.402823466e+38f, l = 0.0f;
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
             for (int tb = t0 + slot; tb < t1; tb += nent * kAU) {
@@ -604,6 +730,7 @@ struct ClsPhase {
     unsigned *bar_ctr;   // grid barrier counters of the token, zeroed for the next one
     int nbar;
     int threads;         // workgroup size of the classifier
+    Poll poll;           // how the input vector is read
 };
 
 constexpr int kCU = 8;
@@ -656,7 +783,11 @@ struct ClsRun {
         float *red = sumx + nch;
         float *bval = red + 16;
         int *bidx = reinterpret_cast<int *>(red + 32);
-        stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
+        if (a.poll.on) {
+            stage_vector_poll(a.xin, n, a.rmsw, xs, sumx, red, a.threads, a.poll);
+        } else {
+            stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
+        }
 
         float best_v = -__builtin_inff();
         int best_i = 0x7fffffff;
@@ -714,8 +845,10 @@ struct TokenGeom {
     const float2 *rope;
     float *x, *xb, *hb, *q, *kcache, *vcache, *logits;
     QMat wq, wk, wv, wo, w1, w2, w3;  // off = 0: layer 0
-    float *attn_part;
-    unsigned *attn_counters;
+    float *knew, *vnew;  // this token's k and v rows per layer (stride skv), for the hand-over by value
+    long skv;
+    float *attn_part;    // per layer: (n_heads, attn_nsplit, head_size + 2)
+    unsigned *attn_counters;  // per layer: n_heads
     int attn_nsplit;
     float sqrt_hs;
     DevState *st;
@@ -778,7 +911,7 @@ __host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_p
     const long kvoff = (long)l * g.seq_len * g.kv_dim;
     AttnPhase t{};
     t.q = g.q + l * g.sd; t.kc = g.kcache + kvoff; t.vc = g.vcache + kvoff; t.out = g.xb + l * g.sd;
-    t.part = g.attn_part; t.counters = g.attn_counters; t.st = g.st;
+    t.part = g.attn_part + (long)l * g.n_heads * g.attn_nsplit * (g.head_size + 2); t.counters = g.attn_counters + l * g.n_heads; t.st = g.st;
     t.n_heads = g.n_heads; t.kv_mul = g.kv_mul; t.head_size = g.head_size; t.kv_dim = g.kv_dim;
     t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split; t.threads = threads;
     t.max_splits = max_splits < g.attn_nsplit ? max_splits : g.attn_nsplit;
@@ -805,13 +938,36 @@ struct TokenArgs {
     int attn_rows;          // cache rows per attention split in this kernel (more when the splits run out)
     int attn_splits;        // at most this many splits per head: one (head, split) item per workgroup
     int maxspin;
+    int by_value;           // 1: consumers wait for the data itself (activations pre-filled with kUnset); 0: grid barriers
 };
+
+// Before a token whose phases hand over by value: every activation vector of the token is marked unwritten.
+struct FillArgs {
+    float *p[6];
+    long n[6];  // floats, multiples of 4
+};
+
+__global__ void k_fill_unset(const FillArgs a)
+{
+    const float u = __uint_as_float(kUnset);
+    const float4 u4 = make_float4(u, u, u, u);
+    for (int b = 0; b < 6; b++) {
+        float4 *p = reinterpret_cast<float4 *>(a.p[b]);
+        const long nq = a.n[b] >> 2;
+        for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < nq; i += (long)gridDim.x * blockDim.x) p[i] = u4;
+    }
+}
 
 // Between two phases: every wave waits for its own stores to be acknowledged, the workgroup arrives at the
 // barrier, requests the first weights of the next phase, and only then waits for the other workgroups.
 template <class Next>
 __device__ __forceinline__ void handoff(const GridBar &b, int inst, Next &nx)
 {
+    if (b.ngroups == 0) {  // hand-over by value: the next phase waits for its input itself
+        __syncthreads();   // every wave is done with the LDS of the phase that ends here
+        nx.preload();
+        return;
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     bar_arrive(b, inst);
@@ -830,10 +986,31 @@ __device__ __forceinline__ TokenArgsPtr token_args()
     return p;
 }
 
+__device__ __forceinline__ Poll token_poll()
+{
+    Poll p;
+    p.on = token_args()->by_value;
+    p.maxspin = token_args()->maxspin;
+    p.fault = token_args()->g.fault;
+    return p;
+}
+
+// A matvec phase of k_token: the arguments of layer l plus how its input arrives.
+__device__ __forceinline__ MatvecPhase token_phase(int kclass, int l)
+{
+    MatvecPhase d = matvec_phase_of(token_args()->g, kclass, l);
+    d.poll = token_poll();
+    if (d.poll.on && kclass == K_QKV) {
+        d.knew = token_args()->g.knew + l * token_args()->g.skv;
+        d.vnew = token_args()->g.vnew + l * token_args()->g.skv;
+    }
+    return d;
+}
+
 template <int W2_MODE>
 __device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4, int token, int pos)
 {
-    MatvecRun<W2_MODE> w2(matvec_phase_of(token_args()->g, K_W2, l));
+    MatvecRun<W2_MODE> w2(token_phase(K_W2, l));
     handoff(b, 5 * l + 3, w2);
     w2.template run<true>(smem4, token, pos);
 }
@@ -841,7 +1018,7 @@ __device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4,
 template <int WO_MODE>
 __device__ __forceinline__ void token_wo(const GridBar &b, int l, float4 *smem4, int token, int pos)
 {
-    MatvecRun<WO_MODE> wo(matvec_phase_of(token_args()->g, K_WO, l));
+    MatvecRun<WO_MODE> wo(token_phase(K_WO, l));
     handoff(b, 5 * l + 1, wo);
     wo.template run<true>(smem4, token, pos);
 }
@@ -855,23 +1032,27 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     const int l0 = t->l0, l1 = t->l1;
     const bool wo_row = row_mode(t->g.dim), w2_row = row_mode(t->g.hidden);
     GridBar b;
-    b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = kBarGroups; b.maxspin = t->maxspin;
+    b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
     for (int l = l0; l < l1; l++) {
         {
-            MatvecRun<PH_QKV> qkv(matvec_phase_of(token_args()->g, K_QKV, l));
+            MatvecRun<PH_QKV> qkv(token_phase(K_QKV, l));
             if (l == l0) qkv.preload();             // launch order guarantees the input
             else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
             qkv.template run<true>(smem4, token, pos);
         }
         {
-            AttnRun<LPR> att(attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads, token_args()->attn_splits), pos);
+            AttnPhase ap = attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads, token_args()->attn_splits);
+            ap.poll = token_poll();
+            ap.knew = token_args()->g.knew + l * token_args()->g.skv;
+            ap.vnew = token_args()->g.vnew + l * token_args()->g.skv;
+            AttnRun<LPR> att(ap, pos);
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
         if (wo_row) token_wo<PH_ROW>(b, l, smem4, token, pos);
         else token_wo<PH_RES>(b, l, smem4, token, pos);
         {
-            MatvecRun<PH_W13> w13(matvec_phase_of(token_args()->g, K_W13, l));
+            MatvecRun<PH_W13> w13(token_phase(K_W13, l));
             handoff(b, 5 * l + 2, w13);
             w13.template run<true>(smem4, token, pos);
         }
@@ -879,7 +1060,9 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
         else token_w2<PH_RES>(b, l, smem4, token, pos);
     }
     if (token_args()->with_cls) {
-        ClsRun cls(cls_phase_of(token_args()->g, gridDim.x));
+        ClsPhase cp = cls_phase_of(token_args()->g, gridDim.x);
+        cp.poll = token_poll();
+        ClsRun cls(cp);
         handoff(b, 5 * (l1 - 1) + 4, cls);
         cls.run(smem4);
     }
