@@ -230,6 +230,16 @@ hipError_t launch_fill_unset(const l2j_ctx *c, hipStream_t s)
     return hipGetLastError();
 }
 
+// The instantiation of k_token for this context: by lanes per cache row.
+template <typename F>
+auto with_token_kernel(const l2j_ctx *c, F f)
+{
+    const int lpr = attn_lpr(c);
+    if (lpr == 16) return f(k_token<16>);
+    if (lpr == 32) return f(k_token<32>);
+    return f(k_token<64>);
+}
+
 // Layers [l0, l1) (and the classifier after the last layer) in one launch of k_token.
 hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
 {
@@ -242,16 +252,11 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.by_value = c->by_value ? 1 : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
-    const int lpr = attn_lpr(c);
-    if (e0) {
-        if (lpr == 16) hipExtLaunchKernelGGL(k_token<16>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
-        else if (lpr == 32) hipExtLaunchKernelGGL(k_token<32>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
-        else hipExtLaunchKernelGGL(k_token<64>, grid, block, (unsigned)smem, s, e0, e1, 0, a);
-    } else {
-        if (lpr == 16) hipLaunchKernelGGL(k_token<16>, grid, block, smem, s, a);
-        else if (lpr == 32) hipLaunchKernelGGL(k_token<32>, grid, block, smem, s, a);
-        else hipLaunchKernelGGL(k_token<64>, grid, block, smem, s, a);
-    }
+    with_token_kernel(c, [&](auto kernel) {
+        if (e0) hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)smem, s, e0, e1, 0, a);
+        else hipLaunchKernelGGL(kernel, grid, block, smem, s, a);
+        return 0;
+    });
     return hipGetLastError();
 }
 
@@ -741,7 +746,7 @@ int l2j_finalize(l2j_ctx *c)
     {
         const int nmax = std::max(c->cfg.dim, c->cfg.hidden_dim);
         c->pk_threads = std::min(1024, std::max(64, env_int("L2J_THREADS", 1024) / 64 * 64));
-        c->pk_grid = std::max(1, env_int("L2J_GRID", c->n_cu * std::max(1, 1024 / c->pk_threads)));
+        c->pk_grid = std::max(1, env_int("L2J_GRID", c->n_cu));  // one workgroup per compute unit
         c->attn_threads = std::min(1024, std::max(64, env_int("L2J_ATTN_THREADS", 256) / 64 * 64));
         c->attn_rows = std::max(1, env_int("L2J_ATTN_ROWS", 32));
         c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
@@ -775,9 +780,7 @@ int l2j_finalize(l2j_ctx *c)
         c->fused = env_int("L2J_FUSE", layer_floats >= (32ull << 20) ? 1 : 0) != 0;
         c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, env_int("L2J_LAYERS_PER_LAUNCH", c->cfg.n_layers)));
         if (c->fused) {
-            const int lpr = attn_lpr(c);
-            const void *kl = lpr == 16 ? reinterpret_cast<const void *>(k_token<16>)
-                           : lpr == 32 ? reinterpret_cast<const void *>(k_token<32>) : reinterpret_cast<const void *>(k_token<64>);
+            const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
             int per_cu = 0;
             HIPCHK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kl, c->pk_threads, layer_smem(c)));
             if (per_cu < 1 || c->pk_grid > per_cu * c->n_cu) c->fused = false;

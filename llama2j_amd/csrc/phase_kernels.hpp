@@ -223,17 +223,19 @@ __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int 
 // Thread t takes the 16-byte words t, t+T, ...; the four lanes of a quad hold the four words of a chunk.
 // (Letting a few waves stage the vector and request their weights afterwards, so that the vector is not queued
 // behind them, was slower: 1.96 against 1.76 ms per 7B token.)
-constexpr int kPollWords = 4;  // words per thread: n <= 16 * T (8 words per thread spill registers)
+// WORDS = 16-byte words per thread: n <= 4 * WORDS * T (8 words spill registers in k_token)
+constexpr int kPollWords = 4;
 
+template <int WORDS>
 __device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
                                                   float *sumx, float *red, int T, const Poll &pl)
 {
     const int nch = n >> 4, nq = n >> 2, tid = phase_tid();
-    const int S = T;  // n <= 4 * kPollWords * T is checked on the host
-    float4 v[kPollWords], w[kPollWords];
+    const int S = T;  // n <= 4 * WORDS * T is checked on the host
+    float4 v[WORDS], w[WORDS];
     float ssq = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kPollWords; k++) {
+    for (int k = 0; k < WORDS; k++) {
         v[k] = w[k] = make_float4(0.f, 0.f, 0.f, 0.f);
         const int i = tid + k * S;
         if (i < nq) {
@@ -249,7 +251,7 @@ __device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin,
         ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
     }
 #pragma unroll
-    for (int k = 0; k < kPollWords; k++) {
+    for (int k = 0; k < WORDS; k++) {
         const int i = tid + k * S;
         float4 xv = v[k];
         if (rmsw) {  // out = weight * (ss * x)   (K/WeightNormalizeAndScale.java:73)
@@ -272,8 +274,9 @@ __device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin,
 
 constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
 
-// One matvec phase of one workgroup: preload() requests the first item's weights (they do not depend on
-// the input vector), run() stages the vector and streams the items.
+// One matvec phase of one workgroup: preload() requests the first weights (they do not depend on the input
+// vector), run() stages the vector and streams the items.  (Two items in flight per wave with 512-thread
+// workgroups, so that a wave may use 256 registers, was measured: 1.82 against 1.78 ms per 7B token.)
 template <int MODE>
 struct MatvecRun {
     // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
@@ -339,6 +342,8 @@ struct MatvecRun {
         cb1 = mb.codes + f1; gb1 = mb.gs + (f1 >> 8); r1 = (unsigned)(f1 & 255);
     }
 
+    // Requests one step (kTU chunks per lane and sub-row) of the resolved item.
+    // (Members are used by name in every helper: a reference to a member keeps the whole object in memory.)
     __device__ __forceinline__ void issue(int base)
     {
 #pragma unroll
@@ -346,10 +351,21 @@ struct MatvecRun {
             const int c = base + 64 * u + lane, c1 = c + kOff1;
             const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 below)
             const unsigned cc1 = c1 < nch ? c1 : nch - 1;
-            w0[u] = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
-            w1[u] = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc1);
-            s0[u] = gb0[(r0 + 16u * cc) >> 8];
-            s1[u] = gb1[(r1 + 16u * cc1) >> 8];
+            const uint4 a0 = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
+            const uint4 a1 = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc1);
+            const float2 g0 = gb0[(r0 + 16u * cc) >> 8];
+            const float2 g1 = gb1[(r1 + 16u * cc1) >> 8];
+            w0[u] = a0; w1[u] = a1; s0[u] = g0; s1[u] = g1;
+        }
+    }
+
+    // Defined on every path: otherwise the registers stay reserved for the whole layer loop of k_token.
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int u = 0; u < kTU; u++) {
+            w0[u] = w1[u] = make_uint4(0u, 0u, 0u, 0u);
+            s0[u] = s1[u] = make_float2(0.f, 0.f);
         }
     }
 
@@ -359,12 +375,8 @@ struct MatvecRun {
         if (first) {
             resolve(item);
             issue(0);
-        } else {  // defined on every path: otherwise the registers stay reserved for the whole layer loop of k_token
-#pragma unroll
-            for (int u = 0; u < kTU; u++) {
-                w0[u] = w1[u] = make_uint4(0u, 0u, 0u, 0u);
-                s0[u] = s1[u] = make_float2(0.f, 0.f);
-            }
+        } else {
+            zero();
         }
     }
 
@@ -387,6 +399,91 @@ struct MatvecRun {
         }
     }
 
+    // The residual inputs of the resolved item (lane 0; in flight while the rows stream).
+    __device__ __forceinline__ void residual(const float *res, float &resv0, float &resv1)
+    {
+        resv0 = resv1 = 0.0f;
+        if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {
+            if (d.poll.on && !d.res_emb) {  // a line of the vector may have been cached while it was half written
+                resv0 = wait_float(res + r, d.poll);
+                if (MODE == PH_RES && has1) resv1 = wait_float(res + r + 1, d.poll);
+            } else {
+                resv0 = res[r];
+                if (MODE == PH_RES && has1) resv1 = res[r + 1];
+            }
+        }
+    }
+
+    // One step of weights against the staged vector: sum (code*rm + min)*x = rm * sum code*x + min * sum x per chunk.
+    __device__ __forceinline__ void fold(int base, const float4 *xs, const float *sumx, float &acc0, float &acc1)
+    {
+#pragma unroll
+        for (int u = 0; u < kTU; u++) {
+            const uint4 a0 = w0[u], a1 = w1[u];
+            const float2 g0 = s0[u], g1 = s1[u];
+            const int c = base + 64 * u + lane;
+            const bool ok = c < nch;
+            const int cc = ok ? c : nch - 1;
+            const float4 x0 = xs[cc], x1 = xs[nch + cc], x2 = xs[2 * nch + cc], x3 = xs[3 * nch + cc];
+            const float sx = sumx[cc];
+            const float t0 = fmaf(g0.x, dot16(a0, x0, x1, x2, x3), g0.y * sx);
+            acc0 += ok ? t0 : 0.0f;
+            if (MODE == PH_ROW) {
+                const int c1 = c + kOff1;
+                const bool ok1 = c1 < nch;
+                const int cc1 = ok1 ? c1 : nch - 1;
+                const float4 y0 = xs[cc1], y1 = xs[nch + cc1], y2 = xs[2 * nch + cc1], y3 = xs[3 * nch + cc1];
+                const float t1 = fmaf(g1.x, dot16(a1, y0, y1, y2, y3), g1.y * sumx[cc1]);
+                acc1 += ok1 ? t1 : 0.0f;
+            } else {
+                const float t1 = fmaf(g1.x, dot16(a1, x0, x1, x2, x3), g1.y * sx);
+                acc1 += ok ? t1 : 0.0f;
+            }
+        }
+    }
+
+    // Reduces the sums of the resolved item over the wave, applies the phase's epilogue and stores the results.
+    template <bool COH>
+    __device__ __forceinline__ void finish(int it, float acc0, float acc1, float resv0, float resv1, int pos)
+    {
+        acc0 = wave_sum(acc0);
+        acc1 = wave_sum(acc1);
+        if (lane == 0) {
+            float v0, v1 = 0.0f;
+            if (MODE == PH_QKV) {
+                v0 = acc0;
+                v1 = acc1;
+                if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
+                    const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
+                    v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
+                    v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
+                }
+            } else if (MODE == PH_W13) {
+                const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
+                v0 = __fmul_rn(acc0, __fmul_rn(s, acc1));
+            } else if (MODE == PH_RES) {
+                v0 = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
+                v1 = __fadd_rn(resv1, acc1);
+            } else {
+                v0 = __fadd_rn(resv0, acc0 + acc1);
+            }
+            float *p0, *p1;
+            dst_of(it, pos, p0, p1);
+            if (COH) {
+                st_coh(p0, v0);
+                if (p1) st_coh(p1, v1);
+                if (MODE == PH_QKV && d.knew && which > 0) {  // where attention waits for this token's rows
+                    float *p = (which == 1 ? d.knew : d.vnew) + r;
+                    st_coh(p, v0);
+                    st_coh(p + 1, v1);
+                }
+            } else {
+                *p0 = v0;
+                if (p1) *p1 = v1;
+            }
+        }
+    }
+
     // smem: 4*nch float4 (vector), nch floats (chunk sums), 16 floats (reduction).
     // COH: results are written through to memory for consumers in the same launch (k_token); a kernel of its
     // own leaves them to the end-of-kernel write-back.
@@ -399,86 +496,22 @@ struct MatvecRun {
         const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
         const float *res = d.res_emb ? emb_row : d.res_src;
         if (d.poll.on && !d.from_emb) {
-            stage_vector_poll(d.xin, n, d.rmsw, xs, sumx, red, d.threads, d.poll);
+            stage_vector_poll<kPollWords>(d.xin, n, d.rmsw, xs, sumx, red, d.threads, d.poll);
         } else {
             stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
         }
 
         for (; item < nitems; item += W * G) {
             if (!first) resolve(item);
-            float resv0 = 0.0f, resv1 = 0.0f;
-            if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {  // in flight while the row streams
-                if (d.poll.on && !d.res_emb) {  // a line of the vector may have been cached while it was half written
-                    resv0 = wait_float(res + r, d.poll);
-                    if (MODE == PH_RES && has1) resv1 = wait_float(res + r + 1, d.poll);
-                } else {
-                    resv0 = res[r];
-                    if (MODE == PH_RES && has1) resv1 = res[r + 1];
-                }
-            }
+            float resv0, resv1;
+            residual(res, resv0, resv1);
             float acc0 = 0.0f, acc1 = 0.0f;
             for (int base = 0; base < nch; base += kStep) {
                 if (!(first && base == 0)) issue(base);
-#pragma unroll
-                for (int u = 0; u < kTU; u++) {
-                    const int c = base + 64 * u + lane;
-                    const bool ok = c < nch;
-                    const int cc = ok ? c : nch - 1;
-                    const float4 x0 = xs[cc], x1 = xs[nch + cc], x2 = xs[2 * nch + cc], x3 = xs[3 * nch + cc];
-                    const float sx = sumx[cc];
-                    // sum (code*rm + min)*x = rm * sum code*x + min * sum x over the chunk
-                    const float t0 = fmaf(s0[u].x, dot16(w0[u], x0, x1, x2, x3), s0[u].y * sx);
-                    acc0 += ok ? t0 : 0.0f;
-                    if (MODE == PH_ROW) {
-                        const int c1 = c + kOff1;
-                        const bool ok1 = c1 < nch;
-                        const int cc1 = ok1 ? c1 : nch - 1;
-                        const float4 y0 = xs[cc1], y1 = xs[nch + cc1], y2 = xs[2 * nch + cc1], y3 = xs[3 * nch + cc1];
-                        const float t1 = fmaf(s1[u].x, dot16(w1[u], y0, y1, y2, y3), s1[u].y * sumx[cc1]);
-                        acc1 += ok1 ? t1 : 0.0f;
-                    } else {
-                        const float t1 = fmaf(s1[u].x, dot16(w1[u], x0, x1, x2, x3), s1[u].y * sx);
-                        acc1 += ok ? t1 : 0.0f;
-                    }
-                }
+                fold(base, xs, sumx, acc0, acc1);
             }
             first = false;
-            acc0 = wave_sum(acc0);
-            acc1 = wave_sum(acc1);
-            if (lane == 0) {
-                float v0, v1 = 0.0f;
-                if (MODE == PH_QKV) {
-                    v0 = acc0;
-                    v1 = acc1;
-                    if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
-                        const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
-                        v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
-                        v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
-                    }
-                } else if (MODE == PH_W13) {
-                    const float s = silu_sigma(d.silu, acc0, d.exact_silu);  // K/Silu.java:72-74
-                    v0 = __fmul_rn(acc0, __fmul_rn(s, acc1));
-                } else if (MODE == PH_RES) {
-                    v0 = __fadd_rn(resv0, acc0);  // K/Accum.java:26-30
-                    v1 = __fadd_rn(resv1, acc1);
-                } else {
-                    v0 = __fadd_rn(resv0, acc0 + acc1);
-                }
-                float *p0, *p1;
-                dst_of(item, pos, p0, p1);
-                if (COH) {
-                    st_coh(p0, v0);
-                    if (p1) st_coh(p1, v1);
-                    if (MODE == PH_QKV && d.knew && which > 0) {  // where attention waits for this token's rows
-                        float *p = (which == 1 ? d.knew : d.vnew) + r;
-                        st_coh(p, v0);
-                        st_coh(p + 1, v1);
-                    }
-                } else {
-                    *p0 = v0;
-                    if (p1) *p1 = v1;
-                }
-            }
+            finish<COH>(item, acc0, acc1, resv0, resv1, pos);
         }
     }
 };
@@ -784,7 +817,7 @@ struct ClsRun {
         float *bval = red + 16;
         int *bidx = reinterpret_cast<int *>(red + 32);
         if (a.poll.on) {
-            stage_vector_poll(a.xin, n, a.rmsw, xs, sumx, red, a.threads, a.poll);
+            stage_vector_poll<kPollWords>(a.xin, n, a.rmsw, xs, sumx, red, a.threads, a.poll);
         } else {
             stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
         }
