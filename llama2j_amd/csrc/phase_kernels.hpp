@@ -6,10 +6,9 @@
 //   PH_RES/ROW  W2 matvec + residual
 // and once per token k_classifier (final rmsnorm + fp32 classifier + per-workgroup first-max) and k_finish
 // (fold the maxima, step the token loop state).  k_token runs all phases of a range of layers (by default
-// the whole token, classifier included) in one launch, one 1024-thread workgroup per compute unit, with grid
-// barriers between the phases; each phase also exists as a kernel of its own (k_matvec<MODE>, k_attention,
-// k_classifier) for per-layer taps and per-phase timing.  The launches of a token are captured once in a
-// hipGraph and replayed.
+// the whole token, classifier included) in one launch, one 1024-thread workgroup per compute unit; each phase
+// also exists as a kernel of its own (k_matvec<MODE>, k_attention, k_classifier) for per-layer taps, per-phase
+// timing and small models.  The launches of a token are captured once in a hipGraph and replayed.
 //
 // Every phase is HBM-bandwidth bound (batch-1 GEMV: no reuse, so no MFMA): int8 codes are streamed
 // with 16-byte nontemporal loads, one wavefront per pair of sub-rows, the activation vector is staged
@@ -17,11 +16,13 @@
 // passed by value so that every pointer is a kernel argument (global address space, scalar base + 32-bit
 // lane offset addressing).
 //
-// Activations cross a grid barrier without cache maintenance: producers store them with device-scope
-// relaxed atomics (write-through), every activation vector of a token has a cache-line-aligned address of
-// its own that nothing reads before its producer has finished, and so consumers use plain loads.  The first
-// weights of the next phase are requested between arriving at a barrier and waiting on it, so HBM stays
-// busy while the slowest workgroups finish the phase.
+// Inside k_token a vector passes from one phase to the next without cache maintenance: producers store it
+// with device-scope relaxed atomics (write-through) and every activation vector of a token has a
+// cache-line-aligned address of its own that nothing reads before its producer has finished.  Consumers
+// either wait for the data itself (the vectors are pre-filled with a NaN pattern and re-read with
+// device-coherent loads until it is gone) or, after a grid barrier of relaxed counters, use plain loads.
+// In both cases the first weights of the next phase are requested before the wait, so HBM stays busy while
+// the slowest workgroups finish the phase.
 #pragma once
 
 #include "kernels.hpp"
