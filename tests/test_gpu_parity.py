@@ -174,6 +174,15 @@ def test_token_kernel_equals_kernel_by_kernel_launch_and_is_deterministic(orc, l
         assert nxt == int(np.argmax(outs[0][p]))
 
 
+@pytest.mark.parametrize("shape", TINY)
+def test_forward_matches_oracle_in_both_launch_modes(orc, shape, launch_mode):
+    # every tiny shape (head 16..256, multiquery, unaligned rows) through l2j_forward at every position
+    m, g = make_pair(orc, shape, seed=23, realistic=True)
+    rng = np.random.default_rng(2)
+    for pos, tok in enumerate(rng.integers(0, shape[5], size=shape[6])):
+        assert rel_err(g.forward(int(tok), pos), m.forward(int(tok), pos)) < 1e-4, pos
+
+
 def test_split_attention_in_both_launch_modes(orc, launch_mode):
     # contexts long enough that attention is split over several workgroups (whole-token launch: beyond 64
     # positions; kernel-by-kernel: beyond 32) and folded by the last arriver; multiquery, head 16
