@@ -85,6 +85,18 @@ def lib():
         "orc_forward": (None, [vp, C.c_int, C.c_int]),
         "orc_forward_layers": (None, [vp, C.c_int, C.c_int, C.c_int]),
         "orc_generate_greedy": (C.c_int, [vp, i32p, C.c_int, C.c_int, i32p, fp, C.POINTER(C.c_double)]),
+        "orc_find_max": (None, [fp, C.c_int, fp, C.c_int64, C.c_int]),
+        "orc_sampler_new": (vp, [C.c_int64, C.c_int]),
+        "orc_sampler_free": (None, [vp]),
+        "orc_sampler_next_bits": (C.c_int32, [vp, C.c_int]),
+        "orc_sampler_next_float": (C.c_float, [vp]),
+        "orc_sample": (C.c_int, [vp, fp, C.c_int]),
+        "orc_sample_topp": (C.c_int, [vp, fp, C.c_int, C.c_float]),
+        "orc_sample_coin": (C.c_int, [fp, C.c_int, C.c_float]),
+        "orc_sample_topp_coin": (C.c_int, [vp, fp, C.c_int, C.c_float, C.c_float]),
+        "orc_sample_step": (C.c_int, [vp, fp, C.c_int, C.c_float, C.c_float]),
+        "orc_generate": (C.c_int, [vp, i32p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int64, i32p,
+                                   C.POINTER(C.c_double)]),
         "orc_write_quant_file": (C.c_int, [C.c_char_p, u8p, C.c_int64]),
         "orc_read_quant_file": (C.c_int64, [C.c_char_p, u8p, C.c_int64]),
         "orc_load_checkpoint": (vp, [C.c_char_p, C.c_int, C.c_char_p, C.c_int]),
@@ -114,6 +126,53 @@ def _u8(a):
 def _i32(a):
     assert a.dtype == np.int32 and a.flags.c_contiguous
     return a.ctypes.data_as(C.POINTER(C.c_int32))
+
+
+# ---- sampling ----------------------------------------------------------------------------
+class Sampler:
+    """J/Sampler.java: java.util.Random(seed) + the ProbIndex array that outlives a call."""
+
+    def __init__(self, rng_seed, vocab_size):
+        self.n = vocab_size
+        self.h = lib().orc_sampler_new(rng_seed, vocab_size)
+        if not self.h:
+            raise MemoryError("orc_sampler_new")
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().orc_sampler_free(self.h)
+            self.h = None
+
+    def next_bits(self, bits):
+        return lib().orc_sampler_next_bits(self.h, bits)
+
+    def next_float(self):
+        return lib().orc_sampler_next_float(self.h)
+
+    def sample(self, probs, coin=None):
+        probs = np.ascontiguousarray(probs, dtype=np.float32)
+        if coin is None:
+            return lib().orc_sample(self.h, _fp(probs), probs.size)
+        return lib().orc_sample_coin(_fp(probs), probs.size, coin)
+
+    def sample_topp(self, probs, topp, coin=None):
+        probs = np.ascontiguousarray(probs, dtype=np.float32)
+        if coin is None:
+            return lib().orc_sample_topp(self.h, _fp(probs), probs.size, topp)
+        return lib().orc_sample_topp_coin(self.h, _fp(probs), probs.size, topp, coin)
+
+    def step(self, logits, temperature, topp):
+        """J/Run.java:643-665 on a copy; returns (next, the array after the step)."""
+        a = np.array(logits, dtype=np.float32, copy=True)
+        nxt = lib().orc_sample_step(self.h, _fp(a), a.size, temperature, topp)
+        return nxt, a
+
+
+def find_max(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros(1, dtype=np.float32)
+    lib().orc_find_max(_fp(out), 0, _fp(x), 0, x.size)
+    return float(out[0])
 
 
 # ---- codec -------------------------------------------------------------------------------
@@ -303,3 +362,13 @@ class Model:
         n = lib().orc_generate_greedy(self.h, _i32(prompt), prompt.size, steps, _i32(out),
                                       _fp(logits) if want_logits else None, C.byref(sec))
         return out[:n], (logits[:n] if want_logits else None), sec.value
+
+    def generate(self, prompt, steps, temperature, topp, rng_seed):
+        """J/Run.java:611-685 with the sampler of J/Run.java:620."""
+        prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        cap = self.cfg.seq_len if steps <= 0 or steps > self.cfg.seq_len else steps
+        out = np.zeros(cap, dtype=np.int32)
+        sec = C.c_double(0)
+        n = lib().orc_generate(self.h, _i32(prompt), prompt.size, steps, temperature, topp, rng_seed,
+                               _i32(out), C.byref(sec))
+        return out[:n], sec.value

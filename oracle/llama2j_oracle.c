@@ -752,6 +752,191 @@ int orc_generate_greedy(orc_model *m, const int32_t *prompt, int n_prompt, int s
 }
 
 /* ------------------------------------------------------------------ */
+/* sampling                                                             */
+/* ------------------------------------------------------------------ */
+
+void orc_find_max(float *max, int max_index, const float *x, int64_t index, int size)
+{
+    /* K/FindMax.java:40-48 */
+    float max_val = x[index];
+    for (int i = 1; i < size; i++) {
+        if (x[index + i] > max_val) max_val = x[index + i];
+    }
+    max[max_index] = max_val;
+}
+
+struct orc_sampler {
+    uint64_t rng;     /* java.util.Random's 48-bit state */
+    int n;
+    float *prob;      /* J/Sampler.java:18,60-62 : the ProbIndex array, kept between calls */
+    int32_t *index;
+    float *tprob;     /* merge buffers */
+    int32_t *tindex;
+};
+
+#define JRAND_MULT 0x5DEECE66DULL
+#define JRAND_MASK ((1ULL << 48) - 1)
+
+orc_sampler *orc_sampler_new(int64_t rng_seed, int vocab_size)
+{
+    /* J/Sampler.java:24-31; new Random(seed): state = (seed ^ 0x5DEECE66D) mod 2^48 */
+    orc_sampler *s = (orc_sampler *)calloc(1, sizeof(*s));
+    if (!s) return NULL;
+    s->rng = ((uint64_t)rng_seed ^ JRAND_MULT) & JRAND_MASK;
+    s->n = vocab_size;
+    s->prob = (float *)calloc((size_t)vocab_size, sizeof(float));      /* new ProbIndex(): prob 0, index 0 */
+    s->index = (int32_t *)calloc((size_t)vocab_size, sizeof(int32_t));
+    s->tprob = (float *)calloc((size_t)vocab_size, sizeof(float));
+    s->tindex = (int32_t *)calloc((size_t)vocab_size, sizeof(int32_t));
+    if (!s->prob || !s->index || !s->tprob || !s->tindex) { orc_sampler_free(s); return NULL; }
+    return s;
+}
+
+void orc_sampler_free(orc_sampler *s)
+{
+    if (!s) return;
+    free(s->prob); free(s->index); free(s->tprob); free(s->tindex);
+    free(s);
+}
+
+int32_t orc_sampler_next_bits(orc_sampler *s, int bits)
+{
+    /* java.util.Random.next(bits) */
+    s->rng = (s->rng * JRAND_MULT + 0xBULL) & JRAND_MASK;
+    return (int32_t)(uint32_t)(s->rng >> (48 - bits));
+}
+
+float orc_sampler_next_float(orc_sampler *s)
+{
+    /* J/Sampler.java:20-22 -> java.util.Random.nextFloat() = next(24) / (float)(1 << 24) */
+    return (float)orc_sampler_next_bits(s, 24) / (float)(1 << 24);
+}
+
+int orc_sample_coin(const float *probs, int n, float r)
+{
+    /* J/Sampler.java:33-44 */
+    float cdf = 0.0f;
+    for (int i = 0; i < n; i++) {
+        cdf += probs[i];
+        if (r < cdf) return i;
+    }
+    return n - 1;
+}
+
+int orc_sample(orc_sampler *s, const float *probs, int n)
+{
+    return orc_sample_coin(probs, n, orc_sampler_next_float(s));
+}
+
+/* Stable descending merge sort of the whole ProbIndex array: Arrays.sort(Object[]) is a stable
+ * merge sort and ProbIndex.compareTo (J/Sampler.java:64-73) orders by prob, larger first. */
+static void sort_prob_index(orc_sampler *s)
+{
+    float *a = s->prob, *b = s->tprob;
+    int32_t *ai = s->index, *bi = s->tindex;
+    const int n = s->n;
+    for (int width = 1; width < n; width *= 2) {
+        for (int lo = 0; lo < n; lo += 2 * width) {
+            int mid = lo + width < n ? lo + width : n;
+            int hi = lo + 2 * width < n ? lo + 2 * width : n;
+            int i = lo, j = mid, k = lo;
+            while (i < mid && j < hi) {
+                if (a[j] > a[i]) { b[k] = a[j]; bi[k] = ai[j]; j++; }   /* strictly larger moves ahead */
+                else { b[k] = a[i]; bi[k] = ai[i]; i++; }
+                k++;
+            }
+            while (i < mid) { b[k] = a[i]; bi[k] = ai[i]; i++; k++; }
+            while (j < hi) { b[k] = a[j]; bi[k] = ai[j]; j++; k++; }
+        }
+        float *t = a; a = b; b = t;
+        int32_t *ti = ai; ai = bi; bi = ti;
+    }
+    if (a != s->prob) {
+        memcpy(s->prob, a, (size_t)n * sizeof(float));
+        memcpy(s->index, ai, (size_t)n * sizeof(int32_t));
+    }
+}
+
+static int topp_pick(orc_sampler *s, const float *probs, int n, float topp, int draw, float coin)
+{
+    /* J/Sampler.java:76-120 */
+    int n0 = 0;
+    float cutoff = (1.0f - topp) / (float)(n - 1);
+    for (int i = 0; i < n; i++) {
+        if (probs[i] != probs[i]) return -1;        /* :88-90 */
+        if (probs[i] >= cutoff) {
+            s->index[n0] = i;
+            s->prob[n0] = probs[i];
+            n0++;
+        }
+    }
+    sort_prob_index(s);                             /* :97 : the whole array */
+    float cumulative_prob = 0.0f;
+    int last_idx = n0 - 1;
+    for (int i = 0; i < n0; i++) {
+        cumulative_prob += s->prob[i];
+        if (cumulative_prob > topp) { last_idx = i; break; }
+    }
+    if (draw) coin = orc_sampler_next_float(s);
+    float r = coin * cumulative_prob;
+    float cdf = 0.0f;
+    for (int i = 0; i <= last_idx; i++) {
+        cdf += s->prob[i];
+        if (r < cdf) return s->index[i];
+    }
+    return s->index[last_idx];   /* n0 == 0 would index -1 in the reference (an exception); callers avoid it */
+}
+
+int orc_sample_topp(orc_sampler *s, const float *probs, int n, float topp)
+{
+    return topp_pick(s, probs, n, topp, 1, 0.0f);
+}
+
+int orc_sample_topp_coin(orc_sampler *s, const float *probs, int n, float topp, float coin)
+{
+    return topp_pick(s, probs, n, topp, 0, coin);
+}
+
+int orc_sample_step(orc_sampler *s, float *logits, int n, float temperature, float topp)
+{
+    /* J/Run.java:643-665 */
+    if (temperature == 0.0f) return orc_argmax(logits, n);
+    for (int q = 0; q < n; q++) logits[q] /= temperature;
+    float max[1] = {0.0f};
+    orc_find_max(max, 0, logits, 0, n);
+    orc_exp_sum_normalize(logits, max, 0, 0, n);
+    if ((double)topp > 0.999) return orc_sample(s, logits, n);
+    return orc_sample_topp(s, logits, n, topp);
+}
+
+int orc_generate(orc_model *m, const int32_t *prompt, int n_prompt, int steps, float temperature,
+                 float topp, int64_t rng_seed, int32_t *out_tokens, double *seconds)
+{
+    /* J/Run.java:599-603, 611-685 */
+    if (steps <= 0 || steps > m->cfg.seq_len) steps = m->cfg.seq_len;
+    orc_sampler *s = orc_sampler_new(rng_seed, m->cfg.vocab_size);
+    if (!s) return -1;
+    double start = 0.0;
+    int started = 0;
+    int token = 1;
+    int pos = 0;
+    while (pos < steps) {
+        orc_forward(m, token, pos);
+        int next;
+        if (pos < n_prompt) next = prompt[pos];
+        else next = orc_sample_step(s, m->logits, m->cfg.vocab_size, temperature, topp);
+        out_tokens[pos] = next;
+        pos++;
+        if (next == 1) break;
+        token = next;
+        if (!started) { start = now_s(); started = 1; }
+    }
+    if (seconds) *seconds = started ? now_s() - start : 0.0;
+    orc_sampler_free(s);
+    return pos;
+}
+
+/* ------------------------------------------------------------------ */
 /* files                                                                */
 /* ------------------------------------------------------------------ */
 

@@ -1,8 +1,9 @@
 /*
  * TEST INFRASTRUCTURE - NOT PART OF THE PRODUCT.
  *
- * CPU restatement of llama2j's per-token forward pass (its CPU mode), the
- * group-int8 codec and the checkpoint / quant-cache formats.  Only tests,
+ * CPU restatement of llama2j's per-token forward pass (its CPU mode), its
+ * sampler (java.util.Random included), the group-int8 codec and the
+ * checkpoint / quant-cache formats.  Only tests,
  * the smoke check and the cpu_baseline leg of the benchmark may link or
  * load this; the HIP library never does.
  *
@@ -104,6 +105,30 @@ void orc_forward_layers(orc_model *m, int token, int pos, int n_layers_run);
  * seconds (may be NULL) = wall time from after the first iteration to the end (J/Run.java:682-684). */
 int orc_generate_greedy(orc_model *m, const int32_t *prompt, int n_prompt, int steps,
                         int32_t *out_tokens, float *logits_out, double *seconds);
+
+/* ---- sampling: J/Sampler.java, K/FindMax.java, J/Run.java:643-665 ---------- */
+void orc_find_max(float *max, int max_index, const float *x, int64_t index, int size); /* K/FindMax.java:40-48 */
+/* java.util.Random (the 48-bit linear congruential generator of the Java SE specification, which
+ * J/Sampler.java:17-25 uses through nextFloat): seed scrambled with 0x5DEECE66D, next(bits) =
+ * top bits of seed*0x5DEECE66D+0xB mod 2^48, nextFloat = next(24) / 2^24. */
+typedef struct orc_sampler orc_sampler;
+orc_sampler *orc_sampler_new(int64_t rng_seed, int vocab_size);     /* J/Sampler.java:24-31 */
+void orc_sampler_free(orc_sampler *s);
+int32_t orc_sampler_next_bits(orc_sampler *s, int bits);            /* java.util.Random.next */
+float orc_sampler_next_float(orc_sampler *s);                       /* J/Sampler.java:20-22 */
+int orc_sample(orc_sampler *s, const float *probs, int n);          /* J/Sampler.java:33-44 */
+/* J/Sampler.java:76-120, including its whole-array sort: entries beyond the candidates of this call
+ * keep what earlier calls left there and take part in the sort.  Returns -1 for a NaN (the reference throws). */
+int orc_sample_topp(orc_sampler *s, const float *probs, int n, float topp);
+/* The same two with the random draw given by the caller instead of taken from the generator. */
+int orc_sample_coin(const float *probs, int n, float coin);
+int orc_sample_topp_coin(orc_sampler *s, const float *probs, int n, float topp, float coin);
+/* J/Run.java:643-665: argmax at temperature 0, else divide, FindMax, ExpSumNormalize (logits become
+ * probabilities in place) and sample / sample_topp (topp > 0.999 selects plain sampling). */
+int orc_sample_step(orc_sampler *s, float *logits, int n, float temperature, float topp);
+/* J/Run.java:611-685 with a sampler; as orc_generate_greedy otherwise. */
+int orc_generate(orc_model *m, const int32_t *prompt, int n_prompt, int steps, float temperature,
+                 float topp, int64_t rng_seed, int32_t *out_tokens, double *seconds);
 
 /* ---- files: J/BinFileReader, J/BinFileWriter, J/TransformerWeights ------- */
 int orc_write_quant_file(const char *path, const uint8_t *bytes, int64_t nbytes); /* J/BinFileWriter.java:20-34 */
