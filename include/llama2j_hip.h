@@ -122,6 +122,25 @@ int l2j_forward_taps(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_
 int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps,
                       int32_t *out_tokens, int32_t *n_out, double *seconds);
 
+/* ---- sampling on the device: J/Sampler.java and the sampling branch of J/Run.java:643-665 ----
+ * The context holds one sampler = the reference's Sampler object: a java.util.Random and the ProbIndex
+ * array that sample_topp sorts whole, so that entries of earlier calls take part in later ones
+ * (J/Sampler.java:17-18, 92-97).  vocab_size is limited to 36864 (the probabilities are kept in LDS). */
+/* = new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31, J/Run.java:620). */
+int l2j_sampler_seed(l2j_ctx *ctx, int64_t rng_seed);
+/* One sampling step (J/Run.java:643-665): temperature 0 = Sampler.argmax; else logits /= temperature,
+ * FindMax (K/FindMax.java:40-48), ExpSumNormalize (K/ExpSumNormalize.java:25-38), then Sampler.sample
+ * (J/Sampler.java:33-44) when topp > 0.999, else Sampler.sample_topp (J/Sampler.java:76-120).
+ * logits_or_null: vocab_size floats of the caller to sample from (Sampler's methods take the array), or NULL for
+ * the logits of the last forward; either way they are probabilities afterwards (L2J_B_LOGITS), as in the reference.
+ * coin: the caller's Random.nextFloat() in [0, 1), or negative to draw from the context's generator (one draw per
+ * call, none at temperature 0).  A NaN among the probabilities is an error, as sample_topp throws. */
+int l2j_sample(l2j_ctx *ctx, const float *logits_or_null, float temperature, float topp, float coin, int32_t *next);
+/* = the token loop of Run.main with a sampler (J/Run.java:599-603, 611-685): as l2j_decode_greedy, but every
+ * unforced token is sampled as in l2j_sample from a sampler seeded with rng_seed; the logits never leave the device. */
+int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature,
+                      float topp, int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds);
+
 /* Activation / cache taps.  layer < 0 reads the live buffer, layer >= 0 the per-layer tap.
  * `off` and `n` are in floats. */
 int l2j_read(l2j_ctx *ctx, int which, int layer, uint64_t off, float *dst, uint64_t n);

@@ -98,6 +98,10 @@ def _signatures():
         "l2j_forward_argmax": (C.c_int, [vp, C.c_int32, C.c_int32, i32p]),
         "l2j_forward_taps": (C.c_int, [vp, C.c_int32, C.c_int32, fp]),
         "l2j_decode_greedy": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, i32p, i32p, C.POINTER(C.c_double)]),
+        "l2j_sampler_seed": (C.c_int, [vp, C.c_int64]),
+        "l2j_sample": (C.c_int, [vp, fp, C.c_float, C.c_float, C.c_float, i32p]),
+        "l2j_decode_sample": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, C.c_float, C.c_float, C.c_int64, i32p, i32p,
+                                        C.POINTER(C.c_double)]),
         "l2j_read": (C.c_int, [vp, C.c_int, C.c_int, C.c_uint64, fp, C.c_uint64]),
         "l2j_write_kv": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, fp, fp]),
         "l2j_sync": (C.c_int, [vp]),
@@ -203,7 +207,8 @@ class Quant:
 
 
 class Sampler:
-    """J/Sampler.java:46-57 (greedy only); the device computes the same first-max inside the forward."""
+    """J/Sampler.java:46-57; the device computes the same first-max inside the forward.  The sampling methods
+    of the reference run on the device through Transformer.sampler_seed / sample / decode_sample."""
 
     @staticmethod
     def argmax(logits):
@@ -303,6 +308,34 @@ class Transformer:
         n = C.c_int32(0)
         sec = C.c_double(0.0)
         _check(lib().l2j_decode_greedy(self._h, _i32(p), p.size, steps, _i32(out), C.byref(n), C.byref(sec)))
+        return out[:n.value], sec.value
+
+    def sampler_seed(self, rng_seed):
+        """new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31): java.util.Random(seed), empty ProbIndex array."""
+        _check(lib().l2j_sampler_seed(self._h, rng_seed))
+
+    def sample(self, temperature, topp, logits=None, coin=None):
+        """The sampling step of J/Run.java:643-665 on the device.  logits: an array to sample from instead of the
+        last forward's; coin: the caller's Random.nextFloat() instead of the context's generator."""
+        nxt = C.c_int32(0)
+        lp = None
+        if logits is not None:
+            logits = np.ascontiguousarray(logits, dtype=np.float32)
+            if logits.size != self.config.vocab_size:
+                raise ValueError("logits must hold vocab_size floats")
+            lp = _fp(logits)
+        _check(lib().l2j_sample(self._h, lp, temperature, topp, -1.0 if coin is None else coin, C.byref(nxt)))
+        return nxt.value
+
+    def decode_sample(self, prompt, steps, temperature, topp, rng_seed):
+        """The token loop of Run.main with its sampler (J/Run.java:611-685)."""
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        cap = self.config.seq_len if steps <= 0 or steps > self.config.seq_len else steps
+        out = np.zeros(cap, dtype=np.int32)
+        n = C.c_int32(0)
+        sec = C.c_double(0.0)
+        _check(lib().l2j_decode_sample(self._h, _i32(p), p.size, steps, temperature, topp, rng_seed, _i32(out),
+                                       C.byref(n), C.byref(sec)))
         return out[:n.value], sec.value
 
     def read(self, which, layer=-1, off=0, n=None):

@@ -3,6 +3,7 @@
 // the per-token launch sequence as a hipGraph and replays it.
 #include "kernels.hpp"
 #include "phase_kernels.hpp"
+#include "sampler_kernels.hpp"
 
 #include <hip/hip_ext.h>
 
@@ -19,6 +20,12 @@
 #include "host_internal.h"
 
 using namespace l2j;
+
+namespace l2j {
+// stable descending sort of (prob, index) pairs; temp == nullptr: only report the scratch size (sampler_sort.hip)
+hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, const float *kin, float *kout, const int *vin, int *vout, unsigned n,
+                                hipStream_t s);
+}  // namespace l2j
 
 namespace {
 
@@ -108,6 +115,15 @@ struct l2j_ctx {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     std::vector<hipEvent_t> events;
+
+    // device sampler (allocated by its first use): the reference's Sampler object
+    SamplerState *ss = nullptr;
+    SamplerState *h_ss = nullptr;               // pinned
+    float *pi_prob[2] = {nullptr, nullptr};     // the ProbIndex array, before and after the sort of a call
+    int *pi_idx[2] = {nullptr, nullptr};
+    int pi_cur = 0;                             // which of the two holds the array between calls
+    void *sort_temp = nullptr;
+    size_t sort_temp_bytes = 0;
 };
 
 namespace {
@@ -415,6 +431,145 @@ void destroy_graph(l2j_ctx *c)
 
 uint64_t quant_bytes_of(uint64_t weights) { return (weights / kGroup) * kGroupBytes + (weights % kGroup ? kGroupBytes : 0); }
 
+// ---- device sampler ------------------------------------------------------------------------------------
+
+int ensure_sampler(l2j_ctx *c)
+{
+    if (c->ss) return L2J_OK;
+    const int n = c->cfg.vocab_size;
+    if (n > kSampleMaxVocab) return fail(L2J_E_SIZE, "device sampler: vocab_size above 36864 does not fit the LDS");
+    if (n < 2) return fail(L2J_E_SIZE, "device sampler: vocab_size below 2");
+    int rc;
+    for (int i = 0; i < 2; i++) {
+        if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n))) return rc;
+        if ((rc = dev_alloc(&c->pi_idx[i], (uint64_t)n))) return rc;
+    }
+    size_t bytes = 0;
+    HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream));
+    c->sort_temp_bytes = bytes;
+    HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
+    HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
+    const int lds = ((n + 7) & ~7) * (int)sizeof(float);
+    HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    if ((rc = dev_alloc(&c->ss, 1))) return rc;
+    return L2J_OK;
+}
+
+// new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31): Random(seed) scrambles its seed, every ProbIndex is (0, 0)
+int seed_sampler(l2j_ctx *c, int64_t rng_seed)
+{
+    int rc = ensure_sampler(c);
+    if (rc) return rc;
+    memset(c->h_ss, 0, sizeof(SamplerState));
+    c->h_ss->rng = ((unsigned long long)rng_seed ^ kJavaRandMult) & kJavaRandMask;
+    HIPCHK(hipMemcpyAsync(c->ss, c->h_ss, sizeof(SamplerState), hipMemcpyHostToDevice, c->stream));
+    const size_t n = (size_t)c->cfg.vocab_size;
+    for (int i = 0; i < 2; i++) {
+        HIPCHK(hipMemsetAsync(c->pi_prob[i], 0, n * sizeof(float), c->stream));
+        HIPCHK(hipMemsetAsync(c->pi_idx[i], 0, n * sizeof(int), c->stream));
+    }
+    HIPCHK(hipStreamSynchronize(c->stream));
+    c->pi_cur = 0;
+    return L2J_OK;
+}
+
+// The sampling step of J/Run.java:643-665 on c->logits; in_loop: the token replaces what k_finish stored.
+hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin, bool in_loop)
+{
+    const int n = c->cfg.vocab_size;
+    const int cur = c->pi_cur, other = cur ^ 1;
+    SampleArgs a{};
+    a.logits = c->logits; a.n = n;
+    a.temperature = temperature; a.topp = topp; a.coin = coin;
+    a.plain = (double)topp > 0.999;
+    a.ss = c->ss;
+    a.cand_prob = c->pi_prob[cur]; a.cand_idx = c->pi_idx[cur];
+    a.sorted_prob = c->pi_prob[other]; a.sorted_idx = c->pi_idx[other];
+    a.st = in_loop ? c->st : nullptr;
+    a.out_tokens = c->out_tokens;
+    const size_t lds = (size_t)((n + 7) & ~7) * sizeof(float);
+    hipLaunchKernelGGL(k_sample_probs, dim3(1), dim3(1024), lds, c->stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || a.plain) return e;
+    size_t bytes = c->sort_temp_bytes;
+    e = sort_prob_index_desc(c->sort_temp, &bytes, c->pi_prob[cur], c->pi_prob[other], c->pi_idx[cur], c->pi_idx[other],
+                             (unsigned)n, c->stream);
+    if (e != hipSuccess) return e;
+    c->pi_cur = other;
+    hipLaunchKernelGGL(k_topp_pick, dim3(1), dim3(1024), lds, c->stream, a);
+    return hipGetLastError();
+}
+
+int check_sampler_args(float temperature, float topp)
+{
+    if (!(temperature >= 0.0f) || !(topp >= 0.0f && topp <= 1.0f)) return fail(L2J_E_ARG, "temperature must be >= 0 and topp in [0, 1]");
+    return L2J_OK;
+}
+
+// J/Run.java:611-685; temperature 0 is the greedy loop, else every unforced token is sampled on the device.
+int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, bool sampled, float temperature, float topp,
+                int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds)
+{
+    if (!c || !out_tokens || !n_out || (n_prompt > 0 && !prompt) || n_prompt < 0) return fail(L2J_E_ARG, "bad argument");
+    if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const int S = c->cfg.seq_len;
+    if (steps <= 0 || steps > S) steps = S;  // J/Run.java:599-603
+    const int np = std::min(n_prompt, S);
+    for (int i = 0; i < np; i++)
+        if (prompt[i] < 0 || prompt[i] >= c->cfg.vocab_size) return fail(L2J_E_ARG, "prompt id out of range");
+    int rc;
+    if (sampled && (rc = seed_sampler(c, rng_seed))) return rc;  // J/Run.java:620
+    if (np > 0) {
+        memcpy(c->h_tokens, prompt, (size_t)np * sizeof(int));
+        HIPCHK(hipMemcpyAsync(c->prompt, c->h_tokens, (size_t)np * sizeof(int), hipMemcpyHostToDevice, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+    }
+    if ((rc = set_state(c, 1, 0, np))) return rc;  // token 1 = BOS at pos 0 (J/Run.java:614)
+
+    // One event after every token of a batch: the stop rule (next == 1) is checked per batch, and the
+    // clock runs from the end of the first token to the end of the token that ended the loop.
+    const int batch = 32;
+    while ((int)c->events.size() < batch + 1) {
+        hipEvent_t ev;
+        HIPCHK(hipEventCreate(&ev));
+        c->events.push_back(ev);
+    }
+    hipEvent_t ev_first = c->events[batch];
+    float total_ms = 0.f;
+    int pos = 0;
+    bool stopped = false;
+    while (pos < steps && !stopped) {
+        const int nb = std::min(batch, steps - pos);
+        for (int i = 0; i < nb; i++) {
+            HIPCHK(launch_one_token(c));
+            if (sampled && pos + i >= np) HIPCHK(launch_sampler(c, temperature, topp, -1.0f, true));  // J/Run.java:635-665
+            if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
+            HIPCHK(hipEventRecord(c->events[i], c->stream));
+        }
+        HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        if (sampled) HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        if ((rc = check_barrier_error(c))) return rc;
+        if (sampled && c->h_ss->nan) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
+        int used = nb;
+        for (int i = 0; i < nb; i++) {
+            out_tokens[pos + i] = c->h_tokens[i];
+            if (c->h_tokens[i] == 1) {  // J/Run.java:670-672
+                used = i + 1;
+                stopped = true;
+                break;
+            }
+        }
+        if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
+        pos += used;
+    }
+    *n_out = pos;
+    if (seconds) *seconds = (double)total_ms * 1e-3;
+    return L2J_OK;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------------------------------------
@@ -549,6 +704,13 @@ void l2j_destroy(l2j_ctx *c)
     (void)hipFree(c->out_tokens);
     (void)hipFree(c->bar_ctr);
     (void)hipFree(c->fault);
+    (void)hipFree(c->ss);
+    for (int i = 0; i < 2; i++) {
+        (void)hipFree(c->pi_prob[i]);
+        (void)hipFree(c->pi_idx[i]);
+    }
+    (void)hipFree(c->sort_temp);
+    if (c->h_ss) (void)hipHostFree(c->h_ss);
     if (c->h_fault) (void)hipHostFree(c->h_fault);
     for (float *t : c->taps) (void)hipFree(t);
     if (c->h_st) (void)hipHostFree(c->h_st);
@@ -877,58 +1039,51 @@ int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32
                       double *seconds)
 {
     std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!c || !out_tokens || !n_out || (n_prompt > 0 && !prompt) || n_prompt < 0) return fail(L2J_E_ARG, "bad argument");
-    if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const int S = c->cfg.seq_len;
-    if (steps <= 0 || steps > S) steps = S;  // J/Run.java:599-603
-    const int np = std::min(n_prompt, S);
-    for (int i = 0; i < np; i++)
-        if (prompt[i] < 0 || prompt[i] >= c->cfg.vocab_size) return fail(L2J_E_ARG, "prompt id out of range");
-    if (np > 0) {
-        memcpy(c->h_tokens, prompt, (size_t)np * sizeof(int));
-        HIPCHK(hipMemcpyAsync(c->prompt, c->h_tokens, (size_t)np * sizeof(int), hipMemcpyHostToDevice, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream));
-    }
-    int rc = set_state(c, 1, 0, np);  // token 1 = BOS at pos 0 (J/Run.java:614)
-    if (rc) return rc;
+    return decode_loop(c, prompt, n_prompt, steps, false, 0.0f, 0.0f, 0, out_tokens, n_out, seconds);
+}
 
-    // One event after every token of a batch: the stop rule (next == 1) is checked per batch, and the
-    // clock runs from the end of the first token to the end of the token that ended the loop.
-    const int batch = 32;
-    while ((int)c->events.size() < batch + 1) {
-        hipEvent_t ev;
-        HIPCHK(hipEventCreate(&ev));
-        c->events.push_back(ev);
+int l2j_decode_sample(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature, float topp,
+                      int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds)
+{
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+    int rc = check_sampler_args(temperature, topp);
+    if (rc) return rc;
+    return decode_loop(c, prompt, n_prompt, steps, temperature != 0.0f, temperature, topp, rng_seed, out_tokens, n_out, seconds);
+}
+
+int l2j_sampler_seed(l2j_ctx *c, int64_t rng_seed)
+{
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+    if (!c) return fail(L2J_E_ARG, "null context");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    return seed_sampler(c, rng_seed);
+}
+
+int l2j_sample(l2j_ctx *c, const float *logits, float temperature, float topp, float coin, int32_t *next)
+{
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+    if (!c || !next) return fail(L2J_E_ARG, "null argument");
+    int rc = check_sampler_args(temperature, topp);
+    if (rc) return rc;
+    if (coin >= 1.0f) return fail(L2J_E_ARG, "coin must be below 1 (negative: the context's generator draws)");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    if (!c->ss && (rc = seed_sampler(c, 0))) return rc;
+    const int n = c->cfg.vocab_size;
+    if (logits) HIPCHK(hipMemcpyAsync(c->logits, logits, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream));
+    if (temperature == 0.0f) {
+        hipLaunchKernelGGL(k_argmax_logits, dim3(1), dim3(1024), 0, c->stream, c->logits, n, c->ss);  // J/Run.java:644-646
+        HIPCHK(hipGetLastError());
+    } else {
+        HIPCHK(launch_sampler(c, temperature, topp, coin, false));
     }
-    hipEvent_t ev_first = c->events[batch];
-    float total_ms = 0.f;
-    int pos = 0;
-    bool stopped = false;
-    while (pos < steps && !stopped) {
-        const int nb = std::min(batch, steps - pos);
-        for (int i = 0; i < nb; i++) {
-            HIPCHK(launch_one_token(c));
-            if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
-            HIPCHK(hipEventRecord(c->events[i], c->stream));
-        }
-        HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream));
-        if ((rc = check_barrier_error(c))) return rc;
-        int used = nb;
-        for (int i = 0; i < nb; i++) {
-            out_tokens[pos + i] = c->h_tokens[i];
-            if (c->h_tokens[i] == 1) {  // J/Run.java:670-672
-                used = i + 1;
-                stopped = true;
-                break;
-            }
-        }
-        if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
-        pos += used;
+    HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
+    HIPCHK(hipStreamSynchronize(c->stream));
+    if (c->h_ss->nan) {
+        c->h_ss->nan = 0;
+        HIPCHK(hipMemcpy(&c->ss->nan, &c->h_ss->nan, sizeof(int), hipMemcpyHostToDevice));
+        return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
     }
-    *n_out = pos;
-    if (seconds) *seconds = (double)total_ms * 1e-3;
+    *next = c->h_ss->result;
     return L2J_OK;
 }
 

@@ -1,0 +1,141 @@
+"""Device sampler (l2j_sampler_seed / l2j_sample / l2j_decode_sample) against the CPU oracle's restatement of
+J/Sampler.java and J/Run.java:643-665, through the C ABI: the sampled tokens must be identical, the
+probabilities left in the logits buffer equal to float32 rounding of the exponential."""
+import numpy as np
+import pytest
+
+import llama2j_amd as l2j
+from llama2j_amd.binding import BUFFER, L2JError
+
+pytestmark = pytest.mark.gpu
+
+
+def small_transformer(vocab, seed=3):
+    g = l2j.Transformer(l2j.Config(32, 64, 1, 2, 2, vocab, 8, 1))
+    g.fill_synthetic(seed, 0.1)
+    g.finalize()
+    return g
+
+
+def logits_of(rng, n, kind):
+    x = rng.standard_normal(n).astype(np.float32)
+    if kind == "flat":
+        return x * np.float32(0.05)
+    if kind == "peaked":
+        x = x * np.float32(4.0)
+        x[rng.integers(0, n)] += np.float32(12.0)
+        return x
+    return x * np.float32(2.0)
+
+
+def check_probabilities(got, want):
+    # the only operation that may differ is the last bit of the double exponential before it is narrowed
+    assert np.abs(got - want).max() <= 2e-7 * want.max(), np.abs(got - want).max()
+
+
+@pytest.mark.parametrize("vocab", [1003, 32000])
+def test_plain_sampling_matches_oracle(orc, vocab):
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(vocab)
+    g.sampler_seed(77)
+    o = orc.Sampler(77, vocab)
+    for call, kind in enumerate(["mid", "flat", "peaked", "mid", "flat", "peaked"]):
+        lg = logits_of(rng, vocab, kind)
+        t = float(rng.choice([0.5, 0.9, 1.0, 1.7]))
+        want, probs = o.step(lg, t, 1.0)                       # topp > 0.999: Sampler.sample
+        assert g.sample(t, 1.0, logits=lg) == want, (call, kind)
+        got = g.read(BUFFER.LOGITS)
+        check_probabilities(got, probs)
+        for coin in (0.0, 0.3, 0.99999994, float(np.float32(rng.random()))):
+            assert g.sample(t, 1.0, logits=lg, coin=coin) == o.sample(got, coin=coin), (call, kind, coin)
+
+
+@pytest.mark.parametrize("vocab", [1003, 32000])
+def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, vocab):
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(vocab + 1)
+    g.sampler_seed(-12345)
+    o = orc.Sampler(-12345, vocab)
+    kinds = ["flat", "peaked", "mid", "peaked", "flat", "mid", "peaked", "peaked", "flat", "mid"] * 2
+    for call, kind in enumerate(kinds):
+        lg = logits_of(rng, vocab, kind)
+        t = float(rng.choice([0.7, 0.9, 1.0]))
+        topp = float(rng.choice([0.5, 0.9, 0.95, 0.99]))
+        want, probs = o.step(lg, t, topp)
+        assert g.sample(t, topp, logits=lg) == want, (call, kind, topp)
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
+
+
+def test_topp_worked_example_with_entries_of_an_earlier_call(orc):
+    # the hand-worked case of the oracle's tests, on the device: eight tokens, padded with impossible ones
+    vocab = 16
+    g = small_transformer(vocab)
+    g.sampler_seed(1)
+    o = orc.Sampler(1, vocab)
+    with np.errstate(divide="ignore"):
+        u = np.log(np.array([0.125] * 8 + [0.0] * 8, dtype=np.float32))
+        p = np.log(np.array([0.9, 0.04, 0.03, 0.01, 0.01, 0.005, 0.0025, 0.0025] + [0.0] * 8, dtype=np.float32))
+    for lg, topp, coin in ((u, 0.5, 0.0), (p, 0.95, 0.95), (p, 0.95, 0.2), (u, 0.9, 0.7)):
+        _, probs = o.step(lg, 1.0, 1.0)
+        assert g.sample(1.0, topp, logits=lg, coin=coin) == o.sample_topp(probs, topp, coin=coin)
+
+
+def test_temperature_zero_is_first_max_and_nan_is_an_error(orc):
+    vocab = 1003
+    g = small_transformer(vocab)
+    lg = np.zeros(vocab, dtype=np.float32)
+    lg[[17, 500, 900]] = 3.0
+    assert g.sample(0.0, 0.9, logits=lg) == 17
+    lg[5] = np.nan
+    with pytest.raises(L2JError):
+        g.sample(0.9, 0.9, logits=lg)
+    lg[5] = 0.0
+    assert g.sample(0.9, 0.9, logits=lg, coin=0.0) in (17, 500, 900)   # the context stays usable
+
+
+def test_sampler_rejects_a_vocabulary_that_does_not_fit(orc):
+    g = small_transformer(40000)
+    with pytest.raises(L2JError):
+        g.sampler_seed(1)
+
+
+@pytest.mark.parametrize("shape,steps,t,topp", [
+    ((64, 128, 2, 4, 4, 512, 64, 1), 64, 1.0, 0.9),
+    ((64, 128, 2, 4, 2, 512, 64, 0), 64, 0.9, 1.0),
+    ((288, 768, 6, 6, 6, 32000, 256, 1), 72, 0.9, 0.9),
+])
+def test_decode_sample_matches_oracle_loop(orc, shape, steps, t, topp):
+    """The device loop against the reference's loop with the oracle's sampler fed the logits of l2j_forward:
+    every token must be identical.  (Against the all-CPU loop the tokens agree until a cumulative probability
+    lands within the forward pass's 1e-7 logit difference of topp or of the draw -- once in 1e2 (vocabulary 32000,
+    flat distribution) to 1e4 steps -- after which two correct samplers legitimately part ways; only the first
+    sampled tokens are asserted there.)"""
+    from tests.test_gpu_parity import make_pair
+    m, g = make_pair(orc, shape, seed=31, realistic=True)
+    prompt = orc.synth_prompt(31, 5, shape[5])
+    got, sec = g.decode_sample(prompt, steps, t, topp, 2024)
+    assert np.array_equal(got[:5], prompt) and sec > 0
+
+    g.reset()
+    s = orc.Sampler(2024, shape[5])
+    tok, want = 1, []
+    for pos in range(len(got)):                               # J/Run.java:623-685 driven from the host
+        lg = g.forward(tok, pos)
+        nxt = int(prompt[pos]) if pos < len(prompt) else s.step(lg, t, topp)[0]
+        want.append(nxt)
+        if nxt == 1:
+            break
+        tok = nxt
+    assert np.array_equal(got, np.array(want, dtype=np.int32)), (got, want)
+
+    cpu, _ = m.generate(prompt, steps, t, topp, 2024)
+    assert np.array_equal(got[:8], cpu[:8])
+
+    g.reset()
+    again, _ = g.decode_sample(prompt, steps, t, topp, 2024)
+    assert np.array_equal(again, got)                         # the seed restarts the generator and the array
+    g.reset()
+    greedy, _ = g.decode_greedy(prompt, steps)
+    g.reset()
+    same, _ = g.decode_sample(prompt, steps, 0.0, topp, 2024)
+    assert np.array_equal(same, greedy)
