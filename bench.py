@@ -76,6 +76,7 @@ def main():
     ap.add_argument("--workload", default="llama2-7b-shape", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-steps", type=int, default=13, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
+    ap.add_argument("--no-sampled", action="store_true", help="skip the extra decode with the device sampler")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
     a = ap.parse_args()
@@ -132,6 +133,22 @@ def main():
         "stream_roofline_tok_s": round(HBM_PEAK_GBS * 1e9 / bytes_tok, 1),
         "frac_of_stream_roofline": round(tok_s * bytes_tok / (HBM_PEAK_GBS * 1e9), 4),
     }
+
+    if not a.no_sampled:
+        # Not the metric: the same decode with the reference's default sampling (temperature 0.9, top-p 0.9,
+        # J/CommandLine.java:24-25) done on the device, for the cost of sampling beside the greedy figure.
+        try:
+            g.reset()
+            g.sync()
+            t0 = time.perf_counter()
+            stoks, _ = g.decode_sample(prompt, steps, 0.9, 0.9, 12345)
+            g.sync()
+            swall = time.perf_counter() - t0
+            out["sampled_decode"] = {"temperature": 0.9, "topp": 0.9, "rng_seed": 12345, "steps": int(len(stoks)),
+                                     "tok_s": round(len(stoks) / swall, 2), "ms_per_step": round(swall / len(stoks) * 1e3, 4)}
+        except l2j.L2JError as e:  # a vocabulary above the device sampler's limit
+            out["sampled_decode"] = {"error": str(e)}
+        g.reset()
 
     if a.calibrate_copy > 0:
         g.calibration_copy(a.calibrate_copy << 20, 3)

@@ -9,6 +9,7 @@ import java.lang.invoke.MethodHandle;
 import java.nio.ByteBuffer;
 
 import static java.lang.foreign.ValueLayout.ADDRESS;
+import static java.lang.foreign.ValueLayout.JAVA_FLOAT;
 import static java.lang.foreign.ValueLayout.JAVA_INT;
 import static java.lang.foreign.ValueLayout.JAVA_LONG;
 
@@ -27,7 +28,7 @@ public final class ContextHIP implements AutoCloseable {
     private final SymbolLookup lib;
     private final Arena arena = Arena.ofShared();
     private final MemorySegment ctx;
-    private final MethodHandle lastError, destroy, uploadQuant, uploadF32, finalizeH, forward, forwardArgmax;
+    private final MethodHandle lastError, destroy, uploadQuant, uploadF32, finalizeH, forward, forwardArgmax, samplerSeed, sample;
 
     private MethodHandle handle(String name, FunctionDescriptor fd) {
         return LINKER.downcallHandle(lib.find(name).orElseThrow(), fd);
@@ -42,6 +43,8 @@ public final class ContextHIP implements AutoCloseable {
         finalizeH = handle("l2j_finalize", FunctionDescriptor.of(JAVA_INT, ADDRESS));
         forward = handle("l2j_forward", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS));
         forwardArgmax = handle("l2j_forward_argmax", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS));
+        samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
+        sample = handle("l2j_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_FLOAT, JAVA_FLOAT, JAVA_FLOAT, ADDRESS));
         MethodHandle create = handle("l2j_create", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS));
 
         // l2j_config: twelve 32-bit fields
@@ -120,6 +123,24 @@ public final class ContextHIP implements AutoCloseable {
         try (Arena a = Arena.ofConfined()) {
             MemorySegment next = a.allocate(JAVA_INT);
             check(invokeInt(forwardArgmax, ctx, token, pos, next));
+            return next.get(JAVA_INT, 0);
+        }
+    }
+
+    /** = new Sampler(rngSeed, vocab_size), kept on the device. */
+    public void samplerSeed(long rngSeed) {
+        check(invokeInt(samplerSeed, ctx, rngSeed));
+    }
+
+    /**
+     * The sampling branch of Run.main (temperature, softmax, sample / sample_topp) on the logits of the last forward,
+     * without reading them back.  coin: Random.nextFloat() of the caller's own generator, or a negative value to let
+     * the device's java.util.Random (seeded by samplerSeed) draw.
+     */
+    public int sample(float temperature, float topp, float coin) {
+        try (Arena a = Arena.ofConfined()) {
+            MemorySegment next = a.allocate(JAVA_INT);
+            check(invokeInt(sample, ctx, MemorySegment.NULL, temperature, topp, coin, next));
             return next.get(JAVA_INT, 0);
         }
     }

@@ -449,7 +449,7 @@ int ensure_sampler(l2j_ctx *c)
     c->sort_temp_bytes = bytes;
     HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
-    const int lds = ((n + 7) & ~7) * (int)sizeof(float);
+    const int lds = (((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
     HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     if ((rc = dev_alloc(&c->ss, 1))) return rc;
@@ -488,7 +488,7 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     a.sorted_prob = c->pi_prob[other]; a.sorted_idx = c->pi_idx[other];
     a.st = in_loop ? c->st : nullptr;
     a.out_tokens = c->out_tokens;
-    const size_t lds = (size_t)((n + 7) & ~7) * sizeof(float);
+    const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
     hipLaunchKernelGGL(k_sample_probs, dim3(1), dim3(1024), lds, c->stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.plain) return e;

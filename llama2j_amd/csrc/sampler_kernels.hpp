@@ -4,15 +4,17 @@
 //
 // The reference adds the probabilities one by one into a float (the softmax denominator, the CDF of
 // sample, the cumulative probability of sample_topp); float addition is not associative, so those sums
-// run here as one dependent chain in a single lane (about 2.5 ns per element) and everything else
+// run here as one dependent chain in a single lane (3.4 ns per element: the eight-cycle latency of a
+// dependent v_add_f32, measured; 0.11 ms for 32000 probabilities) and everything else
 // (divide, max, exp, normalize, candidate filter, the search in the running sums) is spread over the
-// workgroup.  The probabilities live in LDS; the chain overwrites them with its running sums, stops
-// at the end of the 64-element chunk in which the sum passes the draw / topp, and the first
-// element past it is then found in parallel.
+// workgroup.  The probabilities live in LDS; the chain keeps its running sum after every 32 elements, stops
+// at the end of the step in which the sum passes the draw / topp, and the first element past it is
+// then found from those step sums.
 //
 // sample_topp sorts its whole ProbIndex array, not just the candidates of the call: entries of earlier calls
 // stay behind them and take part (J/Sampler.java:92-97).  The array therefore lives in device memory between
-// calls (SampleArgs::cand_*, sorted_*) and is sorted whole, by a stable descending radix sort on the host side.
+// calls (SampleArgs::cand_*, sorted_*) and is sorted whole by rocPRIM's stable descending sort of (key, value) pairs,
+// which the host launches between the two kernels below.
 #pragma once
 
 #include "kernels.hpp"
@@ -53,75 +55,122 @@ __device__ __forceinline__ float java_next_float(unsigned long long *rng)
     return __fdiv_rn((float)(int)(s >> 24), 16777216.0f);
 }
 
-// Running sums of p[0..n) in element order, in place, by the calling thread alone.  Stops after the
-// 64-element chunk at whose end the sum satisfies `STOP_ABOVE ? sum > limit : limit < sum`
-// (both are monotone: the terms are not negative).  Returns the number of elements summed; *total = the
-// last running sum.  p is 16-byte aligned and padded to a multiple of 8 with zeros.
-template <bool WRITE>
-__device__ __forceinline__ int chain_sums(float *p, int n, float limit, bool stop_above, bool bounded, float *total)
+// Sum of p[0..n) in element order by the calling thread alone; ends[k] (if not null) receives the running sum
+// after step k of 32 elements.  With `bounded` it stops after the step at whose end the sum satisfies
+// `stop_above ? sum > limit : limit < sum` (monotone: the terms are not negative).  Returns the number of steps
+// done; *total = the last running sum.  p is 16-byte aligned, padded to a multiple of 32 with zeros and followed by
+// one more step of readable padding.  The next
+// 32 elements are fetched from LDS while the current ones are added, and nothing but the additions and one
+// store per step is issued in between: a lone wavefront issues an instruction every four cycles or so, so
+// every instruction beside the dependent additions lengthens the chain.
+constexpr int kChainStep = 32;
+constexpr int kChainMaxSteps = kSampleMaxVocab / kChainStep;
+
+struct ChainRegs {
+    float4 v[kChainStep / 4];
+};
+
+__device__ __forceinline__ void chain_load(ChainRegs &r, const float *p)
 {
+#pragma unroll
+    for (int u = 0; u < kChainStep / 4; u++) r.v[u] = *(const float4 *)(p + 4 * u);
+}
+
+__device__ __forceinline__ float chain_step(const ChainRegs &r, float acc)
+{
+#pragma unroll
+    for (int u = 0; u < kChainStep / 4; u++) {
+        acc = __fadd_rn(acc, r.v[u].x);
+        acc = __fadd_rn(acc, r.v[u].y);
+        acc = __fadd_rn(acc, r.v[u].z);
+        acc = __fadd_rn(acc, r.v[u].w);
+    }
+    return acc;
+}
+
+template <bool ENDS>
+__device__ __forceinline__ int chain_sums(const float *p, int n, float *ends, float limit, bool stop_above, bool bounded, float *total)
+{
+    const int steps = (n + kChainStep - 1) / kChainStep;
+    ChainRegs ra, rb;
     float acc = 0.0f;
-    int i = 0;
-    const int n8 = (n + 7) & ~7;
-    while (i < n8) {
-        const int end = min(n8, i + 64);
-#pragma unroll 2
-        for (; i < end; i += 8) {
-            float4 a = *(const float4 *)(p + i), b = *(const float4 *)(p + i + 4);
-            a.x = __fadd_rn(acc, a.x);
-            a.y = __fadd_rn(a.x, a.y);
-            a.z = __fadd_rn(a.y, a.z);
-            a.w = __fadd_rn(a.z, a.w);
-            b.x = __fadd_rn(a.w, b.x);
-            b.y = __fadd_rn(b.x, b.y);
-            b.z = __fadd_rn(b.y, b.z);
-            b.w = __fadd_rn(b.z, b.w);
-            acc = b.w;
-            if (WRITE) {
-                *(float4 *)(p + i) = a;
-                *(float4 *)(p + i + 4) = b;
-            }
-        }
+    int k = 0;
+    chain_load(ra, p);
+    while (k < steps) {
+        // The loads are unconditional (hence the step of padding) and fenced: behind a branch the compiler would
+        // wait for them before it uses the older ones, and left alone it moves them down next to their use.
+        chain_load(rb, p + (k + 1) * kChainStep);
+        __builtin_amdgcn_sched_barrier(0);
+        acc = chain_step(ra, acc);
+        if (ENDS) ends[k] = acc;
+        k++;
+        if (k >= steps || (bounded && (stop_above ? acc > limit : limit < acc))) break;
+        chain_load(ra, p + (k + 1) * kChainStep);
+        __builtin_amdgcn_sched_barrier(0);
+        acc = chain_step(rb, acc);
+        if (ENDS) ends[k] = acc;
+        k++;
         if (bounded && (stop_above ? acc > limit : limit < acc)) break;
     }
     *total = acc;
-    return min(i, n);
+    return k;
 }
 
-// First index in [0, m) whose running sum s satisfies (above ? s > limit : limit < s), or m if none.
-// All threads call; `slot` is an LDS word.
-__device__ __forceinline__ int first_past(const float *sums, int m, float limit, bool above, int *slot)
+// The first element i < m (m within the `steps` steps summed) whose running sum s satisfies
+// (above ? s > limit : limit < s), found from the step-end sums: all threads look for the first step whose end
+// passes, thread 0 then walks that step.  Returns the index (m if none); *sum_at = its running sum.  All threads
+// call; slot and fslot are LDS words.
+__device__ __forceinline__ int first_past(const float *p, const float *ends, int steps, int m, float limit, bool above, int *slot,
+                                          float *fslot, float *sum_at)
 {
-    if (threadIdx.x == 0) *slot = m;
+    if (threadIdx.x == 0) *slot = steps;
     __syncthreads();
-    int best = m;
-    for (int i = threadIdx.x; i < m; i += blockDim.x) {
-        const float s = sums[i];
-        if (above ? s > limit : limit < s) { best = i; break; }   // a thread's indices ascend
+    for (int k = threadIdx.x; k < steps; k += blockDim.x) {
+        const float s = ends[k];
+        if (above ? s > limit : limit < s) {   // a thread's indices ascend
+            atomicMin(slot, k);
+            break;
+        }
     }
-    if (best < m) atomicMin(slot, best);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int k = *slot;
+        int found = m;
+        float acc = 0.0f;
+        if (k < steps) {
+            acc = k > 0 ? ends[k - 1] : 0.0f;
+            for (int i = k * kChainStep; i < min(m, (k + 1) * kChainStep); i++) {
+                acc = __fadd_rn(acc, p[i]);
+                if (above ? acc > limit : limit < acc) { found = i; break; }
+            }
+        }
+        *slot = found;
+        *fslot = acc;
+    }
     __syncthreads();
     const int r = *slot;
+    *sum_at = *fslot;
     __syncthreads();
     return r;
 }
 
 // J/Run.java:645-659 (divide by the temperature, FindMax, ExpSumNormalize), then either J/Sampler.java:33-44
-// (plain) or the candidate filter of J/Sampler.java:85-96.  One workgroup; dynamic LDS: (n rounded up to 8) floats.
+// (plain) or the candidate filter of J/Sampler.java:85-96.  One workgroup; dynamic LDS: (n rounded up to 32) + 32 floats.
 __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
 {
     extern __shared__ __align__(16) float sp[];
+    __shared__ float ends[kChainMaxSteps];
     __shared__ float red[16];
     __shared__ int cnt[1024];
-    __shared__ float s_sum, s_coin;
+    __shared__ float s_sum, s_coin, s_f;
     __shared__ int s_slot, s_m;
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
-    const int n8 = (n + 7) & ~7;
+    const int np = (n + kChainStep - 1) & ~(kChainStep - 1);
 
     // logits[q] /= temperature; max
     float mx = -__builtin_inff();
     int bad = 0;
-    for (int i = tid; i < n8; i += nt) {
+    for (int i = tid; i < np; i += nt) {
         float v = 0.0f;
         if (i < n) {
             v = __fdiv_rn(a.logits[i], a.temperature);
@@ -137,7 +186,7 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
     // sum += x, in element order
     if (tid == 0) {
         float t;
-        chain_sums<false>(sp, n, 0.0f, false, false, &t);
+        chain_sums<false>(sp, n, nullptr, 0.0f, false, false, &t);
         s_sum = t;
     }
     __syncthreads();
@@ -160,12 +209,12 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
             if (r < 0.0f) r = java_next_float(&a.ss->rng);
             s_coin = r;
             float t;
-            s_m = chain_sums<true>(sp, n, r, false, true, &t);
+            s_m = chain_sums<true>(sp, n, ends, r, false, true, &t);
         }
         __syncthreads();
-        const int m = s_m;
-        int pick = first_past(sp, m, s_coin, false, &s_slot);
-        if (pick >= m) pick = n - 1;
+        float at;
+        int pick = first_past(sp, ends, s_m, n, s_coin, false, &s_slot, &s_f, &at);
+        if (pick >= n) pick = n - 1;
         if (tid == 0) {
             a.ss->result = pick;
             if (a.st) {
@@ -201,12 +250,13 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
     if (tid == nt - 1) a.ss->n0 = cnt[tid];
 }
 
-// J/Sampler.java:99-119 on the sorted ProbIndex array.  One workgroup; dynamic LDS: (n0 rounded up to 8) floats,
+// J/Sampler.java:99-119 on the sorted ProbIndex array.  One workgroup; dynamic LDS: (n rounded up to 32) + 32 floats,
 // n0 <= n.
 __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
 {
     extern __shared__ __align__(16) float sp[];
-    __shared__ float s_cum, s_r;
+    __shared__ float ends[kChainMaxSteps];
+    __shared__ float s_cum, s_r, s_f;
     __shared__ int s_slot, s_m;
     const int tid = threadIdx.x, nt = blockDim.x;
     const int n0 = a.ss->n0;
@@ -214,28 +264,32 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
         if (tid == 0) a.ss->result = 0;
         return;
     }
-    const int n8 = (n0 + 7) & ~7;
-    for (int i = tid; i < n8; i += nt) sp[i] = i < n0 ? a.sorted_prob[i] : 0.0f;
+    const int np = (n0 + kChainStep - 1) & ~(kChainStep - 1);
+    for (int i = tid; i < np; i += nt) sp[i] = i < n0 ? a.sorted_prob[i] : 0.0f;
     __syncthreads();
     // cumulative_prob += prob until it exceeds topp
     if (tid == 0) {
         float t;
-        s_m = chain_sums<true>(sp, n0, a.topp, true, true, &t);
+        s_m = chain_sums<true>(sp, n0, ends, a.topp, true, true, &t);
         s_cum = t;
     }
     __syncthreads();
-    const int m = s_m;
-    int last = first_past(sp, m, a.topp, true, &s_slot);
-    if (last >= m) last = n0 - 1;   // never exceeded: all candidates, cumulative_prob = their sum
+    const int steps = s_m;
+    float cum;
+    int last = first_past(sp, ends, steps, n0, a.topp, true, &s_slot, &s_f, &cum);
+    if (last >= n0) {   // never exceeded: all candidates, cumulative_prob = their sum
+        last = n0 - 1;
+        cum = s_cum;
+    }
     if (tid == 0) {
-        const float cum = last < m ? sp[last] : s_cum;
         float coin = a.coin;
         if (coin < 0.0f) coin = java_next_float(&a.ss->rng);
         s_r = __fmul_rn(coin, cum);
     }
     __syncthreads();
     // the first i <= last_idx with r < cdf(i), else last_idx
-    int pick = first_past(sp, last + 1, s_r, false, &s_slot);
+    float at;
+    int pick = first_past(sp, ends, min(steps, last / kChainStep + 1), last + 1, s_r, false, &s_slot, &s_f, &at);
     if (pick > last) pick = last;
     if (tid == 0) {
         const int token = a.sorted_idx[pick];
