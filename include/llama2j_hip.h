@@ -141,6 +141,23 @@ int l2j_sample(l2j_ctx *ctx, const float *logits_or_null, float temperature, flo
 int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature,
                       float topp, int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds);
 
+/* ---- tokenizer: J/Tokenizer.java (host only) ----
+ * Strings cross the boundary as NUL-terminated UTF-8; inside, comparisons are on UTF-16 code units as in Java. */
+typedef struct l2j_tokenizer l2j_tokenizer;
+/* = new Tokenizer(path, vocabSize) (J/Tokenizer.java:61-90): LE int32 max_token_length (ignored), then per token
+ * LE fp32 score, LE int32 length, UTF-8 bytes. */
+int l2j_tokenizer_open(const char *path, int32_t vocab_size, l2j_tokenizer **out);
+void l2j_tokenizer_close(l2j_tokenizer *tok);
+/* = bpe_encode (J/Tokenizer.java:102-163): dummy-prefix blank, per-character lookup with byte fallback, then the best
+ * scoring merge until none applies.  *n gets the token count (also when cap is too small: L2J_E_SIZE).  Where the
+ * reference throws ArrayIndexOutOfBoundsException (its byte fallback gives negative ids for bytes above 0x7f), this
+ * returns L2J_E_ARG. */
+int l2j_bpe_encode(l2j_tokenizer *tok, const char *prompt_utf8, int32_t *tokens, int32_t cap, int32_t *n);
+/* = bpe_decode(token, next) (J/Tokenizer.java:189-208): the blank after BOS stripped, raw byte tokens "<0xNN>" as one
+ * Latin-1 character or nothing for control codes.  *len = bytes written before the NUL, or -1 where the reference
+ * returns null. */
+int l2j_bpe_decode(l2j_tokenizer *tok, int32_t token, int32_t next, char *out_utf8, int32_t cap, int32_t *len);
+
 /* Activation / cache taps.  layer < 0 reads the live buffer, layer >= 0 the per-layer tap.
  * `off` and `n` are in floats. */
 int l2j_read(l2j_ctx *ctx, int which, int layer, uint64_t off, float *dst, uint64_t n);

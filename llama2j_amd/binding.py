@@ -117,6 +117,10 @@ def _signatures():
         "l2j_read_checkpoint_header": (C.c_int, [C.c_char_p, cfgp]),
         "l2j_load_checkpoint": (C.c_int, [C.c_char_p, C.c_int, C.c_uint32, C.c_int, C.POINTER(vp)]),
         "l2j_get_config": (C.c_int, [vp, cfgp]),
+        "l2j_tokenizer_open": (C.c_int, [C.c_char_p, C.c_int32, C.POINTER(vp)]),
+        "l2j_tokenizer_close": (None, [vp]),
+        "l2j_bpe_encode": (C.c_int, [vp, C.c_char_p, i32p, C.c_int32, i32p]),
+        "l2j_bpe_decode": (C.c_int, [vp, C.c_int32, C.c_int32, C.c_char_p, C.c_int32, i32p]),
     }
 
 
@@ -213,6 +217,40 @@ class Sampler:
     @staticmethod
     def argmax(logits):
         return int(np.argmax(np.asarray(logits)))  # numpy also returns the first maximum
+
+
+class Tokenizer:
+    """J/Tokenizer.java: tokenizer.bin reader, bpe_encode, bpe_decode (host code inside the library)."""
+
+    def __init__(self, tokenizerFilePath, vocabSize):
+        h = C.c_void_p()
+        _check(lib().l2j_tokenizer_open(os.fsencode(tokenizerFilePath), vocabSize, C.byref(h)))
+        self._h = h
+
+    def bpe_encode(self, prompt):
+        raw = prompt.encode("utf-8", "surrogatepass") if isinstance(prompt, str) else bytes(prompt)
+        cap = 2 * len(raw) + 2
+        out = np.zeros(cap, dtype=np.int32)
+        n = C.c_int32(0)
+        _check(lib().l2j_bpe_encode(self._h, raw, _i32(out), cap, C.byref(n)))
+        return out[:n.value].copy()
+
+    def bpe_decode(self, token, next):
+        buf = C.create_string_buffer(1 << 16)
+        n = C.c_int32(0)
+        _check(lib().l2j_bpe_decode(self._h, token, next, buf, len(buf), C.byref(n)))
+        return None if n.value < 0 else buf.raw[:n.value].decode("utf-8")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().l2j_tokenizer_close(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Transformer:
