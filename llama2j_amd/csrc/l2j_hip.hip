@@ -433,12 +433,25 @@ uint64_t quant_bytes_of(uint64_t weights) { return (weights / kGroup) * kGroupBy
 
 // ---- device sampler ------------------------------------------------------------------------------------
 
-int ensure_sampler(l2j_ctx *c)
+void free_sampler(l2j_ctx *c)
 {
-    if (c->ss) return L2J_OK;
+    (void)hipFree(c->ss);
+    c->ss = nullptr;
+    for (int i = 0; i < 2; i++) {
+        (void)hipFree(c->pi_prob[i]);
+        (void)hipFree(c->pi_idx[i]);
+        c->pi_prob[i] = nullptr;
+        c->pi_idx[i] = nullptr;
+    }
+    (void)hipFree(c->sort_temp);
+    c->sort_temp = nullptr;
+    if (c->h_ss) (void)hipHostFree(c->h_ss);
+    c->h_ss = nullptr;
+}
+
+int alloc_sampler(l2j_ctx *c)
+{
     const int n = c->cfg.vocab_size;
-    if (n > kSampleMaxVocab) return fail(L2J_E_SIZE, "device sampler: vocab_size above 36864 does not fit the LDS");
-    if (n < 2) return fail(L2J_E_SIZE, "device sampler: vocab_size below 2");
     int rc;
     for (int i = 0; i < 2; i++) {
         if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n))) return rc;
@@ -452,8 +465,18 @@ int ensure_sampler(l2j_ctx *c)
     const int lds = (((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
     HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    if ((rc = dev_alloc(&c->ss, 1))) return rc;
-    return L2J_OK;
+    return dev_alloc(&c->ss, 1);   // last: its presence says that the sampler is complete
+}
+
+int ensure_sampler(l2j_ctx *c)
+{
+    if (c->ss) return L2J_OK;
+    const int n = c->cfg.vocab_size;
+    if (n > kSampleMaxVocab) return fail(L2J_E_SIZE, "device sampler: vocab_size above 36864 does not fit the LDS");
+    if (n < 2) return fail(L2J_E_SIZE, "device sampler: vocab_size below 2");
+    const int rc = alloc_sampler(c);
+    if (rc) free_sampler(c);
+    return rc;
 }
 
 // new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31): Random(seed) scrambles its seed, every ProbIndex is (0, 0)
@@ -499,6 +522,17 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     c->pi_cur = other;
     hipLaunchKernelGGL(k_topp_pick, dim3(1), dim3(1024), lds, c->stream, a);
     return hipGetLastError();
+}
+
+// After a synchronize with h_ss read back: the reference's exceptions as an error return; the flag is cleared.
+int check_sampler_status(l2j_ctx *c)
+{
+    const int st = c->h_ss->nan;
+    if (!st) return L2J_OK;
+    c->h_ss->nan = 0;
+    HIPCHK(hipMemcpy(&c->ss->nan, &c->h_ss->nan, sizeof(int), hipMemcpyHostToDevice));
+    if (st & 1) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
+    return fail(L2J_E_ARG, "sampler: no probability reaches the top-p cutoff (ArrayIndexOutOfBoundsException at J/Sampler.java:119)");
 }
 
 int check_sampler_args(float temperature, float topp)
@@ -552,7 +586,7 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
         if (sampled) HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
         HIPCHK(hipStreamSynchronize(c->stream));
         if ((rc = check_barrier_error(c))) return rc;
-        if (sampled && c->h_ss->nan) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
+        if (sampled && (rc = check_sampler_status(c))) return rc;
         int used = nb;
         for (int i = 0; i < nb; i++) {
             out_tokens[pos + i] = c->h_tokens[i];
@@ -704,13 +738,7 @@ void l2j_destroy(l2j_ctx *c)
     (void)hipFree(c->out_tokens);
     (void)hipFree(c->bar_ctr);
     (void)hipFree(c->fault);
-    (void)hipFree(c->ss);
-    for (int i = 0; i < 2; i++) {
-        (void)hipFree(c->pi_prob[i]);
-        (void)hipFree(c->pi_idx[i]);
-    }
-    (void)hipFree(c->sort_temp);
-    if (c->h_ss) (void)hipHostFree(c->h_ss);
+    free_sampler(c);
     if (c->h_fault) (void)hipHostFree(c->h_fault);
     for (float *t : c->taps) (void)hipFree(t);
     if (c->h_st) (void)hipHostFree(c->h_st);
@@ -1078,11 +1106,7 @@ int l2j_sample(l2j_ctx *c, const float *logits, float temperature, float topp, f
     }
     HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
     HIPCHK(hipStreamSynchronize(c->stream));
-    if (c->h_ss->nan) {
-        c->h_ss->nan = 0;
-        HIPCHK(hipMemcpy(&c->ss->nan, &c->h_ss->nan, sizeof(int), hipMemcpyHostToDevice));
-        return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
-    }
+    if ((rc = check_sampler_status(c))) return rc;
     *next = c->h_ss->result;
     return L2J_OK;
 }

@@ -27,7 +27,7 @@ constexpr unsigned long long kJavaRandMult = 0x5DEECE66DULL, kJavaRandMask = (1U
 struct SamplerState {        // the reference's Sampler object, device resident
     unsigned long long rng;  // java.util.Random's 48-bit state
     int n0;                  // candidates of the current sample_topp call
-    int nan;                 // a NaN among the probabilities (J/Sampler.java:88-90 throws)
+    int nan;                 // bit 0: a NaN among the probabilities (J/Sampler.java:88-90 throws); bit 1: no top-p candidate
     int result;              // the token of the last call
     int pad;
 };
@@ -199,7 +199,7 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
         sp[i] = v;
         a.logits[i] = v;
     }
-    if (bad) a.ss->nan = 1;
+    if (bad) atomicOr(&a.ss->nan, 1);
     __syncthreads();
 
     if (a.plain) {
@@ -260,8 +260,11 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
     __shared__ int s_slot, s_m;
     const int tid = threadIdx.x, nt = blockDim.x;
     const int n0 = a.ss->n0;
-    if (n0 <= 0) {   // only with NaN probabilities; the host reports the call as failed
-        if (tid == 0) a.ss->result = 0;
+    if (n0 <= 0) {   // no probability reaches the cutoff (NaNs, or topp near 0 on a flat distribution): the reference
+        if (tid == 0) {   // indexes probIndex[-1] and throws; the host reports the call as failed
+            a.ss->result = 0;
+            a.ss->nan |= 2;
+        }
         return;
     }
     const int np = (n0 + kChainStep - 1) & ~(kChainStep - 1);

@@ -871,6 +871,7 @@ static int topp_pick(orc_sampler *s, const float *probs, int n, float topp, int 
         }
     }
     sort_prob_index(s);                             /* :97 : the whole array */
+    if (n0 == 0) return -2;                         /* :101,119 : probIndex[-1], ArrayIndexOutOfBoundsException */
     float cumulative_prob = 0.0f;
     int last_idx = n0 - 1;
     for (int i = 0; i < n0; i++) {
@@ -884,7 +885,7 @@ static int topp_pick(orc_sampler *s, const float *probs, int n, float topp, int 
         cdf += s->prob[i];
         if (r < cdf) return s->index[i];
     }
-    return s->index[last_idx];   /* n0 == 0 would index -1 in the reference (an exception); callers avoid it */
+    return s->index[last_idx];
 }
 
 int orc_sample_topp(orc_sampler *s, const float *probs, int n, float topp)

@@ -118,7 +118,8 @@ int32_t orc_sampler_next_bits(orc_sampler *s, int bits);            /* java.util
 float orc_sampler_next_float(orc_sampler *s);                       /* J/Sampler.java:20-22 */
 int orc_sample(orc_sampler *s, const float *probs, int n);          /* J/Sampler.java:33-44 */
 /* J/Sampler.java:76-120, including its whole-array sort: entries beyond the candidates of this call
- * keep what earlier calls left there and take part in the sort.  Returns -1 for a NaN (the reference throws). */
+ * keep what earlier calls left there and take part in the sort.  Returns -1 for a NaN and -2 when no probability
+ * reaches the cutoff (the reference throws in both cases). */
 int orc_sample_topp(orc_sampler *s, const float *probs, int n, float topp);
 /* The same two with the random draw given by the caller instead of taken from the generator. */
 int orc_sample_coin(const float *probs, int n, float coin);

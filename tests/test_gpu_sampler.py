@@ -91,6 +91,9 @@ def test_temperature_zero_is_first_max_and_nan_is_an_error(orc):
         g.sample(0.9, 0.9, logits=lg)
     lg[5] = 0.0
     assert g.sample(0.9, 0.9, logits=lg, coin=0.0) in (17, 500, 900)   # the context stays usable
+    with pytest.raises(L2JError):                                      # flat distribution, topp 0: no candidate
+        g.sample(1.0, 0.0, logits=np.zeros(vocab, dtype=np.float32))
+    assert g.sample(1.0, 0.0, logits=lg, coin=0.9) == 17               # ties keep index order; cumulative > 0 at once
 
 
 def test_sampler_rejects_a_vocabulary_that_does_not_fit(orc):

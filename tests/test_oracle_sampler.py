@@ -167,6 +167,13 @@ def test_topp_nan_is_an_error(orc):
     assert orc.Sampler(1, 3).sample_topp(p, 0.9, coin=0.5) == -1
 
 
+def test_topp_without_candidates_is_an_error(orc):
+    # topp 0: cutoff = 1 / (n - 1), above every probability of a flat distribution -> probIndex[-1] in the reference
+    p = np.full(4, 0.25, dtype=np.float32)
+    assert orc.Sampler(1, 4).sample_topp(p, 0.0, coin=0.5) == -2
+    assert orc.Sampler(1, 4).sample_topp(np.array([0.4, 0.2, 0.2, 0.2], dtype=np.float32), 0.0, coin=0.5) == 0
+
+
 # ---------------------------------------------------------------- the step of J/Run.java:643-665
 
 def test_step_softmax_and_branches(orc):
