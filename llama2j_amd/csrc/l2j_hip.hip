@@ -185,7 +185,7 @@ int attn_lpr(const l2j_ctx *c) { return c->head_size <= 64 ? 16 : c->head_size <
 size_t attn_smem_for(const l2j_ctx *c, int threads)
 {
     const int nent = (threads / 64) * (64 / attn_lpr(c));
-    return (size_t)(2 * nent + nent * c->head_size + 1) * sizeof(float);
+    return (size_t)(3 * nent + nent * c->head_size + 2) * sizeof(float);
 }
 
 size_t attn_smem(const l2j_ctx *c) { return attn_smem_for(c, c->attn_threads); }
@@ -234,6 +234,12 @@ bool geom_complete(const TokenGeom &t)
     return true;
 }
 
+// Splits per attention head inside k_token: one (head, split) item per workgroup at most.
+int fused_splits(const l2j_ctx *c)
+{
+    return std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
+}
+
 // Marks every activation vector of a token unwritten (before a k_token that hands over by value).
 hipError_t launch_fill_unset(const l2j_ctx *c, hipStream_t s)
 {
@@ -263,7 +269,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.g = c->geom;
     a.l0 = l0; a.l1 = l1; a.with_cls = l1 == c->cfg.n_layers;
     a.attn_rows = c->fused_attn_rows;
-    a.attn_splits = std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
+    a.attn_splits = fused_splits(c);
     a.maxspin = c->barrier_spins;
     a.by_value = c->by_value ? 1 : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);

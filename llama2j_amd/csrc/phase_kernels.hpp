@@ -87,6 +87,32 @@ __device__ __forceinline__ float wait_float(const float *p, const Poll &pl)
     return v;
 }
 
+// Several 16-byte words at once: all are requested before the one wait, so the words cost one trip to memory
+// together instead of one each.  (Loads and wait are one asm statement: the compiler must not touch the
+// destination registers in between.)  Words that are still unset are requested again, with the others: a few
+// redundant loads are cheaper than divergent bookkeeping.
+__device__ __forceinline__ void load_words(const float *const (&p)[3], float4 (&v)[3])
+{
+    asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"
+                 "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_words(const float *const (&p)[N], float4 (&v)[N], const Poll &pl)
+{
+    int spins = 0;
+    while (true) {
+        load_words(p, v);
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < N; i++) ok = ok && all_set(v[i]);
+        if (ok) break;
+        if (++spins > pl.maxspin || ((spins & 63) == 0 && ld_coh(pl.fault) != 0)) { st_coh(pl.fault, 1); break; }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
+
 // ---- grid barrier ------------------------------------------------------------------------------------
 // Two levels of relaxed device-scope counters: a workgroup bumps the counter of its group (blockIdx % ngroups),
 // the last of a group bumps the top counter, everybody polls the top counter.  Every barrier instance of a
@@ -269,6 +295,15 @@ __device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin,
         }
     }
     __syncthreads();
+}
+
+// The number of splits per head the attention phase uses at a position, and the rows of each.
+__device__ __forceinline__ int attn_splits_at(int len, int rows_per_split, int max_splits, int &chunk)
+{
+    int nsplit = (len + rows_per_split - 1) / rows_per_split;  // short contexts: fewer, fuller splits
+    if (nsplit > max_splits) nsplit = max_splits;
+    chunk = (len + nsplit - 1) / nsplit;
+    return (len + chunk - 1) / chunk;
 }
 
 // ---- W8A32 matvec: an item is a pair of rows, one wavefront per item ---------------------------------
@@ -569,10 +604,7 @@ struct AttnRun {
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         nent = W * RPW;
         len = pos + 1;
-        int nsplit = (len + a.rows_per_split - 1) / a.rows_per_split;  // short contexts: fewer, fuller splits
-        if (nsplit > a.max_splits) nsplit = a.max_splits;
-        chunk = (len + nsplit - 1) / nsplit;
-        nact = (len + chunk - 1) / chunk;
+        nact = attn_splits_at(len, a.rows_per_split, a.max_splits, chunk);
         j = lane % LPR;
         slot = wave * RPW + lane / LPR;
         active = 4 * j < hs;
@@ -618,7 +650,7 @@ struct AttnRun {
         }
     }
 
-    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int.  COH as for the matvec phases (the partials of
+    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int, nent + 1 floats (weights).  COH as for the matvec phases (the partials of
     // a split always travel write-through: other workgroups of the same launch read them).
     template <bool COH>
     __device__ __forceinline__ void run(float *smem)
@@ -627,12 +659,38 @@ struct AttnRun {
         float *sm_l = sm_m + nent;    // nent
         float *sm_acc = sm_l + nent;  // nent * hs
         int &s_last = *reinterpret_cast<int *>(sm_acc + nent * hs);
+        float *sm_w = sm_acc + nent * hs + 1;  // nent + 1: the slots' weights, then their common maximum
 
         for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
             const int h = it % a.n_heads, s = it / a.n_heads;
             const int t0 = s * chunk, t1 = min(len, t0 + chunk);
             float4 q4 = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (active) q4 = a.poll.on ? wait_word(a.q + h * hs + 4 * j, a.poll) : *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
+            bool kv_done = false;  // this token's k and v row arrived together with q
+            if (active && a.poll.on) {
+                // with preloaded cache rows only this position's row is missing: if it is one of this lane group's
+                // rows, wait for q, k and v in one trip to memory instead of three
+                int ucur = -1;
+                if (early && it == (int)blockIdx.x) {
+#pragma unroll
+                    for (int u = 0; u < kAU; u++)
+                        if (t0 + slot + u * nent == len - 1) ucur = u;
+                }
+                if (ucur >= 0) {
+                    const long col = (long)(h / a.kv_mul) * hs + 4 * j;
+                    const float *pp[3] = {a.q + h * hs + 4 * j, a.knew + col, a.vnew + col};
+                    float4 vv[3];
+                    wait_words(pp, vv, a.poll);
+                    q4 = vv[0];
+#pragma unroll
+                    for (int u = 0; u < kAU; u++)
+                        if (u == ucur) { k4[u] = vv[1]; v4[u] = vv[2]; }
+                    kv_done = true;
+                } else {
+                    q4 = wait_word(a.q + h * hs + 4 * j, a.poll);
+                }
+            } else if (active) {
+                q4 = *reinterpret_cast<const float4 *>(a.q + h * hs + 4 * j);
+            }
             float m = -3.402823466e+38f, l = 0.0f;
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
             for (int tb = t0 + slot; tb < t1; tb += nent * kAU) {
@@ -640,7 +698,7 @@ struct AttnRun {
 #pragma unroll
                 for (int u = 0; u < kAU; u++) ok[u] = tb + u * nent < t1;
                 if (early && it == (int)blockIdx.x && tb == t0 + slot) {
-                    fetch(h, tb, t1, 2);  // only the row of this position is still missing
+                    if (!kv_done) fetch(h, tb, t1, 2);  // only the row of this position is still missing
                 } else {
                     clear();
                     fetch(h, tb, t1, 0);
@@ -673,12 +731,21 @@ struct AttnRun {
             if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
             if (active) *reinterpret_cast<float4 *>(sm_acc + slot * hs + 4 * j) = acc;
             __syncthreads();
-            // fold the row slots in a fixed order, so the result does not depend on timing
-            float M = -3.402823466e+38f, L = 0.0f, o = 0.0f;
-            for (int e = 0; e < nent; e++) M = fmaxf(M, sm_m[e]);
+            // Fold the row slots in a fixed order, so the result does not depend on timing.  The slots' weights
+            // exp(m_e - M) come from one lane each (at most 64 slots); the fold itself then only reads LDS.
+            if (tid < 64) {
+                const float me = tid < nent ? sm_m[tid] : -3.402823466e+38f;
+                const float mx = wave_max(me);
+                if (tid < nent) sm_w[tid] = expf(me - mx);  // empty slots: exp(-huge) = 0
+                if (tid == 0) sm_w[nent] = mx;
+            }
+            __syncthreads();
+            const float M = sm_w[nent];
+            float L = 0.0f, o = 0.0f;
             if (tid < hs) {
+#pragma unroll 8
                 for (int e = 0; e < nent; e++) {
-                    const float w = expf(sm_m[e] - M);  // empty slots: exp(-huge) = 0
+                    const float w = sm_w[e];
                     L = fmaf(sm_l[e], w, L);
                     o = fmaf(sm_acc[e * hs + tid], w, o);
                 }
