@@ -185,7 +185,7 @@ int attn_lpr(const l2j_ctx *c) { return c->head_size <= 64 ? 16 : c->head_size <
 size_t attn_smem_for(const l2j_ctx *c, int threads)
 {
     const int nent = (threads / 64) * (64 / attn_lpr(c));
-    return (size_t)(3 * nent + nent * c->head_size + 2) * sizeof(float);
+    return (size_t)(3 * nent + 4 + nent * c->head_size + 1) * sizeof(float);
 }
 
 size_t attn_smem(const l2j_ctx *c) { return attn_smem_for(c, c->attn_threads); }

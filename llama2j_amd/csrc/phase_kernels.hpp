@@ -98,6 +98,29 @@ __device__ __forceinline__ void load_words(const float *const (&p)[3], float4 (&
                  : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
 }
 
+// Eight device-coherent loads at byte offsets off[] from one uniform base, one wait (4 or 8 bytes each).
+__device__ __forceinline__ void load8_coh(const float *base, const unsigned (&off)[8], float (&v)[8])
+{
+    asm volatile("global_load_dword %0, %8, %16 sc1\n\tglobal_load_dword %1, %9, %16 sc1\n\t"
+                 "global_load_dword %2, %10, %16 sc1\n\tglobal_load_dword %3, %11, %16 sc1\n\t"
+                 "global_load_dword %4, %12, %16 sc1\n\tglobal_load_dword %5, %13, %16 sc1\n\t"
+                 "global_load_dword %6, %14, %16 sc1\n\tglobal_load_dword %7, %15, %16 sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+                 : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]), "s"(base)
+                 : "memory");
+}
+
+__device__ __forceinline__ void load8_coh(const float *base, const unsigned (&off)[8], float2 (&v)[8])
+{
+    asm volatile("global_load_dwordx2 %0, %8, %16 sc1\n\tglobal_load_dwordx2 %1, %9, %16 sc1\n\t"
+                 "global_load_dwordx2 %2, %10, %16 sc1\n\tglobal_load_dwordx2 %3, %11, %16 sc1\n\t"
+                 "global_load_dwordx2 %4, %12, %16 sc1\n\tglobal_load_dwordx2 %5, %13, %16 sc1\n\t"
+                 "global_load_dwordx2 %6, %14, %16 sc1\n\tglobal_load_dwordx2 %7, %15, %16 sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+                 : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]), "s"(base)
+                 : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_words(const float *const (&p)[N], float4 (&v)[N], const Poll &pl)
 {
@@ -650,16 +673,16 @@ struct AttnRun {
         }
     }
 
-    // smem: 2*nent floats (max, sum), nent*hs floats (acc), 1 int, nent + 1 floats (weights).  COH as for the matvec phases (the partials of
+    // smem: 3*nent + 4 floats (max, sum, weights), nent*hs floats (acc), 1 int.  COH as for the matvec phases (the partials of
     // a split always travel write-through: other workgroups of the same launch read them).
     template <bool COH>
     __device__ __forceinline__ void run(float *smem)
     {
         float *sm_m = smem;           // nent
         float *sm_l = sm_m + nent;    // nent
-        float *sm_acc = sm_l + nent;  // nent * hs
+        float *sm_w = sm_l + nent;    // nent + 4: the slots' weights, then their common maximum (and padding)
+        float *sm_acc = sm_w + nent + 4;  // nent * hs
         int &s_last = *reinterpret_cast<int *>(sm_acc + nent * hs);
-        float *sm_w = sm_acc + nent * hs + 1;  // nent + 1: the slots' weights, then their common maximum
 
         for (int it = blockIdx.x; it < nitems; it += gridDim.x) {
             const int h = it % a.n_heads, s = it / a.n_heads;
@@ -743,11 +766,21 @@ struct AttnRun {
             const float M = sm_w[nent];
             float L = 0.0f, o = 0.0f;
             if (tid < hs) {
-#pragma unroll 8
-                for (int e = 0; e < nent; e++) {
+                // four slots per step: the LDS reads of a step are issued together, the additions keep slot order
+                const float *ap = sm_acc + tid;
+                int e = 0;
+                for (; (nent & 3) == 0 && e < nent; e += 4) {  // (16-byte LDS reads need nent % 4 == 0)
+                    const float4 w4 = *reinterpret_cast<const float4 *>(sm_w + e), l4 = *reinterpret_cast<const float4 *>(sm_l + e);
+                    const float a0 = ap[(e + 0) * hs], a1 = ap[(e + 1) * hs], a2 = ap[(e + 2) * hs], a3 = ap[(e + 3) * hs];
+                    L = fmaf(l4.x, w4.x, L); o = fmaf(a0, w4.x, o);
+                    L = fmaf(l4.y, w4.y, L); o = fmaf(a1, w4.y, o);
+                    L = fmaf(l4.z, w4.z, L); o = fmaf(a2, w4.z, o);
+                    L = fmaf(l4.w, w4.w, L); o = fmaf(a3, w4.w, o);
+                }
+                for (; e < nent; e++) {
                     const float w = sm_w[e];
                     L = fmaf(sm_l[e], w, L);
-                    o = fmaf(sm_acc[e * hs + tid], w, o);
+                    o = fmaf(ap[e * hs], w, o);
                 }
             }
             if (nact == 1) {
@@ -772,14 +805,20 @@ struct AttnRun {
             if (tid < hs) {
                 float MM = -3.402823466e+38f, LL = 0.0f, oo = 0.0f;
                 for (int i0 = 0; i0 < nact; i0 += 8) {
+                    // the (maximum, sum) pairs and this thread's element of eight partials: two trips to memory
                     float pm[8], pl[8], po[8];
+                    float2 ml[8];
+                    unsigned off[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) off[i] = (unsigned)(min(i0 + i, nact - 1) * (hs + 2)) * 4u;
+                    load8_coh(hp, off, ml);
 #pragma unroll
                     for (int i = 0; i < 8; i++) {
-                        const float *pp = hp + (long)min(i0 + i, nact - 1) * (hs + 2);
-                        pm[i] = ld_coh(pp);
-                        pl[i] = ld_coh(pp + 1);
-                        po[i] = ld_coh(pp + 2 + tid);
+                        pm[i] = ml[i].x;
+                        pl[i] = ml[i].y;
+                        off[i] += (unsigned)(2 + tid) * 4u;
                     }
+                    load8_coh(hp, off, po);
                     float mb = MM;
 #pragma unroll
                     for (int i = 0; i < 8; i++)
