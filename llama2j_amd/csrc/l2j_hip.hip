@@ -303,8 +303,9 @@ hipError_t launch_class(const l2j_ctx *c, int kclass, int l, hipStream_t s, hipE
     case L2J_K_WO:
     case L2J_K_W2: {
         const int n = kclass == L2J_K_WO ? c->cfg.dim : c->cfg.hidden_dim;
-        if (row_mode(n))  // long rows: one row per wave keeps every wave busy
-            return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
+        const int mode = row_mode(n);  // long rows: one row per wave keeps every wave busy
+        if (mode == PH_ROW6) return launch1(k_matvec<PH_ROW6>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
+        if (mode == PH_ROW) return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
         return launch1(k_matvec<PH_RES>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
     }
     case L2J_K_ATTENTION: {
@@ -954,6 +955,7 @@ int l2j_finalize(l2j_ctx *c)
         if (need > 64 * 1024) {
             const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
                                 reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
+                                reinterpret_cast<const void *>(k_matvec<PH_ROW6>),
                                 reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
                                 reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>)};
             for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));

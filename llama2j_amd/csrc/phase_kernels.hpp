@@ -190,7 +190,7 @@ __device__ __forceinline__ int phase_tid()
     return t;
 }
 
-enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2, PH_ROW = 3 };  // PH_RES: row pairs + residual; PH_ROW: one row per wave + residual
+enum { PH_QKV = 0, PH_W13 = 1, PH_RES = 2, PH_ROW = 3, PH_ROW6 = 4 };  // PH_RES: row pairs + residual; PH_ROW, PH_ROW6: one row per wave + residual
 
 // One matvec phase.  Passed by value.
 struct MatvecPhase {
@@ -339,8 +339,14 @@ constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
 template <int MODE>
 struct MatvecRun {
     // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
-    static constexpr int kStep = MODE == PH_ROW ? 2 * 64 * kTU : 64 * kTU;
-    static constexpr int kOff1 = MODE == PH_ROW ? 64 * kTU : 0;
+    // PH_ROW6 holds six chunks per lane and sub-row instead of four: a row of 513..768 chunks (11008 codes are 688) is
+    // then one step, requested whole ahead of the hand-over, where PH_ROW would request its tail only after the first
+    // step (1.72 -> 1.70 ms per 7B token; for shorter or longer rows the extra registers and masked loads cost more
+    // than they gain: 3.24 -> 3.60 ms per 13B token).
+    static constexpr bool kRow = MODE == PH_ROW || MODE == PH_ROW6;
+    static constexpr int TU = MODE == PH_ROW6 ? 6 : kTU;
+    static constexpr int kStep = kRow ? 2 * 64 * TU : 64 * TU;
+    static constexpr int kOff1 = kRow ? 64 * TU : 0;
 
     const MatvecPhase d;
     int n, nch, lane, W, G, nitems, item;
@@ -351,8 +357,8 @@ struct MatvecRun {
     int which = 0, r = 0;
     bool has1 = true, first = false;
     int wave = 0;
-    uint4 w0[kTU], w1[kTU];
-    float2 s0[kTU], s1[kTU];
+    uint4 w0[TU], w1[TU];
+    float2 s0[TU], s1[TU];
 
     __device__ __forceinline__ MatvecRun(const MatvecPhase &d_) : d(d_)
     {
@@ -406,7 +412,7 @@ struct MatvecRun {
     __device__ __forceinline__ void issue(int base)
     {
 #pragma unroll
-        for (int u = 0; u < kTU; u++) {
+        for (int u = 0; u < TU; u++) {
             const int c = base + 64 * u + lane, c1 = c + kOff1;
             const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 below)
             const unsigned cc1 = c1 < nch ? c1 : nch - 1;
@@ -422,7 +428,7 @@ struct MatvecRun {
     __device__ __forceinline__ void zero()
     {
 #pragma unroll
-        for (int u = 0; u < kTU; u++) {
+        for (int u = 0; u < TU; u++) {
             w0[u] = w1[u] = make_uint4(0u, 0u, 0u, 0u);
             s0[u] = s1[u] = make_float2(0.f, 0.f);
         }
@@ -462,7 +468,7 @@ struct MatvecRun {
     __device__ __forceinline__ void residual(const float *res, float &resv0, float &resv1)
     {
         resv0 = resv1 = 0.0f;
-        if ((MODE == PH_RES || MODE == PH_ROW) && lane == 0) {
+        if ((MODE == PH_RES || kRow) && lane == 0) {
             if (d.poll.on && !d.res_emb) {  // a line of the vector may have been cached while it was half written
                 resv0 = wait_float(res + r, d.poll);
                 if (MODE == PH_RES && has1) resv1 = wait_float(res + r + 1, d.poll);
@@ -477,7 +483,7 @@ struct MatvecRun {
     __device__ __forceinline__ void fold(int base, const float4 *xs, const float *sumx, float &acc0, float &acc1)
     {
 #pragma unroll
-        for (int u = 0; u < kTU; u++) {
+        for (int u = 0; u < TU; u++) {
             const uint4 a0 = w0[u], a1 = w1[u];
             const float2 g0 = s0[u], g1 = s1[u];
             const int c = base + 64 * u + lane;
@@ -487,7 +493,7 @@ struct MatvecRun {
             const float sx = sumx[cc];
             const float t0 = fmaf(g0.x, dot16(a0, x0, x1, x2, x3), g0.y * sx);
             acc0 += ok ? t0 : 0.0f;
-            if (MODE == PH_ROW) {
+            if (kRow) {
                 const int c1 = c + kOff1;
                 const bool ok1 = c1 < nch;
                 const int cc1 = ok1 ? c1 : nch - 1;
@@ -1070,7 +1076,12 @@ __host__ __device__ inline ClsPhase cls_phase_of(const G &g, int nparts)
 }
 
 // Long rows are streamed one row per wave (PH_ROW) so every wave has work; shorter ones as row pairs (PH_RES).
-__host__ __device__ inline bool row_mode(int n) { return n / 16 > 64 * kTU; }
+// The mode of a matvec + residual phase for rows of n codes: pairs of rows while a row fits one step of a sub-row.
+__host__ __device__ inline int row_mode(int n)
+{
+    const int nch = n / 16;
+    return nch <= 64 * kTU ? PH_RES : nch > 2 * 64 * kTU && nch <= 2 * 64 * 6 ? PH_ROW6 : PH_ROW;
+}
 
 struct TokenArgs {
     TokenGeom g;
@@ -1170,7 +1181,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     TokenArgsPtr t = token_args();
     const int token = t->g.st->token, pos = t->g.st->pos;
     const int l0 = t->l0, l1 = t->l1;
-    const bool wo_row = row_mode(t->g.dim), w2_row = row_mode(t->g.hidden);
+    const int wo_mode = row_mode(t->g.dim), w2_mode = row_mode(t->g.hidden);
     GridBar b;
     b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
     for (int l = l0; l < l1; l++) {
@@ -1189,14 +1200,16 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
-        if (wo_row) token_wo<PH_ROW>(b, l, smem4, token, pos);
+        if (wo_mode == PH_ROW6) token_wo<PH_ROW6>(b, l, smem4, token, pos);
+        else if (wo_mode == PH_ROW) token_wo<PH_ROW>(b, l, smem4, token, pos);
         else token_wo<PH_RES>(b, l, smem4, token, pos);
         {
             MatvecRun<PH_W13> w13(token_phase(K_W13, l));
             handoff(b, 5 * l + 2, w13);
             w13.template run<true>(smem4, token, pos);
         }
-        if (w2_row) token_w2<PH_ROW>(b, l, smem4, token, pos);
+        if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, smem4, token, pos);
+        else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, smem4, token, pos);
         else token_w2<PH_RES>(b, l, smem4, token, pos);
     }
     if (token_args()->with_cls) {

@@ -72,6 +72,8 @@ TINY = [
     (32, 48, 3, 4, 2, 30, 8, 1),        # multiquery (kv_mul 2), kv_dim 16
     (256, 512, 2, 2, 2, 64, 6, 0),      # 256-aligned, head 128
     (512, 1024, 1, 2, 2, 100, 8, 0),    # head 256 (64 lanes per cache row)
+    (64, 4352, 1, 4, 4, 40, 6, 0),      # W2 rows of 272 chunks: one row per wave, two steps of four chunks per lane
+    (64, 8448, 1, 4, 4, 40, 6, 0),      # W2 rows of 528 chunks: one row per wave, one step of six chunks per lane
 ]
 
 
