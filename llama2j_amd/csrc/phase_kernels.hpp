@@ -445,6 +445,32 @@ struct MatvecRun {
         }
     }
 
+    __device__ __forceinline__ bool has_item() const { return item < nitems; }
+
+    // A wave without an item of this phase lends its registers: the first item of a later phase `o` (rows of the
+    // same length, the same sub-row layout) is requested into them now, while the memory system has little to
+    // do, and `o` takes it over with adopt() when its turn comes.
+    template <class Other>
+    __device__ __forceinline__ void preload_for(Other &o)
+    {
+        static_assert(TU == Other::TU && kOff1 == Other::kOff1, "the two phases must hold an item the same way");
+        first = false;
+        o.resolve(o.item);
+        cb0 = o.cb0; cb1 = o.cb1; gb0 = o.gb0; gb1 = o.gb1; r0 = o.r0; r1 = o.r1;
+        issue(0);
+    }
+
+    template <class Other>
+    __device__ __forceinline__ void adopt(const Other &o)
+    {
+#pragma unroll
+        for (int u = 0; u < TU; u++) {
+            w0[u] = o.w0[u]; w1[u] = o.w1[u];
+            s0[u] = o.s0[u]; s1[u] = o.s1[u];
+        }
+        first = true;
+    }
+
     // Destination of the results of an item (second pointer null when the item has one result).
     __device__ __forceinline__ void dst_of(int it, int pos, float *&p0, float *&p1) const
     {
@@ -1166,12 +1192,61 @@ __device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4,
     w2.template run<true>(smem4, token, pos);
 }
 
+// What handoff() calls on the phase that follows: either the runner's own preload() or one of these.
+template <class A, class B>
+struct LendRegisters {   // a's registers take b's first item when this wave has no item of a
+    A &a;
+    B &b;
+    bool lend;
+    __device__ __forceinline__ void preload()
+    {
+        if (lend) a.preload_for(b);
+        else a.preload();
+    }
+};
+
+template <class A, class B>
+struct TakeRegisters {   // a takes over what LendRegisters requested into b's registers
+    A &a;
+    B &b;
+    bool lend;
+    __device__ __forceinline__ void preload()
+    {
+        if (lend) a.adopt(b);
+        else a.preload();
+    }
+};
+
+// Wo + residual, then rmsnorm + W1,W3 + SwiGLU.  With Wo in row pairs only half the waves of the 7B shape have a Wo item;
+// the others request their first W13 item already when the Wo phase begins (the attention and Wo phases leave the
+// memory system two thirds idle), so that only half of W13's first items remain to be requested at its hand-over.
 template <int WO_MODE>
-__device__ __forceinline__ void token_wo(const GridBar &b, int l, float4 *smem4, int token, int pos)
+__device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, float4 *smem4, int token, int pos)
 {
     MatvecRun<WO_MODE> wo(token_phase(K_WO, l));
-    handoff(b, 5 * l + 1, wo);
+    MatvecRun<PH_W13> w13(token_phase(K_W13, l));
+    bool lend = false;
+    if constexpr (WO_MODE == PH_RES) {
+        // only in workgroups that had no attention item: the others come late, and their wait for the attention
+        // output would queue behind the extra loads
+        int chunk;
+        const int busy = token_args()->g.n_heads * attn_splits_at(pos + 1, token_args()->attn_rows, token_args()->attn_splits, chunk);
+        lend = !wo.has_item() && w13.has_item() && wo.n == w13.n && (int)blockIdx.x >= busy;
+    }
+    if constexpr (WO_MODE == PH_RES) {
+        LendRegisters<MatvecRun<WO_MODE>, MatvecRun<PH_W13>> first{wo, w13, lend};
+        handoff(b, 5 * l + 1, first);
+    } else {
+        handoff(b, 5 * l + 1, wo);
+    }
     wo.template run<true>(smem4, token, pos);
+    if constexpr (WO_MODE == PH_RES) {
+        TakeRegisters<MatvecRun<PH_W13>, MatvecRun<WO_MODE>> second{w13, wo, lend};
+        handoff(b, 5 * l + 2, second);
+    } else {
+        handoff(b, 5 * l + 2, w13);
+    }
+    w13.template run<true>(smem4, token, pos);
 }
 
 template <int LPR>
@@ -1200,14 +1275,9 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
-        if (wo_mode == PH_ROW6) token_wo<PH_ROW6>(b, l, smem4, token, pos);
-        else if (wo_mode == PH_ROW) token_wo<PH_ROW>(b, l, smem4, token, pos);
-        else token_wo<PH_RES>(b, l, smem4, token, pos);
-        {
-            MatvecRun<PH_W13> w13(token_phase(K_W13, l));
-            handoff(b, 5 * l + 2, w13);
-            w13.template run<true>(smem4, token, pos);
-        }
+        if (wo_mode == PH_ROW6) token_wo_w13<PH_ROW6>(b, l, smem4, token, pos);
+        else if (wo_mode == PH_ROW) token_wo_w13<PH_ROW>(b, l, smem4, token, pos);
+        else token_wo_w13<PH_RES>(b, l, smem4, token, pos);
         if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, smem4, token, pos);
         else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, smem4, token, pos);
         else token_w2<PH_RES>(b, l, smem4, token, pos);
