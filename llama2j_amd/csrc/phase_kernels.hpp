@@ -1141,8 +1141,8 @@ template <class Next>
 __device__ __forceinline__ void handoff(const GridBar &b, int inst, Next &nx)
 {
     if (b.ngroups == 0) {  // hand-over by value: the next phase waits for its input itself
+        nx.preload();      // per wave, as soon as its own items are done: it fills the tail of the phase
         __syncthreads();   // every wave is done with the LDS of the phase that ends here
-        nx.preload();
         return;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
