@@ -228,6 +228,22 @@ def test_kernel_timing_entry_point(orc, launch_mode):
     np.testing.assert_array_equal(after, want)
 
 
+@pytest.mark.parametrize("env", [{"L2J_BY_VALUE": "0"}, {"L2J_LAYERS_PER_LAUNCH": "1"}, {"L2J_BY_VALUE": "1"}])
+def test_whole_token_kernel_hand_over_variants(orc, monkeypatch, env):
+    # the whole-token kernel with grid barriers instead of the hand-over by value, with one launch per layer (which
+    # implies barriers), and by value: same tokens as the oracle, deep enough that attention runs in several splits
+    monkeypatch.setenv("L2J_FUSE", "1")
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    for shape in ((64, 96, 3, 4, 2, 40, 200, 1), (256, 512, 2, 2, 2, 64, 96, 0)):
+        m, g = make_pair(orc, shape, seed=61, realistic=True)
+        prompt = orc.synth_prompt(61, 4, shape[5])
+        want, _, _ = m.generate_greedy(prompt, min(160, shape[6]))
+        got, _ = g.decode_greedy(prompt, min(160, shape[6]))
+        np.testing.assert_array_equal(got, want)
+        g.close()
+
+
 def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
     # a spin limit of zero makes the bounded waits of the whole-token kernel give up at once: every kernel still
     # runs to its end, the call reports the failure, and a context with the normal limit is unaffected
