@@ -407,21 +407,25 @@ struct MatvecRun {
         cb1 = mb.codes + f1; gb1 = mb.gs + (f1 >> 8); r1 = (unsigned)(f1 & 255);
     }
 
-    // Requests one step (kTU chunks per lane and sub-row) of the resolved item.
+    // Requests chunk u (of TU per lane and sub-row) of step `base` of the resolved item.
     // (Members are used by name in every helper: a reference to a member keeps the whole object in memory.)
+    __device__ __forceinline__ void issue_chunk(int base, int u)
+    {
+        const int c = base + 64 * u + lane, c1 = c + kOff1;
+        const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 in fold)
+        const unsigned cc1 = c1 < nch ? c1 : nch - 1;
+        const uint4 a0 = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
+        const uint4 a1 = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc1);
+        const float2 g0 = gb0[(r0 + 16u * cc) >> 8];
+        const float2 g1 = gb1[(r1 + 16u * cc1) >> 8];
+        w0[u] = a0; w1[u] = a1; s0[u] = g0; s1[u] = g1;
+    }
+
+    // Requests one step of the resolved item.
     __device__ __forceinline__ void issue(int base)
     {
 #pragma unroll
-        for (int u = 0; u < TU; u++) {
-            const int c = base + 64 * u + lane, c1 = c + kOff1;
-            const unsigned cc = c < nch ? c : nch - 1;  // out-of-range lanes repeat the last chunk (weight 0 below)
-            const unsigned cc1 = c1 < nch ? c1 : nch - 1;
-            const uint4 a0 = load_stream(reinterpret_cast<const uint4 *>(cb0) + cc);
-            const uint4 a1 = load_stream(reinterpret_cast<const uint4 *>(cb1) + cc1);
-            const float2 g0 = gb0[(r0 + 16u * cc) >> 8];
-            const float2 g1 = gb1[(r1 + 16u * cc1) >> 8];
-            w0[u] = a0; w1[u] = a1; s0[u] = g0; s1[u] = g1;
-        }
+        for (int u = 0; u < TU; u++) issue_chunk(base, u);
     }
 
     // Defined on every path: otherwise the registers stay reserved for the whole layer loop of k_token.
@@ -506,7 +510,12 @@ struct MatvecRun {
     }
 
     // One step of weights against the staged vector: sum (code*rm + min)*x = rm * sum code*x + min * sum x per chunk.
-    __device__ __forceinline__ void fold(int base, const float4 *xs, const float *sumx, float &acc0, float &acc1)
+    // With REFILL, the registers of a chunk are requested anew (step `nbase` of the item resolved last) as soon as the
+    // chunk is folded: the requests of the next step go out between the multiply-adds of this one instead of after them,
+    // so the memory system is not left idle while all the waves of a workgroup work off a step at the same time (at the
+    // start of a phase in particular, when every wave holds a step that was requested ahead).
+    template <bool REFILL>
+    __device__ __forceinline__ void fold(int base, const float4 *xs, const float *sumx, float &acc0, float &acc1, int nbase)
     {
 #pragma unroll
         for (int u = 0; u < TU; u++) {
@@ -530,12 +539,17 @@ struct MatvecRun {
                 const float t1 = fmaf(g1.x, dot16(a1, x0, x1, x2, x3), g1.y * sx);
                 acc1 += ok ? t1 : 0.0f;
             }
+            if (REFILL) {  // fenced: left alone, the scheduler moves all the requests to the top, into registers of their own
+                __builtin_amdgcn_sched_barrier(0);
+                issue_chunk(nbase, u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     }
 
     // Reduces the sums of the resolved item over the wave, applies the phase's epilogue and stores the results.
     template <bool COH>
-    __device__ __forceinline__ void finish(int it, float acc0, float acc1, float resv0, float resv1, int pos)
+    __device__ __forceinline__ void finish(int it, int wh, int rr, float acc0, float acc1, float resv0, float resv1, int pos)
     {
         acc0 = wave_sum(acc0);
         acc1 = wave_sum(acc1);
@@ -544,8 +558,8 @@ struct MatvecRun {
             if (MODE == PH_QKV) {
                 v0 = acc0;
                 v1 = acc1;
-                if (which < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
-                    const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((r % d.head_size) >> 1)];
+                if (wh < 2) {  // RoPE on the interleaved pair (r, r+1)  (K/ApplyRope.java:74-90)
+                    const float2 cs = d.rope[(long)pos * (d.head_size >> 1) + ((rr % d.head_size) >> 1)];
                     v0 = __fsub_rn(__fmul_rn(acc0, cs.x), __fmul_rn(acc1, cs.y));
                     v1 = __fadd_rn(__fmul_rn(acc0, cs.y), __fmul_rn(acc1, cs.x));
                 }
@@ -563,8 +577,8 @@ struct MatvecRun {
             if (COH) {
                 st_coh(p0, v0);
                 if (p1) st_coh(p1, v1);
-                if (MODE == PH_QKV && d.knew && which > 0) {  // where attention waits for this token's rows
-                    float *p = (which == 1 ? d.knew : d.vnew) + r;
+                if (MODE == PH_QKV && d.knew && wh > 0) {  // where attention waits for this token's rows
+                    float *p = (wh == 1 ? d.knew : d.vnew) + rr;
                     st_coh(p, v0);
                     st_coh(p + 1, v1);
                 }
@@ -592,18 +606,41 @@ struct MatvecRun {
             stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
         }
 
-        for (; item < nitems; item += W * G) {
-            if (!first) resolve(item);
-            float resv0, resv1;
-            residual(res, resv0, resv1);
-            float acc0 = 0.0f, acc1 = 0.0f;
-            for (int base = 0; base < nch; base += kStep) {
-                if (!(first && base == 0)) issue(base);
-                fold(base, xs, sumx, acc0, acc1);
-            }
-            first = false;
-            finish<COH>(item, acc0, acc1, resv0, resv1, pos);
+        if (item >= nitems) return;
+        if (!first) {
+            resolve(item);
+            issue(0);
         }
+        first = false;
+        // The steps of this wave's items in order; while a step is folded, the step after it is requested.
+        int cur = item, cur_which = which, cur_r = r, base = 0;
+        float resv0, resv1, acc0 = 0.0f, acc1 = 0.0f;
+        residual(res, resv0, resv1);
+        while (true) {
+            int nbase = base + kStep, nitem = cur;
+            const bool last_step = nbase >= nch;
+            if (last_step) {
+                nbase = 0;
+                nitem = cur + W * G;
+            }
+            if (nitem >= nitems) break;  // the step in the registers is the wave's last one
+            float nres0 = 0.0f, nres1 = 0.0f;
+            if (last_step) {  // (the residual of the next item is fetched ahead of its weights: its wait is in order)
+                resolve(nitem);
+                residual(res, nres0, nres1);
+            }
+            fold<true>(base, xs, sumx, acc0, acc1, nbase);
+            if (last_step) {
+                finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos);
+                cur = nitem; cur_which = which; cur_r = r;
+                resv0 = nres0; resv1 = nres1;
+                acc0 = acc1 = 0.0f;
+            }
+            base = nbase;
+        }
+        fold<false>(base, xs, sumx, acc0, acc1, 0);
+        finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos);
+        item = nitems;
     }
 };
 
