@@ -1,7 +1,7 @@
 // The per-token forward pass (J/Run.java:62-169) on gfx950.  Per layer there are five phases:
 //   PH_QKV      rmsnorm + Wq,Wk,Wv matvec + RoPE + KV-cache store
 //   attention   decode attention, split over the sequence, online softmax
-//   PH_RES/ROW  Wo matvec + residual
+//   PH_RES/ROW  Wo matvec + residual (row pairs, or one row per wave when rows are long: PH_ROW, PH_ROW6)
 //   PH_W13      rmsnorm + W1,W3 matvec + SwiGLU (the reference's sigmoid table)
 //   PH_RES/ROW  W2 matvec + residual
 // and once per token k_classifier (final rmsnorm + fp32 classifier + per-workgroup first-max) and k_finish
@@ -23,6 +23,13 @@
 // device-coherent loads until it is gone) or, after a grid barrier of relaxed counters, use plain loads.
 // In both cases the first weights of the next phase are requested before the wait, so HBM stays busy while
 // the slowest workgroups finish the phase.
+//
+// The weight registers of the waves are the only buffer between the phases, so when and by whom they are filled
+// decides how busy the memory system stays: a wave requests the first step of its next phase as soon as its own
+// items are done (before the workgroup's barrier); while it folds a step it requests the next one chunk by chunk
+// (two vector instructions per weight are a fifth of a layer's time and would otherwise leave gaps); waves without
+// a Wo item lend their registers to their first W13 item during the attention and Wo phases; W2's long rows are
+// held whole (PH_ROW6), two thirds requested ahead of the hand-over.
 #pragma once
 
 #include "kernels.hpp"
