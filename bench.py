@@ -181,7 +181,7 @@ def main():
         kern = {}
         for k in range(7):
             try:
-                us, b = g.time_kernel(k, pos, rounds=3)
+                us, b = g.time_kernel(k, pos, rounds=32 if k == KERNEL.TOKEN else 3)
             except l2j.L2JError:
                 if k != KERNEL.TOKEN:
                     raise

@@ -165,8 +165,8 @@ int l2j_read(l2j_ctx *ctx, int which, int layer, uint64_t off, float *dst, uint6
 int l2j_write_kv(l2j_ctx *ctx, int layer, int32_t pos0, int32_t npos, const float *k, const float *v);
 int l2j_sync(l2j_ctx *ctx);
 
-/* Measurement: launches one kernel class `rounds` times at position `pos` and returns the mean kernel time
- * from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
+/* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
+ * and returns the mean kernel time from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
  * every layer and the classifier in one launch.  The other classes launch one phase of it as a kernel of its
  * own, once per layer (cold weights, as inside a token). */
 enum l2j_kernel_class { L2J_K_QKV = 0, L2J_K_ATTENTION, L2J_K_WO, L2J_K_W13, L2J_K_W2, L2J_K_CLASSIFIER, L2J_K_TOKEN, L2J_K_COUNT };

@@ -1218,26 +1218,30 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
     if (bytes) *bytes = b;
     if (kclass == L2J_K_TOKEN) {  // the whole-token kernel, then k_finish (untimed) to reset the barrier counters
         if (!c->fused) return fail(L2J_E_STATE, "the whole-token kernel is switched off or does not fit this shape");
-        while ((int)c->events.size() < 35) {
+        if (rounds > 256) return fail(L2J_E_ARG, "at most 256 rounds of the whole-token kernel");
+        while ((int)c->events.size() < 33 + 2 * rounds) {
             hipEvent_t ev;
             HIPCHK(hipEventCreate(&ev));
             c->events.push_back(ev);
         }
-        double total = 0.0;
+        // the rounds follow each other on the stream without a host round trip in between, as the tokens of a decode do
         for (int r = 0; r < rounds; r++) {
             if ((rc = set_state(c, 1, pos, 0))) return rc;
             if (c->by_value) {
                 hipError_t ef = launch_fill_unset(c, c->stream);
                 if (ef != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(ef));
             }
-            hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33], c->events[34]);
+            hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33 + 2 * r], c->events[34 + 2 * r]);
             if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
             hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));
             HIPCHK(hipGetLastError());
-            HIPCHK(hipStreamSynchronize(c->stream));
-            if ((rc = check_barrier_error(c))) return rc;
+        }
+        HIPCHK(hipStreamSynchronize(c->stream));
+        if ((rc = check_barrier_error(c))) return rc;
+        double total = 0.0;
+        for (int r = 0; r < rounds; r++) {
             float ms = 0.f;
-            HIPCHK(hipEventElapsedTime(&ms, c->events[33], c->events[34]));
+            HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * r], c->events[34 + 2 * r]));
             total += ms;
         }
         *mean_us = total * 1e3 / rounds;
