@@ -972,10 +972,11 @@ int l2j_finalize(l2j_ctx *c)
         HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&c->h_fault), sizeof(int), hipHostMallocDefault));
         *c->h_fault = 0;
         // k_token needs its whole grid resident at once (grid barriers): at most what the occupancy allows.
-        // One launch per token pays off when a layer streams enough to hide its five hand-overs (7B: 208 MB,
-        // 545 vs 511 tok/s); small models run faster as one launch per phase (15M shape: 6100 vs 4700 tok/s).
+        // One launch per token pays off when a layer streams enough to hide its five hand-overs (7B shape, 208 MB a
+        // layer: 645 vs 511 tok/s; 110M shape, 7 MB: 3240 vs 3080); the smallest models run faster as one launch per
+        // phase (15M shape, 1 MB a layer: 6300 vs 5400 tok/s).
         const uint64_t layer_floats = 2ull * c->cfg.dim * c->cfg.dim + 2ull * c->cfg.dim * c->kv_dim + 3ull * c->cfg.dim * c->cfg.hidden_dim;
-        c->fused = env_int("L2J_FUSE", layer_floats >= (32ull << 20) ? 1 : 0) != 0;
+        c->fused = env_int("L2J_FUSE", layer_floats >= (4ull << 20) ? 1 : 0) != 0;
         c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, env_int("L2J_LAYERS_PER_LAUNCH", c->cfg.n_layers)));
         if (c->fused) {
             const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
