@@ -252,15 +252,22 @@ hipError_t launch_fill_unset(const l2j_ctx *c, hipStream_t s)
     return hipGetLastError();
 }
 
-// The instantiation of k_token for this context: by lanes per cache row.
+// The instantiation of k_token for this context: by lanes per cache row, and, for the shapes of the published models,
+// by the chunks per lane that make a row of dim / hidden codes one step (tu_for); the general instantiation runs any shape.
 template <typename F>
 auto with_token_kernel(const l2j_ctx *c, F f)
 {
     const int lpr = attn_lpr(c);
+    const int tud = tu_for(c->cfg.dim), tuh = tu_for(c->cfg.hidden_dim);
+    const bool special = env_int("L2J_TOKEN_SPECIAL", 1) != 0;
+    if (special && lpr == 16 && tud == 1 && tuh == 1) return f(k_token<16, 1, 1>);
+    if (special && lpr == 16 && tud == 1 && tuh == 2) return f(k_token<16, 1, 2>);
+    if (special && lpr == 32 && tud == 5) return f(k_token<32, 5, kTU>);
     if (lpr == 16) return f(k_token<16>);
     if (lpr == 32) return f(k_token<32>);
     return f(k_token<64>);
 }
+
 
 // Layers [l0, l1) (and the classifier after the last layer) in one launch of k_token.
 hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
@@ -293,20 +300,32 @@ hipError_t launch1(K kernel, dim3 grid, dim3 block, size_t smem, hipStream_t s, 
     return hipGetLastError();
 }
 
+// k_matvec<MODE, TU> for rows of n codes streamed as row pairs (QKV, W13, and Wo / W2 with rows of up to 320 chunks).
+template <int MODE, typename A>
+hipError_t launch_pairs(int n, dim3 grid, dim3 block, size_t smem, hipStream_t s, const A &args, hipEvent_t e0, hipEvent_t e1)
+{
+    switch (tu_for(n)) {
+    case 1: return launch1(k_matvec<MODE, 1>, grid, block, smem, s, args, e0, e1);
+    case 2: return launch1(k_matvec<MODE, 2>, grid, block, smem, s, args, e0, e1);
+    case 5: return launch1(k_matvec<MODE, 5>, grid, block, smem, s, args, e0, e1);
+    default: return launch1(k_matvec<MODE, kTU>, grid, block, smem, s, args, e0, e1);
+    }
+}
+
 // One kernel class of layer l.  Optional start/stop events bracket the kernel itself.
 hipError_t launch_class(const l2j_ctx *c, int kclass, int l, hipStream_t s, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
 {
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     switch (kclass) {
-    case L2J_K_QKV: return launch1(k_matvec<PH_QKV>, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
-    case L2J_K_W13: return launch1(k_matvec<PH_W13>, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
+    case L2J_K_QKV: return launch_pairs<PH_QKV>(c->cfg.dim, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
+    case L2J_K_W13: return launch_pairs<PH_W13>(c->cfg.dim, grid, block, mv_smem(c->cfg.dim), s, matvec_phase(c, kclass, l), e0, e1);
     case L2J_K_WO:
     case L2J_K_W2: {
         const int n = kclass == L2J_K_WO ? c->cfg.dim : c->cfg.hidden_dim;
+        if (n / 16 <= 320) return launch_pairs<PH_RES>(n, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
         const int mode = row_mode(n);  // long rows: one row per wave keeps every wave busy
         if (mode == PH_ROW6) return launch1(k_matvec<PH_ROW6>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
-        if (mode == PH_ROW) return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
-        return launch1(k_matvec<PH_RES>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
+        return launch1(k_matvec<PH_ROW>, grid, block, mv_smem(n), s, matvec_phase(c, kclass, l), e0, e1);
     }
     case L2J_K_ATTENTION: {
         const dim3 ag(c->attn_grid), ab(c->attn_threads);
@@ -956,8 +975,12 @@ int l2j_finalize(l2j_ctx *c)
             const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
                                 reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
                                 reinterpret_cast<const void *>(k_matvec<PH_ROW6>),
+                                reinterpret_cast<const void *>(k_matvec<PH_QKV, 5>), reinterpret_cast<const void *>(k_matvec<PH_W13, 5>),
+                                reinterpret_cast<const void *>(k_matvec<PH_RES, 5>),
                                 reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
-                                reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>)};
+                                reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>),
+                                reinterpret_cast<const void *>(k_token<16, 1, 1>), reinterpret_cast<const void *>(k_token<16, 1, 2>),
+                                reinterpret_cast<const void *>(k_token<32, 5, kTU>)};
             for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
         }
         int rc2;

@@ -30,6 +30,10 @@
 // (two vector instructions per weight are a fifth of a layer's time and would otherwise leave gaps); waves without
 // a Wo item lend their registers to their first W13 item during the attention and Wo phases; W2's long rows are
 // held whole (PH_ROW6), two thirds requested ahead of the hand-over.
+//
+// A wave holds TU 16-byte chunks per lane and sub-row (64 * TU chunks = one step).  Four fit the 7B shape (rows of
+// 256 chunks); the kernels are also instantiated with one, two and five chunks for the rows of the small models
+// (18..128 chunks) and of the 13B shape (320 chunks), so that a row is one full step there too (tu_for).
 #pragma once
 
 #include "kernels.hpp"
@@ -343,7 +347,9 @@ constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
 // One matvec phase of one workgroup: preload() requests the first weights (they do not depend on the input
 // vector), run() stages the vector and streams the items.  (Two items in flight per wave with 512-thread
 // workgroups, so that a wave may use 256 registers, was measured: 1.82 against 1.78 ms per 7B token.)
-template <int MODE>
+// TU_ = 16-byte chunks per lane and sub-row that a wave holds at a time (64 * TU_ chunks are one step of a sub-row):
+// rows of up to 64 * TU_ chunks are one step, and a phase whose rows are shorter than its step folds empty chunks.
+template <int MODE, int TU_ = (MODE == PH_ROW6 ? 6 : kTU)>
 struct MatvecRun {
     // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
     // PH_ROW6 holds six chunks per lane and sub-row instead of four: a row of 513..768 chunks (11008 codes are 688) is
@@ -351,14 +357,17 @@ struct MatvecRun {
     // step (1.72 -> 1.70 ms per 7B token; for shorter or longer rows the extra registers and masked loads cost more
     // than they gain: 3.24 -> 3.60 ms per 13B token).
     static constexpr bool kRow = MODE == PH_ROW || MODE == PH_ROW6;
-    static constexpr int TU = MODE == PH_ROW6 ? 6 : kTU;
+    static constexpr int TU = TU_;
     static constexpr int kStep = kRow ? 2 * 64 * TU : 64 * TU;
     static constexpr int kOff1 = kRow ? 64 * TU : 0;
-    // PH_ROW6 requests only kAhead of its six chunks ahead of the hand-over and the others once the input vector is staged:
-    // the wait for the vector ends when the wave's own requests have arrived, and with the whole row requested ahead
-    // all the multiply-adds of the phase would follow after the last arrival instead of overlapping it.
-    static constexpr bool kSplitAhead = MODE == PH_ROW6;
-    static constexpr int kAhead = kTU;  // (measured per 7B token: all six chunks ahead 1.573 ms, four 1.551, three 1.568, two 1.556)
+    // Runners with more than kTU chunks request only kAhead of them ahead of the hand-over and the others once the input
+    // vector is staged: the wait for the vector ends when the wave's own requests have arrived, and with the whole row
+    // requested ahead all the multiply-adds of the phase would follow after the last arrival instead of overlapping it.
+    // Measured per 7B token for W2's six chunks: all ahead 1.573 ms, four 1.551, three 1.568, two 1.556; per 13B token
+    // for the five chunks of QKV and W13: all ahead 3.14 ms, four 2.92, three 2.74, two 2.79; three of QKV's or W13's four
+    // at the 7B shape: no change.  Wo's row pairs are always requested whole: that phase only waits for its input.
+    static constexpr int kAhead = TU == 6 ? kTU : TU == 5 && MODE != PH_RES ? 3 : TU;
+    static constexpr bool kSplitAhead = kAhead < TU;
 
     const MatvecPhase d;
     int n, nch, lane, W, G, nitems, item;
@@ -665,11 +674,11 @@ struct MatvecRun {
     }
 };
 
-template <int MODE>
+template <int MODE, int TU = (MODE == PH_ROW6 ? 6 : kTU)>
 __global__ void __launch_bounds__(1024) k_matvec(const MatvecPhase d)
 {
     extern __shared__ float4 smem4[];
-    MatvecRun<MODE> run(d);
+    MatvecRun<MODE, TU> run(d);
     // The weights do not depend on the input vector: the first loads go out before it is staged, so
     // HBM latency overlaps the rmsnorm prologue.
     run.preload();
@@ -1167,6 +1176,15 @@ __host__ __device__ inline int row_mode(int n)
     return nch <= 64 * kTU ? PH_RES : nch > 2 * 64 * kTU && nch <= 2 * 64 * 6 ? PH_ROW6 : PH_ROW;
 }
 
+// Chunks per lane and sub-row for rows of n codes streamed as row pairs in one step each: the smallest of 1, 2, 4, 5
+// that holds a row (short rows would otherwise fold three empty chunks out of four; rows of 257..320 chunks, the 13B
+// shape's, would take a second step for a quarter of a step's worth).  kTU for everything longer.
+__host__ __device__ inline int tu_for(int n)
+{
+    const int nch = n / 16;
+    return nch <= 64 ? 1 : nch <= 128 ? 2 : nch <= 256 ? 4 : nch <= 320 ? 5 : kTU;
+}
+
 struct TokenArgs {
     TokenGeom g;
     int l0, l1, with_cls;   // layers [l0, l1), then the classifier when with_cls
@@ -1242,10 +1260,10 @@ __device__ __forceinline__ MatvecPhase token_phase(int kclass, int l)
     return d;
 }
 
-template <int W2_MODE>
+template <int W2_MODE, int TU = (W2_MODE == PH_ROW6 ? 6 : kTU)>
 __device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4, int token, int pos)
 {
-    MatvecRun<W2_MODE> w2(token_phase(K_W2, l));
+    MatvecRun<W2_MODE, TU> w2(token_phase(K_W2, l));
     handoff(b, 5 * l + 3, w2);
     w2.template run<true>(smem4, token, pos);
 }
@@ -1278,28 +1296,30 @@ struct TakeRegisters {   // a takes over what LendRegisters requested into b's r
 // Wo + residual, then rmsnorm + W1,W3 + SwiGLU.  With Wo in row pairs only half the waves of the 7B shape have a Wo item;
 // the others request their first W13 item already when the Wo phase begins (the attention and Wo phases leave the
 // memory system two thirds idle), so that only half of W13's first items remain to be requested at its hand-over.
-template <int WO_MODE>
+template <int WO_MODE, int TUD = kTU, bool LEND = true>
 __device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, float4 *smem4, int token, int pos)
 {
-    MatvecRun<WO_MODE> wo(token_phase(K_WO, l));
-    MatvecRun<PH_W13> w13(token_phase(K_W13, l));
+    typedef MatvecRun<WO_MODE, (WO_MODE == PH_RES ? TUD : WO_MODE == PH_ROW6 ? 6 : kTU)> WoRun;
+    typedef MatvecRun<PH_W13, TUD> W13Run;
+    WoRun wo(token_phase(K_WO, l));
+    W13Run w13(token_phase(K_W13, l));
     bool lend = false;
-    if constexpr (WO_MODE == PH_RES) {
+    if constexpr (WO_MODE == PH_RES && LEND) {
         // only in workgroups that had no attention item: the others come late, and their wait for the attention
         // output would queue behind the extra loads
         int chunk;
         const int busy = token_args()->g.n_heads * attn_splits_at(pos + 1, token_args()->attn_rows, token_args()->attn_splits, chunk);
         lend = !wo.has_item() && w13.has_item() && wo.n == w13.n && (int)blockIdx.x >= busy;
     }
-    if constexpr (WO_MODE == PH_RES) {
-        LendRegisters<MatvecRun<WO_MODE>, MatvecRun<PH_W13>> first{wo, w13, lend};
+    if constexpr (WO_MODE == PH_RES && LEND) {
+        LendRegisters<WoRun, W13Run> first{wo, w13, lend};
         handoff(b, 5 * l + 1, first);
     } else {
         handoff(b, 5 * l + 1, wo);
     }
     wo.template run<true>(smem4, token, pos);
-    if constexpr (WO_MODE == PH_RES) {
-        TakeRegisters<MatvecRun<PH_W13>, MatvecRun<WO_MODE>> second{w13, wo, lend};
+    if constexpr (WO_MODE == PH_RES && LEND) {
+        TakeRegisters<W13Run, WoRun> second{w13, wo, lend};
         handoff(b, 5 * l + 2, second);
     } else {
         handoff(b, 5 * l + 2, w13);
@@ -1307,7 +1327,9 @@ __device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, float4 *sm
     w13.template run<true>(smem4, token, pos);
 }
 
-template <int LPR>
+// TUD, TUH: chunks per lane and sub-row for the phases whose rows are dim and hidden codes long (tu_for); kTU is
+// the general case, in which the Wo and W2 phases pick their mode by the row length (row_mode).
+template <int LPR, int TUD = kTU, int TUH = kTU>
 __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
 {
     extern __shared__ float4 smem4[];
@@ -1319,7 +1341,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
     for (int l = l0; l < l1; l++) {
         {
-            MatvecRun<PH_QKV> qkv(token_phase(K_QKV, l));
+            MatvecRun<PH_QKV, TUD> qkv(token_phase(K_QKV, l));
             if (l == l0) qkv.preload();             // launch order guarantees the input
             else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
             qkv.template run<true>(smem4, token, pos);
@@ -1333,12 +1355,22 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
-        if (wo_mode == PH_ROW6) token_wo_w13<PH_ROW6>(b, l, smem4, token, pos);
-        else if (wo_mode == PH_ROW) token_wo_w13<PH_ROW>(b, l, smem4, token, pos);
-        else token_wo_w13<PH_RES>(b, l, smem4, token, pos);
-        if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, smem4, token, pos);
-        else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, smem4, token, pos);
-        else token_w2<PH_RES>(b, l, smem4, token, pos);
+        if constexpr (TUD < kTU) {  // the host picked TUD so that a row of dim codes is one step
+            token_wo_w13<PH_RES, TUD>(b, l, smem4, token, pos);
+        } else if constexpr (TUD > kTU) {  // without lending (measured at the 13B shape: 2.77 with, 2.74 ms without)
+            token_wo_w13<PH_RES, TUD, false>(b, l, smem4, token, pos);
+        } else {
+            if (wo_mode == PH_ROW6) token_wo_w13<PH_ROW6>(b, l, smem4, token, pos);
+            else if (wo_mode == PH_ROW) token_wo_w13<PH_ROW>(b, l, smem4, token, pos);
+            else token_wo_w13<PH_RES>(b, l, smem4, token, pos);
+        }
+        if constexpr (TUH != kTU) {  // likewise for a row of hidden codes
+            token_w2<PH_RES, TUH>(b, l, smem4, token, pos);
+        } else {
+            if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, smem4, token, pos);
+            else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, smem4, token, pos);
+            else token_w2<PH_RES>(b, l, smem4, token, pos);
+        }
     }
     if (token_args()->with_cls) {
         ClsPhase cp = cls_phase_of(token_args()->g, gridDim.x);

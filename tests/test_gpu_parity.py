@@ -47,8 +47,11 @@ def make_pair(orc, shape, seed, sigma=0.02, realistic=False, upload="bytes"):
         rng = np.random.default_rng(seed)
         for t in (orc.T_RMS_ATT, orc.T_RMS_FFN, orc.T_RMS_FINAL):
             m.set_quant(t, orc.quant_encode((1.0 + 0.1 * rng.standard_normal(m.tensor_floats(t))).astype(np.float32)))
+        # (narrower for long rows: the reference shifts its softmax by a running maximum of element products, and scores
+        # more than 87 below it underflow to an all-zero attention row there, which the GPU's true softmax does not copy)
+        wide = 0.12 * min(1.0, 256.0 / dim)
         for t in (orc.T_WQ, orc.T_WK):
-            m.set_quant(t, orc.quant_encode((0.12 * rng.standard_normal(m.tensor_floats(t))).astype(np.float32)))
+            m.set_quant(t, orc.quant_encode((wide * rng.standard_normal(m.tensor_floats(t))).astype(np.float32)))
     g = l2j.Transformer(l2j.Config(dim, hidden, L, H, kvH, vocab, seq, shared))
     if upload == "synthetic":
         g.fill_synthetic(seed, sigma)
@@ -74,6 +77,8 @@ TINY = [
     (512, 1024, 1, 2, 2, 100, 8, 0),    # head 256 (64 lanes per cache row)
     (64, 4352, 1, 4, 4, 40, 6, 0),      # W2 rows of 272 chunks: one row per wave, two steps of four chunks per lane
     (64, 8448, 1, 4, 4, 40, 6, 0),      # W2 rows of 528 chunks: one row per wave, one step of six chunks per lane
+    (1280, 1536, 1, 10, 10, 64, 6, 0),  # rows of 80 and 96 chunks: two chunks per lane
+    (4352, 256, 1, 34, 34, 40, 6, 0),   # rows of 272 chunks: five chunks per lane, three of them requested ahead
 ]
 
 
