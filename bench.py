@@ -76,7 +76,7 @@ def main():
     ap.add_argument("--steps", type=int, default=288, help="tokens decoded in the timed region (32 prompt + 256 greedy)")
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--workload", default="llama2-7b-shape", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-steps", type=int, default=13, help="forwards of the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=97, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
     ap.add_argument("--no-sampled", action="store_true", help="skip the extra decode with the device sampler")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
