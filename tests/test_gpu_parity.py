@@ -190,6 +190,28 @@ def test_forward_matches_oracle_in_both_launch_modes(orc, shape, launch_mode):
         assert rel_err(g.forward(int(tok), pos), m.forward(int(tok), pos)) < 1e-4, pos
 
 
+# Row lengths on both sides of the steps at which the kernels change the chunks a lane holds (64, 128, 256, 320 chunks
+# for row pairs; 512 and 768 for single rows), odd head counts, multiquery, shared and separate classifier.
+BOUNDARY = [
+    (1024, 12304, 1, 8, 4, 40, 6, 1),     # rows of 64 chunks; W2 rows of 769
+    (1040, 8208, 1, 65, 65, 40, 6, 1),    # 65 chunks; 513
+    (2048, 4112, 1, 8, 8, 40, 6, 0),      # 128; 257
+    (2064, 5136, 2, 43, 43, 40, 6, 1),    # 129; 321
+    (3200, 1040, 1, 40, 20, 40, 6, 1),    # 200; 65
+    (4112, 5120, 1, 257, 257, 40, 6, 0),  # 257; 320
+    (5120, 12288, 1, 32, 16, 40, 6, 1),   # 320; 768
+    (5136, 8192, 1, 107, 107, 40, 6, 1),  # 321; 512
+]
+
+
+@pytest.mark.parametrize("shape", BOUNDARY)
+def test_row_length_boundaries_in_both_launch_modes(orc, shape, launch_mode):
+    m, g = make_pair(orc, shape, seed=29, realistic=True)
+    rng = np.random.default_rng(4)
+    for pos, tok in enumerate(rng.integers(0, shape[5], size=4)):
+        assert rel_err(g.forward(int(tok), pos), m.forward(int(tok), pos)) < 1e-4, pos
+
+
 def test_split_attention_in_both_launch_modes(orc, launch_mode):
     # contexts long enough that attention is split over several workgroups (whole-token launch: beyond 64
     # positions; kernel-by-kernel: beyond 32) and folded by the last arriver; multiquery, head 16
