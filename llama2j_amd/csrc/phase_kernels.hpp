@@ -109,26 +109,16 @@ __device__ __forceinline__ void load_words(const float *const (&p)[3], float4 (&
                  : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]) : "v"(p[0]), "v"(p[1]), "v"(p[2]) : "memory");
 }
 
-// Eight device-coherent loads at byte offsets off[] from one uniform base, one wait (4 or 8 bytes each).
-__device__ __forceinline__ void load8_coh(const float *base, const unsigned (&off)[8], float (&v)[8])
-{
-    asm volatile("global_load_dword %0, %8, %16 sc1\n\tglobal_load_dword %1, %9, %16 sc1\n\t"
-                 "global_load_dword %2, %10, %16 sc1\n\tglobal_load_dword %3, %11, %16 sc1\n\t"
-                 "global_load_dword %4, %12, %16 sc1\n\tglobal_load_dword %5, %13, %16 sc1\n\t"
-                 "global_load_dword %6, %14, %16 sc1\n\tglobal_load_dword %7, %15, %16 sc1\n\ts_waitcnt vmcnt(0)"
-                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
-                 : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]), "s"(base)
-                 : "memory");
-}
-
-__device__ __forceinline__ void load8_coh(const float *base, const unsigned (&off)[8], float2 (&v)[8])
+// Four 8-byte and four 4-byte device-coherent loads at byte offsets from one uniform base, one wait.
+__device__ __forceinline__ void load4x2_coh(const float *base, const unsigned (&off2)[4], float2 (&v2)[4], const unsigned (&off1)[4],
+                                            float (&v1)[4])
 {
     asm volatile("global_load_dwordx2 %0, %8, %16 sc1\n\tglobal_load_dwordx2 %1, %9, %16 sc1\n\t"
                  "global_load_dwordx2 %2, %10, %16 sc1\n\tglobal_load_dwordx2 %3, %11, %16 sc1\n\t"
-                 "global_load_dwordx2 %4, %12, %16 sc1\n\tglobal_load_dwordx2 %5, %13, %16 sc1\n\t"
-                 "global_load_dwordx2 %6, %14, %16 sc1\n\tglobal_load_dwordx2 %7, %15, %16 sc1\n\ts_waitcnt vmcnt(0)"
-                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
-                 : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]), "s"(base)
+                 "global_load_dword %4, %12, %16 sc1\n\tglobal_load_dword %5, %13, %16 sc1\n\t"
+                 "global_load_dword %6, %14, %16 sc1\n\tglobal_load_dword %7, %15, %16 sc1\n\ts_waitcnt vmcnt(0)"
+                 : "=&v"(v2[0]), "=&v"(v2[1]), "=&v"(v2[2]), "=&v"(v2[3]), "=&v"(v1[0]), "=&v"(v1[1]), "=&v"(v1[2]), "=&v"(v1[3])
+                 : "v"(off2[0]), "v"(off2[1]), "v"(off2[2]), "v"(off2[3]), "v"(off1[0]), "v"(off1[1]), "v"(off1[2]), "v"(off1[3]), "s"(base)
                  : "memory");
 }
 
@@ -903,30 +893,29 @@ struct AttnRun {
             const float *hp = a.part + (long)h * a.nsplit * (hs + 2);
             if (tid < hs) {
                 float MM = -3.402823466e+38f, LL = 0.0f, oo = 0.0f;
-                for (int i0 = 0; i0 < nact; i0 += 8) {
-                    // the (maximum, sum) pairs and this thread's element of eight partials: two trips to memory
-                    float pm[8], pl[8], po[8];
-                    float2 ml[8];
-                    unsigned off[8];
+                for (int i0 = 0; i0 < nact; i0 += 4) {
+                    // the (maximum, sum) pairs and this thread's element of four partials: one trip to memory
+                    float pm[4], pl[4], po[4];
+                    float2 ml[4];
+                    unsigned off2[4], off1[4];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) off[i] = (unsigned)(min(i0 + i, nact - 1) * (hs + 2)) * 4u;
-                    load8_coh(hp, off, ml);
-#pragma unroll
-                    for (int i = 0; i < 8; i++) {
-                        pm[i] = ml[i].x;
-                        pl[i] = ml[i].y;
-                        off[i] += (unsigned)(2 + tid) * 4u;
+                    for (int i = 0; i < 4; i++) {
+                        off2[i] = (unsigned)(min(i0 + i, nact - 1) * (hs + 2)) * 4u;
+                        off1[i] = off2[i] + (unsigned)(2 + tid) * 4u;
                     }
-                    load8_coh(hp, off, po);
+                    load4x2_coh(hp, off2, ml, off1, po);
                     float mb = MM;
 #pragma unroll
-                    for (int i = 0; i < 8; i++)
+                    for (int i = 0; i < 4; i++) {
+                        pm[i] = ml[i].x;
+                        pl[i] = ml[i].y;
                         if (i0 + i < nact) mb = fmaxf(mb, pm[i]);
+                    }
                     const float scale = expf(MM - mb);
                     LL *= scale;
                     oo *= scale;
 #pragma unroll
-                    for (int i = 0; i < 8; i++) {
+                    for (int i = 0; i < 4; i++) {
                         if (i0 + i < nact) {
                             const float w = expf(pm[i] - mb);
                             LL = fmaf(pl[i], w, LL);
