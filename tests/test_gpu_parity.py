@@ -271,6 +271,17 @@ def test_whole_token_kernel_hand_over_variants(orc, monkeypatch, env):
         g.close()
 
 
+@pytest.mark.parametrize("shape", [(4352, 256, 1, 34, 34, 40, 6, 0), (768, 2048, 2, 12, 12, 64, 8, 1), (288, 768, 2, 6, 6, 64, 8, 1)])
+def test_general_token_kernel_on_shapes_that_have_an_instance_of_their_own(orc, monkeypatch, shape):
+    # rows of 272, 48 and 18 chunks: by default k_token is instantiated with five, one and one chunks per lane for them
+    monkeypatch.setenv("L2J_FUSE", "1")
+    monkeypatch.setenv("L2J_TOKEN_SPECIAL", "0")
+    m, g = make_pair(orc, shape, seed=67, realistic=True)
+    rng = np.random.default_rng(6)
+    for pos, tok in enumerate(rng.integers(0, shape[5], size=shape[6])):
+        assert rel_err(g.forward(int(tok), pos), m.forward(int(tok), pos)) < 1e-4, pos
+
+
 def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
     # a spin limit of zero makes the bounded waits of the whole-token kernel give up at once: every kernel still
     # runs to its end, the call reports the failure, and a context with the normal limit is unaffected
