@@ -354,7 +354,8 @@ struct MatvecRun {
     // vector is staged: the wait for the vector ends when the wave's own requests have arrived, and with the whole row
     // requested ahead all the multiply-adds of the phase would follow after the last arrival instead of overlapping it.
     // Measured per 7B token for W2's six chunks: all ahead 1.573 ms, four 1.551, three 1.568, two 1.556; per 13B token
-    // for the five chunks of QKV and W13: all ahead 3.14 ms, four 2.92, three 2.74, two 2.79; three of QKV's or W13's four
+    // for the five chunks of QKV and W13: all ahead 3.14 ms, four 2.92, three 2.74, two 2.79 (four for QKV and three for W13
+    // 2.89, three and two 2.73, two and three 2.73 against 2.70); three of QKV's or W13's four
     // at the 7B shape: no change.  Wo's row pairs are always requested whole: that phase only waits for its input.
     static constexpr int kAhead = TU == 6 ? kTU : TU == 5 && MODE != PH_RES ? 3 : TU;
     static constexpr bool kSplitAhead = kAhead < TU;
