@@ -136,6 +136,10 @@ int l2j_sampler_seed(l2j_ctx *ctx, int64_t rng_seed);
  * coin: the caller's Random.nextFloat() in [0, 1), or negative to draw from the context's generator (one draw per
  * call, none at temperature 0).  A NaN among the probabilities is an error, as sample_topp throws. */
 int l2j_sample(l2j_ctx *ctx, const float *logits_or_null, float temperature, float topp, float coin, int32_t *next);
+/* Measurement and test: the running float32 sums of n <= 36864 non-negative terms in element order, as the reference's
+ * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
+ * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
+int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
 /* = the token loop of Run.main with a sampler (J/Run.java:599-603, 611-685): as l2j_decode_greedy, but every
  * unforced token is sampled as in l2j_sample from a sampler seeded with rng_seed; the logits never leave the device. */
 int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature,

@@ -537,6 +537,7 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     a.sorted_prob = c->pi_prob[other]; a.sorted_idx = c->pi_idx[other];
     a.st = in_loop ? c->st : nullptr;
     a.out_tokens = c->out_tokens;
+    a.scan = env_int("L2J_SAMPLER_SCAN", 1) != 0 ? 1 : 0;
     const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
     hipLaunchKernelGGL(k_sample_probs, dim3(1), dim3(1024), lds, c->stream, a);
     hipError_t e = hipGetLastError();
@@ -1140,6 +1141,28 @@ int l2j_sample(l2j_ctx *c, const float *logits, float temperature, float topp, f
     HIPCHK(hipStreamSynchronize(c->stream));
     if ((rc = check_sampler_status(c))) return rc;
     *next = c->h_ss->result;
+    return L2J_OK;
+}
+
+int l2j_running_sums(l2j_ctx *c, const float *terms, int32_t n, float *sums)
+{
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+    if (!c || !terms || !sums) return fail(L2J_E_ARG, "null argument");
+    if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "1 to 36864 terms");
+    HIPCHK(hipSetDevice(c->cfg.device));
+    float *d = nullptr;
+    HIPCHK(hipMalloc(reinterpret_cast<void **>(&d), (size_t)n * sizeof(float)));
+    const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
+    hipError_t e = hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e == hipSuccess) e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, env_int("L2J_SAMPLER_SCAN", 1) != 0 ? 1 : 0);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    (void)hipFree(d);
+    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("running sums: ") + hipGetErrorString(e));
     return L2J_OK;
 }
 

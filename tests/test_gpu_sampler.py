@@ -80,6 +80,58 @@ def test_topp_worked_example_with_entries_of_an_earlier_call(orc):
         assert g.sample(1.0, topp, logits=lg, coin=coin) == o.sample_topp(probs, topp, coin=coin)
 
 
+def running_sum_cases():
+    rng = np.random.default_rng(11)
+    n = 32000
+    yield "uniform", rng.random(n)
+    yield "flat softmax", np.exp(rng.standard_normal(n) * 0.05)
+    yield "peaked softmax", np.exp(rng.standard_normal(n) * 6 - 20)
+    yield "forty orders of magnitude", np.exp(rng.uniform(-80, 5, n))
+    yield "sorted descending", np.sort(rng.random(n) / n)[::-1]
+    yield "powers of two (ties)", np.ldexp(1.0, rng.integers(-30, 3, n))
+    yield "3 * powers of two (ties)", 3 * np.ldexp(1.0, rng.integers(-30, 3, n))
+    yield "halves", np.full(n, 0.5)
+    yield "ones, then terms of half an ulp and of three quarters", np.concatenate(
+        [np.ones(9000), np.full(9000, 2.0 ** -11), np.full(9000, 1.5 * 2.0 ** -11)])
+    yield "denormals", np.concatenate([np.full(3000, 1e-45), np.full(3000, 1e-40), rng.random(3000) * 1e-38])
+    yield "half of them zero", np.where(rng.random(n) < 0.5, 0.0, rng.random(n))
+    yield "leading zeros", np.concatenate([np.zeros(5000), rng.random(5000)])
+    yield "every term leaves the binade", np.ldexp(1.0, np.arange(-100, 100))
+    yield "a large term late", np.concatenate([rng.random(20000) * 1e-3, [1e6], rng.random(5000)])
+    for m in (1, 2, 31, 32, 33, 1023, 1024, 1025, 1024 + 8192, 1024 + 8193, 36864):
+        yield "n = %d" % m, rng.random(m)
+
+
+@pytest.mark.parametrize("scan", ["1", "0"])
+def test_running_sums_are_the_sequential_float32_sums(orc, monkeypatch, scan):
+    # numpy's cumsum adds one element after the other in float32: the order of the reference's loops
+    monkeypatch.setenv("L2J_SAMPLER_SCAN", scan)
+    g = small_transformer(64)
+    for name, terms in running_sum_cases():
+        terms = np.asarray(terms, dtype=np.float32)
+        want = np.cumsum(terms, dtype=np.float32)
+        got = g.running_sums(terms)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (name, int(np.argmax(got != want)))
+
+
+@pytest.mark.parametrize("topp", [1.0, 0.9])
+def test_scanned_and_single_lane_sums_pick_the_same_tokens(orc, monkeypatch, topp):
+    vocab = 32000
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(5)
+    for kind in ("flat", "peaked", "mid"):
+        lg = logits_of(rng, vocab, kind)
+        for coin in [0.0, 0.99999994] + [float(np.float32(c)) for c in rng.random(6)]:
+            picks, probs = [], []
+            for scan in ("1", "0"):
+                monkeypatch.setenv("L2J_SAMPLER_SCAN", scan)
+                g.sampler_seed(9)                    # (top-p keeps entries of earlier calls: the same history for both)
+                picks.append(g.sample(0.9, topp, logits=lg, coin=coin))
+                probs.append(g.read(BUFFER.LOGITS))
+            assert picks[0] == picks[1], (kind, coin)
+            assert np.array_equal(probs[0].view(np.uint32), probs[1].view(np.uint32)), kind
+
+
 def test_temperature_zero_is_first_max_and_nan_is_an_error(orc):
     vocab = 1003
     g = small_transformer(vocab)
