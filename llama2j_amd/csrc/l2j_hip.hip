@@ -124,6 +124,7 @@ struct l2j_ctx {
     int pi_cur = 0;                             // which of the two holds the array between calls
     void *sort_temp = nullptr;
     size_t sort_temp_bytes = 0;
+    float *sample_exp = nullptr;   // exp(logit / temperature - max) of one sampling step (k_sample_exp)
 };
 
 namespace {
@@ -471,6 +472,8 @@ void free_sampler(l2j_ctx *c)
     }
     (void)hipFree(c->sort_temp);
     c->sort_temp = nullptr;
+    (void)hipFree(c->sample_exp);
+    c->sample_exp = nullptr;
     if (c->h_ss) (void)hipHostFree(c->h_ss);
     c->h_ss = nullptr;
 }
@@ -487,6 +490,7 @@ int alloc_sampler(l2j_ctx *c)
     HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream));
     c->sort_temp_bytes = bytes;
     HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
+    if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n))) return rc;
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
     const int lds = (((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
     HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -538,6 +542,13 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     a.st = in_loop ? c->st : nullptr;
     a.out_tokens = c->out_tokens;
     a.scan = env_int("L2J_SAMPLER_SCAN", 1) != 0 ? 1 : 0;
+    const int exp_wgs = env_int("L2J_SAMPLER_EXP_WGS", 32);   // 0: the exponentials in k_sample_probs' one workgroup
+    a.expbuf = exp_wgs > 0 ? c->sample_exp : nullptr;
+    if (a.expbuf) {
+        hipLaunchKernelGGL(k_sample_exp, dim3(exp_wgs), dim3(1024), 0, c->stream, a);
+        hipError_t ee = hipGetLastError();
+        if (ee != hipSuccess) return ee;
+    }
     const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
     hipLaunchKernelGGL(k_sample_probs, dim3(1), dim3(1024), lds, c->stream, a);
     hipError_t e = hipGetLastError();

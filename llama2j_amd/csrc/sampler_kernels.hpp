@@ -46,6 +46,7 @@ struct SampleArgs {
     DevState *st;            // token loop (null outside it): the sampled token replaces the argmax
     int *out_tokens;         //   that k_finish stored for position st->pos - 1
     int scan;                // 1: the running sums by windows of equal exponent (chain_scan), 0: one lane adds them all
+    float *expbuf;           // not null: k_sample_exp has left exp(x / temperature - max) here (n floats)
 };
 
 // java.util.Random.nextFloat(): next(24) / (float)(1 << 24)
@@ -167,7 +168,8 @@ __device__ __forceinline__ int first_past(const float *p, const float *ends, int
 // grows through a binade per doubling, so after a short head that one lane adds (where the sum doubles every few terms)
 // a few rounds per tile remain; an input that leaves binades faster than that falls back to the single lane.
 constexpr int kScanHead = 1024;      // terms added by one lane before the scan starts
-constexpr int kScanPer = 8;          // terms per thread and round (measured per sampled 7B token: 4: 1.761, 8: 1.754, 16: 1.777 ms)
+constexpr int kScanPer = 9;          // terms per thread and round; odd: the lanes of a wave then read different LDS banks
+                                     // (measured per sampled 7B token: 7: 1.729, 8: 1.740, 9: 1.730, 13: 1.741 ms)
 constexpr int kScanMaxRounds = 48;
 constexpr int kScanBig = 1 << 25;    // an increment that leaves any binade; sums saturate here
 
@@ -313,7 +315,7 @@ __device__ __forceinline__ int first_over(const float *p, int m, float limit, bo
 {
     if (threadIdx.x == 0) *slot = m;
     __syncthreads();
-    const int per = (m + blockDim.x - 1) / blockDim.x, lo = threadIdx.x * per, hi = min(m, lo + per);
+    const int per = ((m + blockDim.x - 1) / blockDim.x) | 1, lo = min(m, (int)threadIdx.x * per), hi = min(m, lo + per);
     for (int i = lo; i < hi; i++) {
         const float s = p[i];
         if (above ? s > limit : limit < s) { atomicMin(slot, i); break; }
@@ -322,6 +324,27 @@ __device__ __forceinline__ int first_over(const float *p, int m, float limit, bo
     const int r = *slot;
     __syncthreads();
     return r;
+}
+
+// The element-wise front of the step spread over many workgroups (the double-precision exponential of 32000 logits
+// takes 0.04 ms on one compute unit): every workgroup divides all the logits by the temperature and takes the maximum
+// (the same value everywhere: a maximum does not depend on the order), then exponentiates its own slice into expbuf.
+__global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
+{
+    __shared__ float red[16];
+    const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
+    float mx = -__builtin_inff();
+    int bad = 0;
+    for (int i = tid; i < n; i += nt) {
+        const float v = __fdiv_rn(a.logits[i], a.temperature);
+        bad |= v != v;
+        mx = fmaxf(mx, v);
+    }
+    mx = block_max(mx, red);
+    const int per = (n + gridDim.x - 1) / gridDim.x, lo = blockIdx.x * per, hi = min(n, lo + per);
+    for (int i = lo + tid; i < hi; i += nt)
+        a.expbuf[i] = (float)exp((double)__fsub_rn(__fdiv_rn(a.logits[i], a.temperature), mx));
+    if (bad && blockIdx.x == 0) atomicOr(&a.ss->nan, 1);
 }
 
 // J/Run.java:645-659 (divide by the temperature, FindMax, ExpSumNormalize), then either J/Sampler.java:33-44
@@ -338,21 +361,25 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
     const int np = (n + kChainStep - 1) & ~(kChainStep - 1);
 
-    // logits[q] /= temperature; max
-    float mx = -__builtin_inff();
     int bad = 0;
-    for (int i = tid; i < np; i += nt) {
-        float v = 0.0f;
-        if (i < n) {
-            v = __fdiv_rn(a.logits[i], a.temperature);
-            bad |= v != v;
-            mx = fmaxf(mx, v);
+    if (a.expbuf) {
+        for (int i = tid; i < np; i += nt) sp[i] = i < n ? a.expbuf[i] : 0.0f;
+    } else {
+        // logits[q] /= temperature; max
+        float mx = -__builtin_inff();
+        for (int i = tid; i < np; i += nt) {
+            float v = 0.0f;
+            if (i < n) {
+                v = __fdiv_rn(a.logits[i], a.temperature);
+                bad |= v != v;
+                mx = fmaxf(mx, v);
+            }
+            sp[i] = v;
         }
-        sp[i] = v;
+        mx = block_max(mx, red);
+        // x = (float) Math.exp(x - max)
+        for (int i = tid; i < n; i += nt) sp[i] = (float)exp((double)__fsub_rn(sp[i], mx));
     }
-    mx = block_max(mx, red);
-    // x = (float) Math.exp(x - max)
-    for (int i = tid; i < n; i += nt) sp[i] = (float)exp((double)__fsub_rn(sp[i], mx));
     __syncthreads();
     // sum += x, in element order
     if (a.scan) {
@@ -409,7 +436,8 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
 
     // J/Sampler.java:85-96: candidates in index order into the front of the ProbIndex array
     const float cutoff = __fdiv_rn(__fsub_rn(1.0f, a.topp), (float)(n - 1));
-    const int per = (n + nt - 1) / nt, lo = min(n, tid * per), hi = min(n, lo + per);
+    // (an odd number of elements per thread: the lanes of a wave then read different LDS banks)
+    const int per = ((n + nt - 1) / nt) | 1, lo = min(n, tid * per), hi = min(n, lo + per);
     int c = 0;
     for (int i = lo; i < hi; i++) c += sp[i] >= cutoff;
     cnt[tid] = c;
