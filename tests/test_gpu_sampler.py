@@ -148,6 +148,19 @@ def test_temperature_zero_is_first_max_and_nan_is_an_error(orc):
     assert g.sample(1.0, 0.0, logits=lg, coin=0.9) == 17               # ties keep index order; cumulative > 0 at once
 
 
+def test_largest_vocabulary_the_sampler_takes(orc):
+    vocab = 36864
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(8)
+    g.sampler_seed(5)
+    o = orc.Sampler(5, vocab)
+    for kind, topp in (("flat", 0.9), ("peaked", 0.95), ("mid", 1.0), ("flat", 1.0)):
+        lg = logits_of(rng, vocab, kind)
+        want, probs = o.step(lg, 0.9, topp)
+        assert g.sample(0.9, topp, logits=lg) == want, (kind, topp)
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
+
+
 def test_sampler_rejects_a_vocabulary_that_does_not_fit(orc):
     g = small_transformer(40000)
     with pytest.raises(L2JError):
