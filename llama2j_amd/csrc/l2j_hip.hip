@@ -23,8 +23,8 @@ using namespace l2j;
 
 namespace l2j {
 // stable descending sort of (prob, index) pairs; temp == nullptr: only report the scratch size (sampler_sort.hip)
-hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, const float *kin, float *kout, const int *vin, int *vout, unsigned n,
-                                hipStream_t s);
+hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, float *k0, float *k1, int *v0, int *v1, unsigned n, hipStream_t s,
+                                int *in_second);
 }  // namespace l2j
 
 namespace {
@@ -487,7 +487,7 @@ int alloc_sampler(l2j_ctx *c)
         if ((rc = dev_alloc(&c->pi_idx[i], (uint64_t)n))) return rc;
     }
     size_t bytes = 0;
-    HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream));
+    HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream, nullptr));
     c->sort_temp_bytes = bytes;
     HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
     if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n))) return rc;
@@ -554,10 +554,13 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.plain) return e;
     size_t bytes = c->sort_temp_bytes;
+    int in_second = 0;
     e = sort_prob_index_desc(c->sort_temp, &bytes, c->pi_prob[cur], c->pi_prob[other], c->pi_idx[cur], c->pi_idx[other],
-                             (unsigned)n, c->stream);
+                             (unsigned)n, c->stream, &in_second);
     if (e != hipSuccess) return e;
-    c->pi_cur = other;
+    const int sorted = in_second ? other : cur;   // the array stays there until the next call
+    a.sorted_prob = c->pi_prob[sorted]; a.sorted_idx = c->pi_idx[sorted];
+    c->pi_cur = sorted;
     hipLaunchKernelGGL(k_topp_pick, dim3(1), dim3(1024), lds, c->stream, a);
     return hipGetLastError();
 }

@@ -8,10 +8,16 @@
 
 namespace l2j {
 
-hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, const float *kin, float *kout, const int *vin, int *vout, unsigned n,
-                                hipStream_t s)
+// The pairs are in (k0, v0) on entry; either pair of arrays may be overwritten, and *in_second says where the sorted
+// pairs are (with the two buffers handed over as such, rocPRIM need not copy the result into place).
+hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, float *k0, float *k1, int *v0, int *v1, unsigned n, hipStream_t s,
+                                int *in_second)
 {
-    return rocprim::radix_sort_pairs_desc(temp, *temp_bytes, kin, kout, vin, vout, n, 0u, 32u, s, false);
+    rocprim::double_buffer<float> keys(k0, k1);
+    rocprim::double_buffer<int> values(v0, v1);
+    const hipError_t e = rocprim::radix_sort_pairs_desc(temp, *temp_bytes, keys, values, n, 0u, 32u, s, false);
+    if (in_second) *in_second = keys.current() == k1 ? 1 : 0;
+    return e;
 }
 
 }  // namespace l2j
