@@ -45,6 +45,18 @@ def synth_prompt(seed, n, vocab):
     return np.array(out, dtype=np.int32)
 
 
+# HBM bytes per launch of k_token from hardware counters.  bench.py cannot read counters itself (they need a profiler
+# around the process), so this is a labelled constant from the two `rocprofv3 --pmc` runs summarised in
+# profiles/hbm_traffic_llama2-7b.md (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for a
+# 256 MiB copy kernel); it is reported with its source and only for the workload and kernel it was collected on.
+COUNTER_TRAFFIC = {
+    "llama2-7b-shape": {"hbm_bytes_per_launch": 7300987206, "positions": "0-9",
+                        "algorithmic_bytes_at_those_positions": 7209775232,
+                        "source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), profiles/hbm_traffic_llama2-7b.md",
+                        "collected": "2026-11-25"},
+}
+
+
 def cpu_baseline(shape, seed, prompt, gpu_tokens, budget_steps):
     """The CPU oracle (a C restatement of llama2j's CPU mode, same row/head-parallel decomposition,
     OpenMP over the host cores) timed on a bounded sample of the same workload, by the reference's
@@ -56,7 +68,9 @@ def cpu_baseline(shape, seed, prompt, gpu_tokens, budget_steps):
     m.fill_synth(seed, 0.02)
     fill_s = time.time() - t0
     toks, _, sec = m.generate_greedy(prompt, budget_steps)
-    same = bool(np.array_equal(toks, gpu_tokens[:len(toks)]))
+    # only tokens past the prompt are generated (the prompt ids are forced outputs on both sides, J/Run.java:635-642)
+    n_gen = max(0, min(len(toks), len(gpu_tokens)) - len(prompt))
+    same = bool(np.array_equal(toks[len(prompt):len(prompt) + n_gen], gpu_tokens[len(prompt):len(prompt) + n_gen])) if n_gen > 0 else None
     cores = orc.lib().orc_num_threads()
     m.close()
     return {
@@ -66,6 +80,7 @@ def cpu_baseline(shape, seed, prompt, gpu_tokens, budget_steps):
         "kind": "port",
         "sample": "first %d forwards of the same workload (same seeded weights and prompt); C restatement of "
                   "llama2j CPU mode, reference never executed (no JVM); weights generated in %.1f s" % (len(toks), fill_s),
+        "generated_tokens_compared": n_gen,
         "tokens_match_gpu": same,
     }
 
@@ -148,9 +163,10 @@ def main():
         "dtype": "u8 weights x f32 activations (W8A32), f32 accumulate",
         "data": "synthetic: seeded N(0,0.02)-like weights quantized by the reference's group-int8 encoder, seeded prompt ids",
         "config": {"workload": "%s: dim %d, hidden %d, %d layers, %d heads, vocab %d, seq_len %d; batch 1 greedy, "
-                               "%d prompt ids + %d generated%s" % ((a.workload,) + shape[:4] + shape[5:7] +
-                                                                 (n_prompt, steps - n_prompt,
+                               "%d forced prompt positions + %d generated%s" % ((a.workload,) + shape[:4] + shape[5:7] +
+                                                                 (min(n_prompt, steps), max(0, steps - n_prompt),
                                                                   "; timed: the generated positions only" if long_context else "")),
+                   "forced_steps": 0 if long_context else min(n_prompt, done), "generated_steps": max(0, steps - n_prompt),
                    "weights_load_s": round(load_s, 2)},
         "tok_s_reference_rule": round((done - 1) / sec_after_first, 2) if sec_after_first > 0 else None,
         "bytes_per_token": bytes_tok,
@@ -193,22 +209,22 @@ def main():
         out["kernels"] = kern
         dom_name = "token" if "token" in kern else "w13"
         dom = kern[dom_name]
-        traffic = None
-        tpath = os.path.join(ROOT, "profiles", "k_token_llama2-7b_traffic.json")
-        if a.workload == "llama2-7b-shape" and os.path.exists(tpath):
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        ct = COUNTER_TRAFFIC.get(a.workload) if dom_name == "token" else None
         out["roofline"] = {"bound": "hbm",
                            "kernel": "k_token (all phases of all layers + classifier), one launch per token" if dom_name == "token"
                            else "k_matvec<PH_W13> (rmsnorm + W1,W3 matvec + SwiGLU), one launch per layer",
                            "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"],
                            "algorithmic_bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"],
-                           "position": pos, "traffic": traffic}
+                           "position": pos, "traffic": ct["hbm_bytes_per_launch"] if ct else None,
+                           "traffic_source": ("not measured by this run: %s, positions %s (algorithmic bytes there: %d), collected %s" %
+                                              (ct["source"], ct["positions"], ct["algorithmic_bytes_at_those_positions"], ct["collected"]))
+                           if ct else None}
     else:
         out["roofline"] = None
 
+    g_tokens = tokens.copy()
+    g.close()  # graph, events, buffers and stream are released here, before anything of the CPU leg or of exit runs
     if a.cpu_steps > 1:
-        g_tokens = tokens.copy()
-        g.close()
         out["cpu_baseline"] = cpu_baseline(shape, seed, prompt, g_tokens, min(a.cpu_steps, steps))
     else:
         out["cpu_baseline"] = None

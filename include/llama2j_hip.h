@@ -8,8 +8,8 @@
  * names the reference interface it replaces (paths relative to the reference root,
  * J/ = src/main/java/com/lastbot/llama2j/, K/ = J/kernel/).
  *
- * Conventions: plain C, no exceptions cross the boundary, 0 = success and negative = error
- * (the text is in l2j_last_error(), thread local).  Entry points that run the forward pass are
+ * Conventions: plain C, no exceptions cross the boundary, 0 = success and negative = error (the text is
+ * kept per context, l2j_ctx_last_error, and per calling thread, l2j_last_error).  Entry points that run the forward pass are
  * not re-entrant per context, and forwards of different contexts of one process take turns (the
  * whole-token kernel occupies every compute unit); uploads are thread safe (the reference uploads from
  * ten threads, J/TransformerWeights.java:52,204).  There is no CPU fallback: without a GPU l2j_create fails.
@@ -74,8 +74,22 @@ enum l2j_buffer {
 int l2j_create(const l2j_config *cfg, l2j_ctx **out);
 /* = Context.close / RunState.close (J/Run.java:697-701, J/ContextCUDA.java:311-323). */
 void l2j_destroy(l2j_ctx *ctx);
+/* Text of the calling thread's last failed call (also for calls that have no context, l2j_create included). */
 const char *l2j_last_error(void);
+/* Text of the last failed call on this context, whatever thread made it, copied into buf (NUL-terminated, at most
+ * cap - 1 bytes); returns the length.  For callers whose threads move between two downcalls: the reference uploads
+ * from ten virtual threads (J/TransformerWeights.java:52,204) and turns a device error into
+ * RuntimeException(message) (J/ContextCUDA.java:296-304). */
+int l2j_ctx_last_error(l2j_ctx *ctx, char *buf, int32_t cap);
 int l2j_device_count(void);
+/* Launch shapes and algorithm switches of one context, the counterpart of the constants the reference compiles into
+ * its kernels' launch code (the block sizes in the K/ classes, J/Run.java:27-28).  A context starts from the process
+ * defaults (environment variable L2J_<NAME>, read once by l2j_create; unset: the built-in value), this call overrides
+ * one of them, and the library never reads the environment afterwards.  Before l2j_finalize: "threads", "grid",
+ * "attn_threads", "attn_rows", "attn_nsplit", "fused_attn_rows", "fused_attn_splits", "barrier_spins", "fuse" (1 whole-token
+ * kernel, 0 one launch per phase, -1 by model size), "layers_per_launch", "by_value", "token_special", "graph" (0: launch
+ * kernel by kernel instead of replaying a captured hipGraph).  At any time: "sampler_scan", "sampler_exp_wgs". */
+int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
 
 /* = allocateQuantAndCopyToDevice (J/ContextCUDA.java:138-158, J/TransformerWeights.java:238-257).
  * `ref_bytes` is the exact payload of a .quant cache: ceil(n/256) groups of 264 bytes
@@ -95,12 +109,6 @@ int l2j_upload_f32(l2j_ctx *ctx, int tensor, const float *data, uint64_t nfloats
 int l2j_upload_f32_quantize(l2j_ctx *ctx, int tensor, uint64_t first, const float *data, uint64_t nfloats);
 /* Serialises a device tensor back to .quant payload bytes (groups [group0, group0+ngroups)). */
 int l2j_read_quant(l2j_ctx *ctx, int tensor, uint64_t group0, uint64_t ngroups, uint8_t *ref_bytes_out);
-/* Benchmark input: fills every tensor on the device with seeded values
- * ((sum of the four 16-bit fields of splitmix64(seed*0x9E3779B97F4A7C15 + stream*0xD1B54A32D192ED03 + i))
- *  - 131070) * (sigma / 37837.2265625f), stream 0 = embedding, 1..10 = quant tensors in file
- * order, 11 = classifier, and quantizes the ten quant tensors with the reference's encoder. */
-int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
-
 /* Ends the load phase: tables (RoPE K/ApplyRope.java:34-59, SiLU K/Silu.java:47-57) are built,
  * the KV cache is zeroed and the per-token graph is captured. */
 int l2j_finalize(l2j_ctx *ctx);
@@ -136,10 +144,6 @@ int l2j_sampler_seed(l2j_ctx *ctx, int64_t rng_seed);
  * coin: the caller's Random.nextFloat() in [0, 1), or negative to draw from the context's generator (one draw per
  * call, none at temperature 0).  A NaN among the probabilities is an error, as sample_topp throws. */
 int l2j_sample(l2j_ctx *ctx, const float *logits_or_null, float temperature, float topp, float coin, int32_t *next);
-/* Measurement and test: the running float32 sums of n <= 36864 non-negative terms in element order, as the reference's
- * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
- * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
-int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
 /* = the token loop of Run.main with a sampler (J/Run.java:599-603, 611-685): as l2j_decode_greedy, but every
  * unforced token is sampled as in l2j_sample from a sampler seeded with rng_seed; the logits never leave the device. */
 int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature,
@@ -169,20 +173,6 @@ int l2j_read(l2j_ctx *ctx, int which, int layer, uint64_t off, float *dst, uint6
 int l2j_write_kv(l2j_ctx *ctx, int layer, int32_t pos0, int32_t npos, const float *k, const float *v);
 int l2j_sync(l2j_ctx *ctx);
 
-/* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
- * and returns the mean kernel time from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
- * every layer and the classifier in one launch.  The other classes launch one phase of it as a kernel of its
- * own, once per layer (cold weights, as inside a token). */
-enum l2j_kernel_class { L2J_K_QKV = 0, L2J_K_ATTENTION, L2J_K_WO, L2J_K_W13, L2J_K_W2, L2J_K_CLASSIFIER, L2J_K_TOKEN, L2J_K_COUNT };
-int l2j_time_kernel(l2j_ctx *ctx, int kernel_class, int32_t pos, int32_t rounds, double *mean_us,
-                    uint64_t *algorithmic_bytes);
-/* Measurement: runs k_copy16 (reads nbytes, writes nbytes) `rounds` times; hardware byte counters of the
- * other kernels are scaled by what the same counters report for this kernel of known size. */
-int l2j_calibration_copy(l2j_ctx *ctx, uint64_t nbytes, int32_t rounds);
-/* Algorithmic bytes one token streams at position pos: weights in the reference's storage format
- * (264 bytes per 256 weights, fp32 classifier and embedding row) plus KV cache read and write. */
-uint64_t l2j_bytes_per_token(const l2j_config *cfg, int32_t pos);
-
 /* ---- host side of the load path (no GPU needed) ---------------------------------------- */
 /* = Quant.numberOfBytesByFloatSize / Quant.encode / Quant.decode (J/Quant.java:39-48,156-193,79-108). */
 uint64_t l2j_quant_nbytes(uint64_t nfloats);
@@ -202,6 +192,32 @@ int l2j_read_checkpoint_header(const char *bin_path, l2j_config *cfg);
  * quantizes (on the GPU) and, when write_caches != 0, writes the cache; uploads; finalizes. */
 int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int write_caches, l2j_ctx **out);
 int l2j_get_config(l2j_ctx *ctx, l2j_config *cfg);
+
+/* ======================================================================================================
+ * Measurement and test entry points.  Not part of what a Mode.HIP binds: bench.py and the test-suite use them.
+ * ====================================================================================================== */
+/* Benchmark input: fills every tensor on the device with seeded values
+ * ((sum of the four 16-bit fields of splitmix64(seed*0x9E3779B97F4A7C15 + stream*0xD1B54A32D192ED03 + i))
+ *  - 131070) * (sigma / 37837.2265625f), stream 0 = embedding, 1..10 = quant tensors in file
+ * order, 11 = classifier, and quantizes the ten quant tensors with the reference's encoder. */
+int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
+/* Measurement and test: the running float32 sums of n <= 36864 non-negative terms in element order, as the reference's
+ * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
+ * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
+int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
+/* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
+ * and returns the mean kernel time from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
+ * every layer and the classifier in one launch.  The other classes launch one phase of it as a kernel of its
+ * own, once per layer (cold weights, as inside a token). */
+enum l2j_kernel_class { L2J_K_QKV = 0, L2J_K_ATTENTION, L2J_K_WO, L2J_K_W13, L2J_K_W2, L2J_K_CLASSIFIER, L2J_K_TOKEN, L2J_K_COUNT };
+int l2j_time_kernel(l2j_ctx *ctx, int kernel_class, int32_t pos, int32_t rounds, double *mean_us,
+                    uint64_t *algorithmic_bytes);
+/* Measurement: runs k_copy16 (reads nbytes, writes nbytes) `rounds` times; hardware byte counters of the
+ * other kernels are scaled by what the same counters report for this kernel of known size. */
+int l2j_calibration_copy(l2j_ctx *ctx, uint64_t nbytes, int32_t rounds);
+/* Algorithmic bytes one token streams at position pos: weights in the reference's storage format
+ * (264 bytes per 256 weights, fp32 classifier and embedding row) plus KV cache read and write. */
+uint64_t l2j_bytes_per_token(const l2j_config *cfg, int32_t pos);
 
 #ifdef __cplusplus
 }

@@ -8,9 +8,11 @@ Reference classes mirrored (J/ = src/main/java/com/lastbot/llama2j/ in the refer
 Errors become exceptions carrying the library's message, as the reference turns CUDA errors into
 RuntimeException (J/ContextCUDA.java:296-304).
 """
+import atexit
 import ctypes as C
 import os
 import subprocess
+import weakref
 
 import numpy as np
 
@@ -85,6 +87,8 @@ def _signatures():
         "l2j_create": (C.c_int, [cfgp, C.POINTER(vp)]),
         "l2j_destroy": (None, [vp]),
         "l2j_last_error": (C.c_char_p, []),
+        "l2j_ctx_last_error": (C.c_int, [vp, C.c_char_p, C.c_int32]),
+        "l2j_set_option": (C.c_int, [vp, C.c_char_p, C.c_int32]),
         "l2j_device_count": (C.c_int, []),
         "l2j_upload_quant": (C.c_int, [vp, C.c_int, u8p, C.c_uint64]),
         "l2j_upload_quant_layer": (C.c_int, [vp, C.c_int, C.c_int, u8p, C.c_uint64]),
@@ -254,18 +258,50 @@ class Tokenizer:
             pass
 
 
+_live = weakref.WeakSet()
+
+
+@atexit.register
+def _close_live():
+    """Contexts still open at interpreter exit are destroyed here, while the HIP runtime is still whole: graph,
+    events, buffers and stream go before any library's own exit handlers run."""
+    for t in list(_live):
+        t.close()
+
+
 class Transformer:
     """Weights + run state + forward on the GPU (TransformerWeights, RunState, Run.transformer)."""
 
-    def __init__(self, config=None, _handle=None):
+    def __init__(self, config=None, _handle=None, options=None):
+        """options: {name: int} passed to l2j_set_option before anything else (launch shapes, see the header)."""
         L = lib()
         if _handle is None:
             h = C.c_void_p()
             _check(L.l2j_create(C.byref(config), C.byref(h)))
             _handle = h
         self._h = _handle
+        _live.add(self)
         self.config = Config()
-        _check(L.l2j_get_config(self._h, C.byref(self.config)))
+        self._check(L.l2j_get_config(self._h, C.byref(self.config)))
+        for k, v in (options or {}).items():
+            self.set_option(k, v)
+
+    def _check(self, rc):
+        """Negative return codes become L2JError with the context's own error text (l2j_ctx_last_error: right
+        whatever thread made the failing call)."""
+        if rc < 0:
+            buf = C.create_string_buffer(1024)
+            n = lib().l2j_ctx_last_error(self._h, buf, len(buf)) if self._h else -1
+            raise L2JError(rc, buf.value.decode(errors="replace") if n >= 0 else lib().l2j_last_error().decode(errors="replace"))
+        return rc
+
+    def last_error(self):
+        buf = C.create_string_buffer(1024)
+        self._check(lib().l2j_ctx_last_error(self._h, buf, len(buf)))
+        return buf.value.decode(errors="replace")
+
+    def set_option(self, name, value):
+        self._check(lib().l2j_set_option(self._h, name.encode(), int(value)))
 
     @classmethod
     def from_checkpoint(cls, bin_path, device=0, flags=0, write_caches=True):
@@ -278,6 +314,7 @@ class Transformer:
         if getattr(self, "_h", None):
             lib().l2j_destroy(self._h)
             self._h = None
+            _live.discard(self)
 
     def __del__(self):
         try:
@@ -294,49 +331,49 @@ class Transformer:
     # ---- load phase
     def upload_quant(self, tensor, ref_bytes):
         b = np.ascontiguousarray(ref_bytes, dtype=np.uint8)
-        _check(lib().l2j_upload_quant(self._h, tensor, _u8(b), b.size))
+        self._check(lib().l2j_upload_quant(self._h, tensor, _u8(b), b.size))
 
     def upload_quant_layer(self, tensor, layer, ref_bytes):
         b = np.ascontiguousarray(ref_bytes, dtype=np.uint8)
-        _check(lib().l2j_upload_quant_layer(self._h, tensor, layer, _u8(b), b.size))
+        self._check(lib().l2j_upload_quant_layer(self._h, tensor, layer, _u8(b), b.size))
 
     def upload_f32(self, tensor, values):
         v = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
-        _check(lib().l2j_upload_f32(self._h, tensor, _fp(v), v.size))
+        self._check(lib().l2j_upload_f32(self._h, tensor, _fp(v), v.size))
 
     def upload_f32_quantize(self, tensor, values, first=0):
         v = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
-        _check(lib().l2j_upload_f32_quantize(self._h, tensor, first, _fp(v), v.size))
+        self._check(lib().l2j_upload_f32_quantize(self._h, tensor, first, _fp(v), v.size))
 
     def read_quant(self, tensor, group0, ngroups):
         out = np.empty(ngroups * 264, dtype=np.uint8)
-        _check(lib().l2j_read_quant(self._h, tensor, group0, ngroups, _u8(out)))
+        self._check(lib().l2j_read_quant(self._h, tensor, group0, ngroups, _u8(out)))
         return out
 
     def fill_synthetic(self, seed, sigma=0.02):
-        _check(lib().l2j_fill_synthetic(self._h, seed, C.c_float(sigma)))
+        self._check(lib().l2j_fill_synthetic(self._h, seed, C.c_float(sigma)))
 
     def finalize(self):
-        _check(lib().l2j_finalize(self._h))
+        self._check(lib().l2j_finalize(self._h))
 
     def reset(self):
-        _check(lib().l2j_reset(self._h))
+        self._check(lib().l2j_reset(self._h))
 
     # ---- forward
     def forward(self, token, pos, want_logits=True):
         """Run.transformer(token, pos, ...) + the logits copy (J/Run.java:625-632)."""
         logits = np.empty(self.config.vocab_size, dtype=np.float32) if want_logits else None
-        _check(lib().l2j_forward(self._h, token, pos, _fp(logits) if want_logits else None))
+        self._check(lib().l2j_forward(self._h, token, pos, _fp(logits) if want_logits else None))
         return logits
 
     def forward_argmax(self, token, pos):
         nxt = C.c_int32(-1)
-        _check(lib().l2j_forward_argmax(self._h, token, pos, C.byref(nxt)))
+        self._check(lib().l2j_forward_argmax(self._h, token, pos, C.byref(nxt)))
         return nxt.value
 
     def forward_taps(self, token, pos):
         logits = np.empty(self.config.vocab_size, dtype=np.float32)
-        _check(lib().l2j_forward_taps(self._h, token, pos, _fp(logits)))
+        self._check(lib().l2j_forward_taps(self._h, token, pos, _fp(logits)))
         return logits
 
     def decode_greedy(self, prompt, steps):
@@ -346,12 +383,12 @@ class Transformer:
         out = np.zeros(cap, dtype=np.int32)
         n = C.c_int32(0)
         sec = C.c_double(0.0)
-        _check(lib().l2j_decode_greedy(self._h, _i32(p), p.size, steps, _i32(out), C.byref(n), C.byref(sec)))
+        self._check(lib().l2j_decode_greedy(self._h, _i32(p), p.size, steps, _i32(out), C.byref(n), C.byref(sec)))
         return out[:n.value], sec.value
 
     def sampler_seed(self, rng_seed):
         """new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31): java.util.Random(seed), empty ProbIndex array."""
-        _check(lib().l2j_sampler_seed(self._h, rng_seed))
+        self._check(lib().l2j_sampler_seed(self._h, rng_seed))
 
     def sample(self, temperature, topp, logits=None, coin=None):
         """The sampling step of J/Run.java:643-665 on the device.  logits: an array to sample from instead of the
@@ -363,7 +400,7 @@ class Transformer:
             if logits.size != self.config.vocab_size:
                 raise ValueError("logits must hold vocab_size floats")
             lp = _fp(logits)
-        _check(lib().l2j_sample(self._h, lp, temperature, topp, -1.0 if coin is None else coin, C.byref(nxt)))
+        self._check(lib().l2j_sample(self._h, lp, temperature, topp, -1.0 if coin is None else coin, C.byref(nxt)))
         return nxt.value
 
     def running_sums(self, terms):
@@ -371,7 +408,7 @@ class Transformer:
         softmax denominator and cdf loops), by the routine the device sampler uses."""
         terms = np.ascontiguousarray(terms, dtype=np.float32)
         out = np.empty_like(terms)
-        _check(lib().l2j_running_sums(self._h, _fp(terms), terms.size, _fp(out)))
+        self._check(lib().l2j_running_sums(self._h, _fp(terms), terms.size, _fp(out)))
         return out
 
     def decode_sample(self, prompt, steps, temperature, topp, rng_seed):
@@ -381,7 +418,7 @@ class Transformer:
         out = np.zeros(cap, dtype=np.int32)
         n = C.c_int32(0)
         sec = C.c_double(0.0)
-        _check(lib().l2j_decode_sample(self._h, _i32(p), p.size, steps, temperature, topp, rng_seed, _i32(out),
+        self._check(lib().l2j_decode_sample(self._h, _i32(p), p.size, steps, temperature, topp, rng_seed, _i32(out),
                                        C.byref(n), C.byref(sec)))
         return out[:n.value], sec.value
 
@@ -391,26 +428,26 @@ class Transformer:
             n = {BUFFER.HB: c.hidden_dim, BUFFER.K: c.kv_dim, BUFFER.V: c.kv_dim, BUFFER.LOGITS: c.vocab_size,
                  BUFFER.KCACHE: c.seq_len * c.kv_dim, BUFFER.VCACHE: c.seq_len * c.kv_dim}.get(which, c.dim) - off
         out = np.empty(n, dtype=np.float32)
-        _check(lib().l2j_read(self._h, which, layer, off, _fp(out), n))
+        self._check(lib().l2j_read(self._h, which, layer, off, _fp(out), n))
         return out
 
     def write_kv(self, layer, pos0, k, v):
         k = np.ascontiguousarray(k, dtype=np.float32).reshape(-1)
         v = np.ascontiguousarray(v, dtype=np.float32).reshape(-1)
         assert k.size == v.size and k.size % self.config.kv_dim == 0
-        _check(lib().l2j_write_kv(self._h, layer, pos0, k.size // self.config.kv_dim, _fp(k), _fp(v)))
+        self._check(lib().l2j_write_kv(self._h, layer, pos0, k.size // self.config.kv_dim, _fp(k), _fp(v)))
 
     def sync(self):
-        _check(lib().l2j_sync(self._h))
+        self._check(lib().l2j_sync(self._h))
 
     def time_kernel(self, kernel_class, pos, rounds=3):
         us = C.c_double(0)
         b = C.c_uint64(0)
-        _check(lib().l2j_time_kernel(self._h, kernel_class, pos, rounds, C.byref(us), C.byref(b)))
+        self._check(lib().l2j_time_kernel(self._h, kernel_class, pos, rounds, C.byref(us), C.byref(b)))
         return us.value, b.value
 
     def calibration_copy(self, nbytes, rounds=3):
-        _check(lib().l2j_calibration_copy(self._h, nbytes, rounds))
+        self._check(lib().l2j_calibration_copy(self._h, nbytes, rounds))
 
     def bytes_per_token(self, pos):
         return int(lib().l2j_bytes_per_token(C.byref(self.config), pos))

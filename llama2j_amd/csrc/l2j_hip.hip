@@ -53,16 +53,55 @@ struct QTensor {
     uint64_t groups_loaded = 0;
 };
 
-int env_int(const char *name, int dflt)
+// Launch-shape and algorithm switches of a context.  kAuto = the library picks (by shape, at l2j_finalize).  A context
+// starts from the process defaults (environment variable L2J_<NAME IN CAPITALS>, read once by l2j_create) and
+// l2j_set_option overrides them per context; nothing reads the environment afterwards.
+enum {
+    OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
+    OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
+    OPT_GRAPH, OPT_COUNT
+};
+constexpr int kAuto = -1;
+struct OptionDef {
+    const char *name;
+    int dflt;
+    bool after_finalize;  // may still be changed once the launch shapes are fixed
+};
+const OptionDef kOptions[OPT_COUNT] = {
+    {"threads", 1024, false},          // workgroup size of the weight-streaming kernels
+    {"grid", kAuto, false},            // their workgroups (auto: one per compute unit)
+    {"attn_threads", 256, false},      // k_attention as a kernel of its own
+    {"attn_rows", 32, false},
+    {"attn_nsplit", 32, false},
+    {"fused_attn_rows", 64, false},    // cache rows per attention split inside k_token
+    {"fused_attn_splits", kAuto, false},
+    {"barrier_spins", 20000, false},    // polls of a bounded wait inside k_token before it gives up
+    {"fuse", kAuto, false},            // 1: whole-token kernel, 0: one launch per phase (auto: by layer size)
+    {"layers_per_launch", kAuto, false},
+    {"by_value", 1, false},            // k_token hands vectors over by value (0: grid barriers)
+    {"token_special", 1, false},       // use the k_token instances specialised for the published shapes
+    {"sampler_scan", 1, true},         // running sums by the parallel scan (0: one lane, element after element)
+    {"sampler_exp_wgs", 32, true},     // workgroups of k_sample_exp (0: the exponentials in k_sample_probs)
+    {"graph", 1, false},               // 1: replay a captured hipGraph per token, 0: launch the kernels one by one
+};
+
+int option_from_env(int i)
 {
-    const char *v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
+    char var[64] = "L2J_";
+    size_t k = 4;
+    for (const char *p = kOptions[i].name; *p && k + 1 < sizeof(var); p++) var[k++] = (char)toupper((unsigned char)*p);
+    var[k] = 0;
+    const char *v = getenv(var);
+    return v && *v ? atoi(v) : kOptions[i].dflt;
 }
 
 }  // namespace
 
 struct l2j_ctx {
     l2j_config cfg{};
+    std::mutex err_mu;
+    std::string last_err;  // text of the last failed call on this context, whatever thread made it
+    int opt[OPT_COUNT];
     int head_size = 0, kv_dim = 0, kv_mul = 0;
     int n_cu = 256;
     hipStream_t stream = nullptr;
@@ -109,7 +148,6 @@ struct l2j_ctx {
     bool by_value = false;        // k_token hands activations over by value (no grid barriers)
     float *knew = nullptr, *vnew = nullptr;  // this token's k and v rows per layer
     uint64_t skv = 0;
-    int barrier_spins = 20000;    // polls of a grid barrier before it gives up (each poll is a memory round trip, >= 1 us)
     TokenGeom geom{};             // set by l2j_finalize
 
     hipGraph_t graph = nullptr;
@@ -128,6 +166,18 @@ struct l2j_ctx {
 };
 
 namespace {
+
+// Every entry point that takes a context passes its return code through here: the text of a failure is kept in the
+// context as well as in the calling thread, so that a caller whose threads migrate between calls (Java virtual threads)
+// can fetch it with l2j_ctx_last_error.
+int ctx_rc(l2j_ctx *c, int rc)
+{
+    if (rc < 0 && c) {
+        std::lock_guard<std::mutex> lock(c->err_mu);
+        c->last_err = g_err;
+    }
+    return rc;
+}
 
 uint64_t tensor_floats(const l2j_config &c, int t)
 {
@@ -238,7 +288,8 @@ bool geom_complete(const TokenGeom &t)
 // Splits per attention head inside k_token: one (head, split) item per workgroup at most.
 int fused_splits(const l2j_ctx *c)
 {
-    return std::max(1, env_int("L2J_FUSED_ATTN_SPLITS", std::max(1, c->pk_grid / c->cfg.n_heads)));
+    const int o = c->opt[OPT_FUSED_ATTN_SPLITS];
+    return std::max(1, o != kAuto ? o : c->pk_grid / c->cfg.n_heads);
 }
 
 // Marks every activation vector of a token unwritten (before a k_token that hands over by value).
@@ -260,7 +311,7 @@ auto with_token_kernel(const l2j_ctx *c, F f)
 {
     const int lpr = attn_lpr(c);
     const int tud = tu_for(c->cfg.dim), tuh = tu_for(c->cfg.hidden_dim);
-    const bool special = env_int("L2J_TOKEN_SPECIAL", 1) != 0;
+    const bool special = c->opt[OPT_TOKEN_SPECIAL] != 0;
     if (special && lpr == 16 && tud == 1 && tuh == 1) return f(k_token<16, 1, 1>);
     if (special && lpr == 16 && tud == 1 && tuh == 2) return f(k_token<16, 1, 2>);
     if (special && lpr == 32 && tud == 5) return f(k_token<32, 5, kTU>);
@@ -278,7 +329,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.l0 = l0; a.l1 = l1; a.with_cls = l1 == c->cfg.n_layers;
     a.attn_rows = c->fused_attn_rows;
     a.attn_splits = fused_splits(c);
-    a.maxspin = c->barrier_spins;
+    a.maxspin = std::max(0, c->opt[OPT_BARRIER_SPINS]);  // each poll is a memory round trip, >= 1 us
     a.by_value = c->by_value ? 1 : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
@@ -382,8 +433,8 @@ hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
     return hipGetLastError();
 }
 
-// L2J_MODE=eager launches the kernels one by one instead of replaying the graph (for tools that do not
-// follow graph launches).
+// With option "graph" = 0 the kernels are launched one by one instead of replaying the graph (for tools that do
+// not follow graph launches).
 hipError_t launch_one_token(l2j_ctx *c)
 {
     return c->graph_exec ? hipGraphLaunch(c->graph_exec, c->stream) : launch_token(c, c->stream, false);
@@ -541,8 +592,8 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     a.sorted_prob = c->pi_prob[other]; a.sorted_idx = c->pi_idx[other];
     a.st = in_loop ? c->st : nullptr;
     a.out_tokens = c->out_tokens;
-    a.scan = env_int("L2J_SAMPLER_SCAN", 1) != 0 ? 1 : 0;
-    const int exp_wgs = env_int("L2J_SAMPLER_EXP_WGS", 32);   // 0: the exponentials in k_sample_probs' one workgroup
+    a.scan = c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0;
+    const int exp_wgs = std::min(1024, std::max(0, c->opt[OPT_SAMPLER_EXP_WGS]));   // 0: the exponentials in k_sample_probs' one workgroup
     a.expbuf = exp_wgs > 0 ? c->sample_exp : nullptr;
     if (a.expbuf) {
         hipLaunchKernelGGL(k_sample_exp, dim3(exp_wgs), dim3(1024), 0, c->stream, a);
@@ -657,6 +708,16 @@ const char *l2j_last_error(void) { return g_err.c_str(); }
 
 void l2j_set_error_(const char *msg) { g_err = msg ? msg : ""; }
 
+int l2j_ctx_last_error(l2j_ctx *c, char *buf, int32_t cap)
+{
+    if (!c || !buf || cap <= 0) return fail(L2J_E_ARG, "null argument");
+    std::lock_guard<std::mutex> lock(c->err_mu);
+    const size_t n = std::min(c->last_err.size(), (size_t)cap - 1);
+    memcpy(buf, c->last_err.data(), n);
+    buf[n] = 0;
+    return (int)n;
+}
+
 int l2j_device_count(void)
 {
     int n = 0;
@@ -679,6 +740,7 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     l2j_ctx *c = new (std::nothrow) l2j_ctx();
     if (!c) return fail(L2J_E_OOM, "l2j_create: host allocation failed");
     c->cfg = *cfg;
+    for (int i = 0; i < OPT_COUNT; i++) c->opt[i] = option_from_env(i);
     c->head_size = cfg->dim / cfg->n_heads;
     c->kv_dim = cfg->n_kv_heads * c->head_size;
     c->kv_mul = cfg->n_heads / cfg->n_kv_heads;
@@ -750,12 +812,30 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     return L2J_OK;
 }
 
+// What l2j_finalize allocates (also after a finalize that failed part-way, so that it can be called again).
+static void release_finalize(l2j_ctx *c)
+{
+    destroy_graph(c);
+    (void)hipFree(c->cls_val);
+    (void)hipFree(c->cls_idx);
+    (void)hipFree(c->attn_part);
+    (void)hipFree(c->rmsw);
+    (void)hipFree(c->bar_ctr);
+    (void)hipFree(c->fault);
+    if (c->h_fault) (void)hipHostFree(c->h_fault);
+    c->cls_val = nullptr; c->cls_idx = nullptr; c->attn_part = nullptr; c->rmsw = nullptr; c->bar_ctr = nullptr;
+    c->fault = nullptr; c->h_fault = nullptr;
+}
+
 void l2j_destroy(l2j_ctx *c)
 {
     if (!c) return;
+    // Order: nothing of the context may still run, then the graph (its nodes name kernels and buffers of the
+    // context), the events, the buffers, and the stream last.
+    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
     (void)hipSetDevice(c->cfg.device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    destroy_graph(c);
+    release_finalize(c);
     for (hipEvent_t ev : c->events) (void)hipEventDestroy(ev);
     for (int t = 0; t < L2J_TENSOR_COUNT; t++) {
         (void)hipFree(c->qt[t].codes);
@@ -767,20 +847,13 @@ void l2j_destroy(l2j_ctx *c)
     float *bufs[] = {c->x, c->xb, c->hb, c->q, c->logits, c->kcache, c->vcache, c->silu};
     for (float *b : bufs) (void)hipFree(b);
     (void)hipFree(c->rope);
-    (void)hipFree(c->cls_val);
-    (void)hipFree(c->cls_idx);
-    (void)hipFree(c->attn_part);
-    (void)hipFree(c->rmsw);
     (void)hipFree(c->counters);
     (void)hipFree(c->knew);
     (void)hipFree(c->vnew);
     (void)hipFree(c->st);
     (void)hipFree(c->prompt);
     (void)hipFree(c->out_tokens);
-    (void)hipFree(c->bar_ctr);
-    (void)hipFree(c->fault);
     free_sampler(c);
-    if (c->h_fault) (void)hipHostFree(c->h_fault);
     for (float *t : c->taps) (void)hipFree(t);
     if (c->h_st) (void)hipHostFree(c->h_st);
     if (c->h_tokens) (void)hipHostFree(c->h_tokens);
@@ -788,14 +861,33 @@ void l2j_destroy(l2j_ctx *c)
     delete c;
 }
 
-int l2j_get_config(l2j_ctx *c, l2j_config *cfg)
+int l2j_set_option(l2j_ctx *c, const char *name, int32_t value)
 {
-    if (!c || !cfg) return fail(L2J_E_ARG, "null argument");
-    *cfg = c->cfg;
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !name) return fail(L2J_E_ARG, "null argument");
+        for (int i = 0; i < OPT_COUNT; i++) {
+            if (strcmp(name, kOptions[i].name) != 0) continue;
+            std::lock_guard<std::mutex> lock(c->upload_mu);
+            if (c->finalized && !kOptions[i].after_finalize)
+                return fail(L2J_E_STATE, std::string("option '") + name + "' fixes a launch shape: set it before l2j_finalize");
+            c->opt[i] = value;
+            return L2J_OK;
+        }
+        return fail(L2J_E_ARG, std::string("unknown option '") + name + "'");
+    }());
 }
 
-static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t ngroups, const uint8_t *bytes, uint64_t nbytes)
+int l2j_get_config(l2j_ctx *c, l2j_config *cfg)
+{
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !cfg) return fail(L2J_E_ARG, "null argument");
+        *cfg = c->cfg;
+        return L2J_OK;
+    }());
+}
+
+// whole: the call replaces the tensor (its count of loaded groups starts again)
+static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t ngroups, const uint8_t *bytes, uint64_t nbytes, bool whole)
 {
     if (nbytes != ngroups * kGroupBytes)
         return fail(L2J_E_SIZE, "totalByteSize != quant.numberOfBytesByFloatSize(floatSize)");
@@ -803,6 +895,7 @@ static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t 
     if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
     HIPCHK(hipSetDevice(c->cfg.device));
     QTensor &t = c->qt[tensor];
+    if (whole) t.groups_loaded = 0;
     int rc = unpack_into(c, t, group0, bytes, ngroups);
     if (rc == L2J_OK) t.groups_loaded += ngroups;
     return rc;
@@ -810,441 +903,491 @@ static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t 
 
 int l2j_upload_quant(l2j_ctx *c, int tensor, const uint8_t *ref_bytes, uint64_t nbytes)
 {
-    if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
-    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
-    c->qt[tensor].groups_loaded = 0;
-    return upload_quant_range(c, tensor, 0, c->qt[tensor].ngroups, ref_bytes, nbytes);
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
+        if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+        return upload_quant_range(c, tensor, 0, c->qt[tensor].ngroups, ref_bytes, nbytes, true);
+    }());
 }
 
 int l2j_upload_quant_layer(l2j_ctx *c, int tensor, int layer, const uint8_t *ref_bytes, uint64_t nbytes)
 {
-    if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
-    if (!is_quant(tensor) || !per_layer(tensor)) return fail(L2J_E_ARG, "not a per-layer quantized tensor");
-    if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
-    const uint64_t per = c->qt[tensor].nfloats / c->cfg.n_layers;
-    if (per % kGroup) return fail(L2J_E_ARG, "layer size is not a multiple of the group size; upload the whole tensor");
-    return upload_quant_range(c, tensor, (uint64_t)layer * (per / kGroup), per / kGroup, ref_bytes, nbytes);
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !ref_bytes) return fail(L2J_E_ARG, "null argument");
+        if (!is_quant(tensor) || !per_layer(tensor)) return fail(L2J_E_ARG, "not a per-layer quantized tensor");
+        if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        const uint64_t per = c->qt[tensor].nfloats / c->cfg.n_layers;
+        if (per % kGroup) return fail(L2J_E_ARG, "layer size is not a multiple of the group size; upload the whole tensor");
+        return upload_quant_range(c, tensor, (uint64_t)layer * (per / kGroup), per / kGroup, ref_bytes, nbytes, false);
+    }());
 }
 
 int l2j_upload_f32(l2j_ctx *c, int tensor, const float *data, uint64_t nfloats)
 {
-    if (!c || !data) return fail(L2J_E_ARG, "null argument");
-    if (tensor != L2J_TOK_EMB && tensor != L2J_WCLS) return fail(L2J_E_ARG, "only the embedding and the classifier are fp32");
-    if (nfloats != (uint64_t)c->cfg.vocab_size * c->cfg.dim) return fail(L2J_E_SIZE, "float count != vocab_size * dim");
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    if (tensor == L2J_WCLS && c->cfg.shared_weights) return L2J_OK;  // J/TransformerWeights.java:122
-    HIPCHK(hipMemcpy(tensor == L2J_TOK_EMB ? c->emb : c->wcls, data, nfloats * sizeof(float), hipMemcpyHostToDevice));
-    (tensor == L2J_TOK_EMB ? c->emb_loaded : c->wcls_loaded) = true;
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !data) return fail(L2J_E_ARG, "null argument");
+        if (tensor != L2J_TOK_EMB && tensor != L2J_WCLS) return fail(L2J_E_ARG, "only the embedding and the classifier are fp32");
+        if (nfloats != (uint64_t)c->cfg.vocab_size * c->cfg.dim) return fail(L2J_E_SIZE, "float count != vocab_size * dim");
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        if (tensor == L2J_WCLS && c->cfg.shared_weights) return L2J_OK;  // J/TransformerWeights.java:122
+        HIPCHK(hipMemcpy(tensor == L2J_TOK_EMB ? c->emb : c->wcls, data, nfloats * sizeof(float), hipMemcpyHostToDevice));
+        (tensor == L2J_TOK_EMB ? c->emb_loaded : c->wcls_loaded) = true;
+        return L2J_OK;
+    }());
 }
 
 int l2j_upload_f32_quantize(l2j_ctx *c, int tensor, uint64_t first, const float *data, uint64_t nfloats)
 {
-    if (!c || !data) return fail(L2J_E_ARG, "null argument");
-    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
-    QTensor &t = c->qt[tensor];
-    if (first % kGroup) return fail(L2J_E_ARG, "first must be a multiple of the group size");
-    if (first + nfloats > t.nfloats) return fail(L2J_E_SIZE, "range exceeds the tensor");
-    if (nfloats % kGroup && first + nfloats != t.nfloats) return fail(L2J_E_ARG, "only the tensor's tail may be a partial group");
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const uint64_t slice = 16ull << 20;  // floats per staging slice (64 MiB)
-    float *stage = nullptr;
-    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(slice, std::max<uint64_t>(nfloats, 1)) * sizeof(float)));
-    int rc = L2J_OK;
-    for (uint64_t o = 0; o < nfloats && rc == L2J_OK; o += slice) {
-        const uint64_t nf = std::min(slice, nfloats - o);
-        const uint64_t ng = (nf + kGroup - 1) / kGroup;
-        hipError_t e = hipMemcpy(stage, data + o, nf * sizeof(float), hipMemcpyHostToDevice);
-        if (e == hipSuccess) {
-            hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(256), 0, c->stream, stage, (long)nf,
-                               (long)((first + o) / kGroup), (long)ng, (long)t.nfloats, 0ull, 0.0f, t.codes, t.gs, t.mm);
-            e = hipGetLastError();
-            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !data) return fail(L2J_E_ARG, "null argument");
+        if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+        QTensor &t = c->qt[tensor];
+        if (first % kGroup) return fail(L2J_E_ARG, "first must be a multiple of the group size");
+        if (first + nfloats > t.nfloats) return fail(L2J_E_SIZE, "range exceeds the tensor");
+        if (nfloats % kGroup && first + nfloats != t.nfloats) return fail(L2J_E_ARG, "only the tensor's tail may be a partial group");
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const uint64_t slice = 16ull << 20;  // floats per staging slice (64 MiB)
+        float *stage = nullptr;
+        HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(slice, std::max<uint64_t>(nfloats, 1)) * sizeof(float)));
+        int rc = L2J_OK;
+        for (uint64_t o = 0; o < nfloats && rc == L2J_OK; o += slice) {
+            const uint64_t nf = std::min(slice, nfloats - o);
+            const uint64_t ng = (nf + kGroup - 1) / kGroup;
+            hipError_t e = hipMemcpy(stage, data + o, nf * sizeof(float), hipMemcpyHostToDevice);
+            if (e == hipSuccess) {
+                hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(256), 0, c->stream, stage, (long)nf,
+                                   (long)((first + o) / kGroup), (long)ng, (long)t.nfloats, 0ull, 0.0f, t.codes, t.gs, t.mm);
+                e = hipGetLastError();
+                if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+            }
+            if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("quantize: ") + hipGetErrorString(e));
+            else t.groups_loaded += ng;
         }
-        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("quantize: ") + hipGetErrorString(e));
-        else t.groups_loaded += ng;
-    }
-    (void)hipFree(stage);
-    return rc;
+        (void)hipFree(stage);
+        return rc;
+    }());
 }
 
 int l2j_read_quant(l2j_ctx *c, int tensor, uint64_t group0, uint64_t ngroups, uint8_t *out)
 {
-    if (!c || !out) return fail(L2J_E_ARG, "null argument");
-    if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
-    QTensor &t = c->qt[tensor];
-    if (group0 + ngroups > t.ngroups) return fail(L2J_E_SIZE, "group range exceeds the tensor");
-    if (ngroups == 0) return L2J_OK;
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const uint64_t slice_groups = (64ull << 20) / kGroupBytes;
-    uint8_t *stage = nullptr;
-    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(ngroups, slice_groups) * kGroupBytes));
-    int rc = L2J_OK;
-    for (uint64_t g = 0; g < ngroups && rc == L2J_OK; g += slice_groups) {
-        const uint64_t ng = std::min(slice_groups, ngroups - g);
-        hipLaunchKernelGGL(k_pack_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(64), 0, c->stream, stage, (long)ng,
-                           t.codes + (group0 + g) * kGroup, t.mm + group0 + g);
-        hipError_t e = hipGetLastError();
-        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
-        if (e == hipSuccess) e = hipMemcpy(out + g * kGroupBytes, stage, ng * kGroupBytes, hipMemcpyDeviceToHost);
-        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("read_quant: ") + hipGetErrorString(e));
-    }
-    (void)hipFree(stage);
-    return rc;
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !out) return fail(L2J_E_ARG, "null argument");
+        if (!is_quant(tensor)) return fail(L2J_E_ARG, "not a quantized tensor");
+        QTensor &t = c->qt[tensor];
+        if (group0 + ngroups > t.ngroups) return fail(L2J_E_SIZE, "group range exceeds the tensor");
+        if (ngroups == 0) return L2J_OK;
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const uint64_t slice_groups = (64ull << 20) / kGroupBytes;
+        uint8_t *stage = nullptr;
+        HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(ngroups, slice_groups) * kGroupBytes));
+        int rc = L2J_OK;
+        for (uint64_t g = 0; g < ngroups && rc == L2J_OK; g += slice_groups) {
+            const uint64_t ng = std::min(slice_groups, ngroups - g);
+            hipLaunchKernelGGL(k_pack_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(64), 0, c->stream, stage, (long)ng,
+                               t.codes + (group0 + g) * kGroup, t.mm + group0 + g);
+            hipError_t e = hipGetLastError();
+            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+            if (e == hipSuccess) e = hipMemcpy(out + g * kGroupBytes, stage, ng * kGroupBytes, hipMemcpyDeviceToHost);
+            if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("read_quant: ") + hipGetErrorString(e));
+        }
+        (void)hipFree(stage);
+        return rc;
+    }());
 }
 
 int l2j_fill_synthetic(l2j_ctx *c, uint64_t seed, float sigma)
 {
-    if (!c) return fail(L2J_E_ARG, "null context");
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const float scale = sigma / 37837.2265625f;
-    auto base_of = [&](uint32_t stream) { return seed * 0x9E3779B97F4A7C15ULL + (uint64_t)stream * 0xD1B54A32D192ED03ULL; };
-    const uint64_t vd = (uint64_t)c->cfg.vocab_size * c->cfg.dim;
-    hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->emb, (long)vd, base_of(0), scale);
-    HIPCHK(hipGetLastError());
-    if (c->wcls != c->emb) {
-        hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->wcls, (long)vd, base_of(11), scale);
+    return ctx_rc(c, [&]() -> int {
+        if (!c) return fail(L2J_E_ARG, "null context");
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const float scale = sigma / 37837.2265625f;
+        auto base_of = [&](uint32_t stream) { return seed * 0x9E3779B97F4A7C15ULL + (uint64_t)stream * 0xD1B54A32D192ED03ULL; };
+        const uint64_t vd = (uint64_t)c->cfg.vocab_size * c->cfg.dim;
+        hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->emb, (long)vd, base_of(0), scale);
         HIPCHK(hipGetLastError());
-    }
-    for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++) {
-        QTensor &q = c->qt[t];
-        hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(q.ngroups, 1u << 20)), dim3(256), 0, c->stream,
-                           (const float *)nullptr, 0L, 0L, (long)q.ngroups, (long)q.nfloats, base_of((uint32_t)t), scale, q.codes, q.gs,
-                           q.mm);
-        HIPCHK(hipGetLastError());
-        q.groups_loaded = q.ngroups;
-    }
-    HIPCHK(hipStreamSynchronize(c->stream));
-    c->emb_loaded = c->wcls_loaded = true;
-    return L2J_OK;
+        if (c->wcls != c->emb) {
+            hipLaunchKernelGGL(k_synth_f32, dim3(4096), dim3(256), 0, c->stream, c->wcls, (long)vd, base_of(11), scale);
+            HIPCHK(hipGetLastError());
+        }
+        for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++) {
+            QTensor &q = c->qt[t];
+            hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(q.ngroups, 1u << 20)), dim3(256), 0, c->stream,
+                               (const float *)nullptr, 0L, 0L, (long)q.ngroups, (long)q.nfloats, base_of((uint32_t)t), scale, q.codes, q.gs,
+                               q.mm);
+            HIPCHK(hipGetLastError());
+            q.groups_loaded = q.ngroups;
+        }
+        HIPCHK(hipStreamSynchronize(c->stream));
+        c->emb_loaded = c->wcls_loaded = true;
+        return L2J_OK;
+    }());
 }
 
 int l2j_finalize(l2j_ctx *c)
 {
-    if (!c) return fail(L2J_E_ARG, "null context");
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    if (c->finalized) return fail(L2J_E_STATE, "already finalized");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    if (!c->emb_loaded) return fail(L2J_E_STATE, "token_embedding_table was not uploaded");
-    if (!c->cfg.shared_weights && !c->wcls_loaded) return fail(L2J_E_STATE, "wcls was not uploaded");
-    for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++)
-        if (c->qt[t].groups_loaded < c->qt[t].ngroups)
-            return fail(L2J_E_STATE, std::string("tensor not fully uploaded: ") + l2j_host::tensor_stem(t));
+    const int rc = ctx_rc(c, [&]() -> int {
+        if (!c) return fail(L2J_E_ARG, "null context");
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (c->finalized) return fail(L2J_E_STATE, "already finalized");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        if (!c->emb_loaded) return fail(L2J_E_STATE, "token_embedding_table was not uploaded");
+        if (!c->cfg.shared_weights && !c->wcls_loaded) return fail(L2J_E_STATE, "wcls was not uploaded");
+        for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++)
+            if (c->qt[t].groups_loaded < c->qt[t].ngroups)
+                return fail(L2J_E_STATE, std::string("tensor not fully uploaded: ") + l2j_host::tensor_stem(t));
 
-    // RoPE table (K/ApplyRope.java:34-59): freq = (float)(1.0 / pow(10000.0f, (i % hs) / (float) hs)),
-    // val = pos * freq in fp32, cos/sin in double then narrowed.  Only i % head_size matters.
-    const int hs = c->head_size, half = hs / 2, S = c->cfg.seq_len;
-    std::vector<float2> rope((size_t)S * half);
-    for (int k = 0; k < half; k++) {
-        const float ex = (float)(2 * k) / (float)hs;
-        const float freq = (float)(1.0 / std::pow((double)10000.0f, (double)ex));
-        for (int pos = 0; pos < S; pos++) {
-            const float val = (float)pos * freq;
-            rope[(size_t)pos * half + k] = make_float2((float)std::cos((double)val), (float)std::sin((double)val));
+        // RoPE table (K/ApplyRope.java:34-59): freq = (float)(1.0 / pow(10000.0f, (i % hs) / (float) hs)),
+        // val = pos * freq in fp32, cos/sin in double then narrowed.  Only i % head_size matters.
+        const int hs = c->head_size, half = hs / 2, S = c->cfg.seq_len;
+        std::vector<float2> rope((size_t)S * half);
+        for (int k = 0; k < half; k++) {
+            const float ex = (float)(2 * k) / (float)hs;
+            const float freq = (float)(1.0 / std::pow((double)10000.0f, (double)ex));
+            for (int pos = 0; pos < S; pos++) {
+                const float val = (float)pos * freq;
+                rope[(size_t)pos * half + k] = make_float2((float)std::cos((double)val), (float)std::sin((double)val));
+            }
         }
-    }
-    HIPCHK(hipMemcpy(c->rope, rope.data(), rope.size() * sizeof(float2), hipMemcpyHostToDevice));
-    // sigmoid table (K/Silu.java:47-57)
-    std::vector<float> tab(kSiluTable);
-    for (int i = 0; i < kSiluTable; i++) {
-        const double v = ((double)i / (double)kSiluTable) * 10.0 - 5.0;
-        tab[i] = (float)(1.0 / (1.0 + std::exp(-v)));
-    }
-    HIPCHK(hipMemcpy(c->silu, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice));
+        HIPCHK(hipMemcpy(c->rope, rope.data(), rope.size() * sizeof(float2), hipMemcpyHostToDevice));
+        // sigmoid table (K/Silu.java:47-57)
+        std::vector<float> tab(kSiluTable);
+        for (int i = 0; i < kSiluTable; i++) {
+            const double v = ((double)i / (double)kSiluTable) * 10.0 - 5.0;
+            tab[i] = (float)(1.0 / (1.0 + std::exp(-v)));
+        }
+        HIPCHK(hipMemcpy(c->silu, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice));
 
-    // rmsnorm weights dequantized once with the reference's expression
-    {
-        const uint64_t dim = c->cfg.dim, L = c->cfg.n_layers;
-        int rc2;
-        if ((rc2 = dev_alloc(&c->rmsw, (2 * L + 1) * dim))) return rc2;
-        const int src[3] = {L2J_RMS_ATT, L2J_RMS_FFN, L2J_RMS_FINAL};
-        float *dst[3] = {c->rmsw, c->rmsw + L * dim, c->rmsw + 2 * L * dim};
-        for (int i = 0; i < 3; i++) {
-            const long n = (long)c->qt[src[i]].nfloats;
-            hipLaunchKernelGGL(k_dequant_rms, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, c->stream, c->qt[src[i]].codes,
-                               c->qt[src[i]].mm, n, dst[i]);
-            HIPCHK(hipGetLastError());
+        // rmsnorm weights dequantized once with the reference's expression
+        {
+            const uint64_t dim = c->cfg.dim, L = c->cfg.n_layers;
+            int rc2;
+            if ((rc2 = dev_alloc(&c->rmsw, (2 * L + 1) * dim))) return rc2;
+            const int src[3] = {L2J_RMS_ATT, L2J_RMS_FFN, L2J_RMS_FINAL};
+            float *dst[3] = {c->rmsw, c->rmsw + L * dim, c->rmsw + 2 * L * dim};
+            for (int i = 0; i < 3; i++) {
+                const long n = (long)c->qt[src[i]].nfloats;
+                hipLaunchKernelGGL(k_dequant_rms, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, c->stream, c->qt[src[i]].codes,
+                                   c->qt[src[i]].mm, n, dst[i]);
+                HIPCHK(hipGetLastError());
+            }
         }
-    }
-    // launch shapes: one 1024-thread workgroup per compute unit for the weight-streaming kernels
-    {
-        const int nmax = std::max(c->cfg.dim, c->cfg.hidden_dim);
-        c->pk_threads = std::min(1024, std::max(64, env_int("L2J_THREADS", 1024) / 64 * 64));
-        c->pk_grid = std::max(1, env_int("L2J_GRID", c->n_cu));  // one workgroup per compute unit
-        c->attn_threads = std::min(1024, std::max(64, env_int("L2J_ATTN_THREADS", 256) / 64 * 64));
-        c->attn_rows = std::max(1, env_int("L2J_ATTN_ROWS", 32));
-        c->attn_nsplit = std::max(1, env_int("L2J_ATTN_NSPLIT", 32));
-        c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
-        c->fused_attn_rows = std::max(1, env_int("L2J_FUSED_ATTN_ROWS", 64));
-        c->barrier_spins = std::max(0, env_int("L2J_BARRIER_SPINS", 20000));
-        const size_t need = std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c));
-        if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
-        if (need > 64 * 1024) {
-            const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
-                                reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
-                                reinterpret_cast<const void *>(k_matvec<PH_ROW6>),
-                                reinterpret_cast<const void *>(k_matvec<PH_QKV, 5>), reinterpret_cast<const void *>(k_matvec<PH_W13, 5>),
-                                reinterpret_cast<const void *>(k_matvec<PH_RES, 5>),
-                                reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
-                                reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>),
-                                reinterpret_cast<const void *>(k_token<16, 1, 1>), reinterpret_cast<const void *>(k_token<16, 1, 2>),
-                                reinterpret_cast<const void *>(k_token<32, 5, kTU>)};
-            for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
+        // launch shapes: one 1024-thread workgroup per compute unit for the weight-streaming kernels
+        {
+            const int nmax = std::max(c->cfg.dim, c->cfg.hidden_dim);
+            const int *o = c->opt;
+            c->pk_threads = std::min(1024, std::max(64, o[OPT_THREADS] / 64 * 64));
+            c->pk_grid = std::max(1, o[OPT_GRID] != kAuto ? o[OPT_GRID] : c->n_cu);  // one workgroup per compute unit
+            c->attn_threads = std::min(1024, std::max(64, o[OPT_ATTN_THREADS] / 64 * 64));
+            c->attn_rows = std::max(1, o[OPT_ATTN_ROWS]);
+            c->attn_nsplit = std::max(1, o[OPT_ATTN_NSPLIT]);
+            c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
+            c->fused_attn_rows = std::max(1, o[OPT_FUSED_ATTN_ROWS]);
+            const size_t need = std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c));
+            if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
+            if (need > 64 * 1024) {
+                const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
+                                    reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
+                                    reinterpret_cast<const void *>(k_matvec<PH_ROW6>),
+                                    reinterpret_cast<const void *>(k_matvec<PH_QKV, 5>), reinterpret_cast<const void *>(k_matvec<PH_W13, 5>),
+                                    reinterpret_cast<const void *>(k_matvec<PH_RES, 5>),
+                                    reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
+                                    reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>),
+                                    reinterpret_cast<const void *>(k_token<16, 1, 1>), reinterpret_cast<const void *>(k_token<16, 1, 2>),
+                                    reinterpret_cast<const void *>(k_token<32, 5, kTU>)};
+                for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
+            }
+            int rc2;
+            if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
+            if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
+            if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_layers * c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
+            c->nbar = 5 * c->cfg.n_layers;
+            if ((rc2 = dev_alloc(&c->bar_ctr, (uint64_t)c->nbar * kBarStride))) return rc2;
+            if ((rc2 = dev_alloc(&c->fault, 1))) return rc2;
+            HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));
+            HIPCHK(hipMemset(c->fault, 0, sizeof(int)));
+            HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&c->h_fault), sizeof(int), hipHostMallocDefault));
+            *c->h_fault = 0;
+            // k_token needs its whole grid resident at once (grid barriers): at most what the occupancy allows.
+            // One launch per token pays off when a layer streams enough to hide its five hand-overs (7B shape, 208 MB a
+            // layer: 645 vs 511 tok/s; 110M shape, 7 MB: 3240 vs 3080); the smallest models run faster as one launch per
+            // phase (15M shape, 1 MB a layer: 6300 vs 5400 tok/s).
+            const uint64_t layer_floats = 2ull * c->cfg.dim * c->cfg.dim + 2ull * c->cfg.dim * c->kv_dim + 3ull * c->cfg.dim * c->cfg.hidden_dim;
+            c->fused = (c->opt[OPT_FUSE] != kAuto ? c->opt[OPT_FUSE] : layer_floats >= (4ull << 20) ? 1 : 0) != 0;
+            c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, c->opt[OPT_LAYERS_PER_LAUNCH] != kAuto ? c->opt[OPT_LAYERS_PER_LAUNCH] : c->cfg.n_layers));
+            if (c->fused) {
+                const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
+                int per_cu = 0;
+                HIPCHK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kl, c->pk_threads, layer_smem(c)));
+                if (per_cu < 1 || c->pk_grid > per_cu * c->n_cu) c->fused = false;
+            }
+            c->by_value = c->fused && c->layers_per_launch == c->cfg.n_layers && c->opt[OPT_BY_VALUE] != 0 &&
+                          std::max(c->cfg.dim, c->cfg.hidden_dim) <= 4 * kPollWords * c->pk_threads;
+            build_geom(c);
+            if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
         }
-        int rc2;
-        if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
-        if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
-        if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_layers * c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
-        c->nbar = 5 * c->cfg.n_layers;
-        if ((rc2 = dev_alloc(&c->bar_ctr, (uint64_t)c->nbar * kBarStride))) return rc2;
-        if ((rc2 = dev_alloc(&c->fault, 1))) return rc2;
-        HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));
-        HIPCHK(hipMemset(c->fault, 0, sizeof(int)));
-        HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&c->h_fault), sizeof(int), hipHostMallocDefault));
-        *c->h_fault = 0;
-        // k_token needs its whole grid resident at once (grid barriers): at most what the occupancy allows.
-        // One launch per token pays off when a layer streams enough to hide its five hand-overs (7B shape, 208 MB a
-        // layer: 645 vs 511 tok/s; 110M shape, 7 MB: 3240 vs 3080); the smallest models run faster as one launch per
-        // phase (15M shape, 1 MB a layer: 6300 vs 5400 tok/s).
-        const uint64_t layer_floats = 2ull * c->cfg.dim * c->cfg.dim + 2ull * c->cfg.dim * c->kv_dim + 3ull * c->cfg.dim * c->cfg.hidden_dim;
-        c->fused = env_int("L2J_FUSE", layer_floats >= (4ull << 20) ? 1 : 0) != 0;
-        c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, env_int("L2J_LAYERS_PER_LAUNCH", c->cfg.n_layers)));
-        if (c->fused) {
-            const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
-            int per_cu = 0;
-            HIPCHK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kl, c->pk_threads, layer_smem(c)));
-            if (per_cu < 1 || c->pk_grid > per_cu * c->n_cu) c->fused = false;
-        }
-        c->by_value = c->fused && c->layers_per_launch == c->cfg.n_layers && env_int("L2J_BY_VALUE", 1) != 0 &&
-                      std::max(c->cfg.dim, c->cfg.hidden_dim) <= 4 * kPollWords * c->pk_threads;
-        build_geom(c);
-        if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
-    }
 
-    // capture one token
-    HIPCHK(hipStreamSynchronize(c->stream));
-    const char *mode = getenv("L2J_MODE");
-    if (mode && strcmp(mode, "eager") == 0) {
+        // capture one token
+        HIPCHK(hipStreamSynchronize(c->stream));
+        if (c->opt[OPT_GRAPH] == 0) {
+            c->finalized = true;
+            return L2J_OK;
+        }
+        HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+        hipError_t le = launch_token(c, c->stream, false);
+        hipError_t ce = hipStreamEndCapture(c->stream, &c->graph);
+        if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
+        HIPCHK(ce);
+        HIPCHK(hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0));
         c->finalized = true;
         return L2J_OK;
+    }());
+    if (rc && c) {  // a finalize that failed part-way leaves nothing behind: it may be called again
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (!c->finalized) {
+            (void)hipSetDevice(c->cfg.device);
+            release_finalize(c);
+        }
     }
-    HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
-    hipError_t le = launch_token(c, c->stream, false);
-    hipError_t ce = hipStreamEndCapture(c->stream, &c->graph);
-    if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
-    HIPCHK(ce);
-    HIPCHK(hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0));
-    c->finalized = true;
-    return L2J_OK;
+    return rc;
 }
 
 int l2j_reset(l2j_ctx *c)
 {
-    if (!c) return fail(L2J_E_ARG, "null context");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const uint64_t kvn = (uint64_t)c->cfg.n_layers * c->cfg.seq_len * c->kv_dim;
-    HIPCHK(hipMemsetAsync(c->kcache, 0, kvn * sizeof(float), c->stream));
-    HIPCHK(hipMemsetAsync(c->vcache, 0, kvn * sizeof(float), c->stream));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c) return fail(L2J_E_ARG, "null context");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const uint64_t kvn = (uint64_t)c->cfg.n_layers * c->cfg.seq_len * c->kv_dim;
+        HIPCHK(hipMemsetAsync(c->kcache, 0, kvn * sizeof(float), c->stream));
+        HIPCHK(hipMemsetAsync(c->vcache, 0, kvn * sizeof(float), c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        return L2J_OK;
+    }());
 }
 
 int l2j_sync(l2j_ctx *c)
 {
-    if (!c) return fail(L2J_E_ARG, "null context");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c) return fail(L2J_E_ARG, "null context");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        return L2J_OK;
+    }());
 }
 
 int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    int rc = check_forward_args(c, token, pos);
-    if (rc) return rc;
-    if ((rc = set_state(c, token, pos, 0))) return rc;
-    HIPCHK(launch_one_token(c));
-    if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    return check_barrier_error(c);
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        int rc = check_forward_args(c, token, pos);
+        if (rc) return rc;
+        if ((rc = set_state(c, token, pos, 0))) return rc;
+        HIPCHK(launch_one_token(c));
+        if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        return check_barrier_error(c);
+    }());
 }
 
 int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!next) return fail(L2J_E_ARG, "null argument");
-    int rc = check_forward_args(c, token, pos);
-    if (rc) return rc;
-    if ((rc = set_state(c, token, pos, 0))) return rc;
-    HIPCHK(launch_one_token(c));
-    HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    *next = c->h_tokens[0];
-    return check_barrier_error(c);
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!next) return fail(L2J_E_ARG, "null argument");
+        int rc = check_forward_args(c, token, pos);
+        if (rc) return rc;
+        if ((rc = set_state(c, token, pos, 0))) return rc;
+        HIPCHK(launch_one_token(c));
+        HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        *next = c->h_tokens[0];
+        return check_barrier_error(c);
+    }());
 }
 
 int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    int rc = check_forward_args(c, token, pos);
-    if (rc) return rc;
-    const uint64_t L = c->cfg.n_layers;
-    const int which[] = {L2J_B_X, L2J_B_XB, L2J_B_XB2, L2J_B_HB, L2J_B_Q, L2J_B_K, L2J_B_V};
-    for (int w : which) {
-        if (c->taps[w]) continue;
-        const uint64_t n = w == L2J_B_HB ? c->cfg.hidden_dim : (w == L2J_B_K || w == L2J_B_V) ? c->kv_dim : c->cfg.dim;
-        if ((rc = dev_alloc(&c->taps[w], L * n))) return rc;
-    }
-    if ((rc = set_state(c, token, pos, 0))) return rc;
-    hipError_t e = launch_token(c, c->stream, true);
-    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
-    if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        int rc = check_forward_args(c, token, pos);
+        if (rc) return rc;
+        const uint64_t L = c->cfg.n_layers;
+        const int which[] = {L2J_B_X, L2J_B_XB, L2J_B_XB2, L2J_B_HB, L2J_B_Q, L2J_B_K, L2J_B_V};
+        for (int w : which) {
+            if (c->taps[w]) continue;
+            const uint64_t n = w == L2J_B_HB ? c->cfg.hidden_dim : (w == L2J_B_K || w == L2J_B_V) ? c->kv_dim : c->cfg.dim;
+            if ((rc = dev_alloc(&c->taps[w], L * n))) return rc;
+        }
+        if ((rc = set_state(c, token, pos, 0))) return rc;
+        hipError_t e = launch_token(c, c->stream, true);
+        if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
+        if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        return L2J_OK;
+    }());
 }
 
 int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, int32_t *out_tokens, int32_t *n_out,
                       double *seconds)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    return decode_loop(c, prompt, n_prompt, steps, false, 0.0f, 0.0f, 0, out_tokens, n_out, seconds);
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        return decode_loop(c, prompt, n_prompt, steps, false, 0.0f, 0.0f, 0, out_tokens, n_out, seconds);
+    }());
 }
 
 int l2j_decode_sample(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature, float topp,
                       int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    int rc = check_sampler_args(temperature, topp);
-    if (rc) return rc;
-    return decode_loop(c, prompt, n_prompt, steps, temperature != 0.0f, temperature, topp, rng_seed, out_tokens, n_out, seconds);
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        int rc = check_sampler_args(temperature, topp);
+        if (rc) return rc;
+        return decode_loop(c, prompt, n_prompt, steps, temperature != 0.0f, temperature, topp, rng_seed, out_tokens, n_out, seconds);
+    }());
 }
 
 int l2j_sampler_seed(l2j_ctx *c, int64_t rng_seed)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!c) return fail(L2J_E_ARG, "null context");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    return seed_sampler(c, rng_seed);
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c) return fail(L2J_E_ARG, "null context");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        return seed_sampler(c, rng_seed);
+    }());
 }
 
 int l2j_sample(l2j_ctx *c, const float *logits, float temperature, float topp, float coin, int32_t *next)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!c || !next) return fail(L2J_E_ARG, "null argument");
-    int rc = check_sampler_args(temperature, topp);
-    if (rc) return rc;
-    if (coin >= 1.0f) return fail(L2J_E_ARG, "coin must be below 1 (negative: the context's generator draws)");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    if (!c->ss && (rc = seed_sampler(c, 0))) return rc;
-    const int n = c->cfg.vocab_size;
-    if (logits) HIPCHK(hipMemcpyAsync(c->logits, logits, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream));
-    if (temperature == 0.0f) {
-        hipLaunchKernelGGL(k_argmax_logits, dim3(1), dim3(1024), 0, c->stream, c->logits, n, c->ss);  // J/Run.java:644-646
-        HIPCHK(hipGetLastError());
-    } else {
-        HIPCHK(launch_sampler(c, temperature, topp, coin, false));
-    }
-    HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
-    HIPCHK(hipStreamSynchronize(c->stream));
-    if ((rc = check_sampler_status(c))) return rc;
-    *next = c->h_ss->result;
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !next) return fail(L2J_E_ARG, "null argument");
+        int rc = check_sampler_args(temperature, topp);
+        if (rc) return rc;
+        if (coin >= 1.0f) return fail(L2J_E_ARG, "coin must be below 1 (negative: the context's generator draws)");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        if (!c->ss && (rc = seed_sampler(c, 0))) return rc;
+        const int n = c->cfg.vocab_size;
+        if (logits) HIPCHK(hipMemcpyAsync(c->logits, logits, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        if (temperature == 0.0f) {
+            hipLaunchKernelGGL(k_argmax_logits, dim3(1), dim3(1024), 0, c->stream, c->logits, n, c->ss);  // J/Run.java:644-646
+            HIPCHK(hipGetLastError());
+        } else {
+            HIPCHK(launch_sampler(c, temperature, topp, coin, false));
+        }
+        HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        if ((rc = check_sampler_status(c))) return rc;
+        *next = c->h_ss->result;
+        return L2J_OK;
+    }());
 }
 
 int l2j_running_sums(l2j_ctx *c, const float *terms, int32_t n, float *sums)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!c || !terms || !sums) return fail(L2J_E_ARG, "null argument");
-    if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "1 to 36864 terms");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    float *d = nullptr;
-    HIPCHK(hipMalloc(reinterpret_cast<void **>(&d), (size_t)n * sizeof(float)));
-    const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
-    hipError_t e = hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e == hipSuccess) e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
-    if (e == hipSuccess) {
-        hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, env_int("L2J_SAMPLER_SCAN", 1) != 0 ? 1 : 0);
-        e = hipGetLastError();
-    }
-    if (e == hipSuccess) e = hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
-    (void)hipFree(d);
-    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("running sums: ") + hipGetErrorString(e));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !terms || !sums) return fail(L2J_E_ARG, "null argument");
+        if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "1 to 36864 terms");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        float *d = nullptr;
+        HIPCHK(hipMalloc(reinterpret_cast<void **>(&d), (size_t)n * sizeof(float)));
+        const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
+        hipError_t e = hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        (void)hipFree(d);
+        if (e != hipSuccess) return fail(L2J_E_HIP, std::string("running sums: ") + hipGetErrorString(e));
+        return L2J_OK;
+    }());
 }
 
 int l2j_read(l2j_ctx *c, int which, int layer, uint64_t off, float *dst, uint64_t n)
 {
-    if (!c || !dst) return fail(L2J_E_ARG, "null argument");
-    if (which < 0 || which >= L2J_B_COUNT) return fail(L2J_E_ARG, "unknown buffer");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const l2j_config &g = c->cfg;
-    const float *src = nullptr;
-    uint64_t len = 0;
-    if (which == L2J_B_KCACHE || which == L2J_B_VCACHE) {
-        if (layer < 0 || layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
-        len = (uint64_t)g.seq_len * c->kv_dim;
-        src = (which == L2J_B_KCACHE ? c->kcache : c->vcache) + (uint64_t)layer * len;
-    } else if (which == L2J_B_LOGITS) {
-        src = c->logits; len = g.vocab_size;
-    } else if (layer < 0) {
-        switch (which) {
-        case L2J_B_X: src = c->x + 2ull * g.n_layers * c->sd; len = g.dim; break;  // the last layer's vectors
-        case L2J_B_XB: src = c->xb + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
-        case L2J_B_HB: src = c->hb + (uint64_t)(g.n_layers - 1) * c->sh; len = g.hidden_dim; break;
-        case L2J_B_Q: src = c->q + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
-        default: return fail(L2J_E_ARG, "this buffer only exists as a per-layer tap");
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !dst) return fail(L2J_E_ARG, "null argument");
+        if (which < 0 || which >= L2J_B_COUNT) return fail(L2J_E_ARG, "unknown buffer");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const l2j_config &g = c->cfg;
+        const float *src = nullptr;
+        uint64_t len = 0;
+        if (which == L2J_B_KCACHE || which == L2J_B_VCACHE) {
+            if (layer < 0 || layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
+            len = (uint64_t)g.seq_len * c->kv_dim;
+            src = (which == L2J_B_KCACHE ? c->kcache : c->vcache) + (uint64_t)layer * len;
+        } else if (which == L2J_B_LOGITS) {
+            src = c->logits; len = g.vocab_size;
+        } else if (layer < 0) {
+            switch (which) {
+            case L2J_B_X: src = c->x + 2ull * g.n_layers * c->sd; len = g.dim; break;  // the last layer's vectors
+            case L2J_B_XB: src = c->xb + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
+            case L2J_B_HB: src = c->hb + (uint64_t)(g.n_layers - 1) * c->sh; len = g.hidden_dim; break;
+            case L2J_B_Q: src = c->q + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
+            default: return fail(L2J_E_ARG, "this buffer only exists as a per-layer tap");
+            }
+        } else {
+            if (layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
+            if (!c->taps[which]) return fail(L2J_E_STATE, "no taps recorded: call l2j_forward_taps first");
+            len = which == L2J_B_HB ? g.hidden_dim : (which == L2J_B_K || which == L2J_B_V) ? c->kv_dim : g.dim;
+            src = c->taps[which] + (uint64_t)layer * len;
         }
-    } else {
-        if (layer >= g.n_layers) return fail(L2J_E_ARG, "layer out of range");
-        if (!c->taps[which]) return fail(L2J_E_STATE, "no taps recorded: call l2j_forward_taps first");
-        len = which == L2J_B_HB ? g.hidden_dim : (which == L2J_B_K || which == L2J_B_V) ? c->kv_dim : g.dim;
-        src = c->taps[which] + (uint64_t)layer * len;
-    }
-    if (off + n > len) return fail(L2J_E_SIZE, "read past the end of the buffer");
-    HIPCHK(hipStreamSynchronize(c->stream));
-    HIPCHK(hipMemcpy(dst, src + off, n * sizeof(float), hipMemcpyDeviceToHost));
-    return L2J_OK;
+        if (off + n > len) return fail(L2J_E_SIZE, "read past the end of the buffer");
+        HIPCHK(hipStreamSynchronize(c->stream));
+        HIPCHK(hipMemcpy(dst, src + off, n * sizeof(float), hipMemcpyDeviceToHost));
+        return L2J_OK;
+    }());
 }
 
 int l2j_write_kv(l2j_ctx *c, int layer, int32_t pos0, int32_t npos, const float *k, const float *v)
 {
-    if (!c || !k || !v) return fail(L2J_E_ARG, "null argument");
-    if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
-    if (pos0 < 0 || npos < 0 || (int64_t)pos0 + npos > c->cfg.seq_len) return fail(L2J_E_ARG, "positions out of range");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    const uint64_t o = ((uint64_t)layer * c->cfg.seq_len + pos0) * c->kv_dim, n = (uint64_t)npos * c->kv_dim;
-    HIPCHK(hipStreamSynchronize(c->stream));
-    HIPCHK(hipMemcpy(c->kcache + o, k, n * sizeof(float), hipMemcpyHostToDevice));
-    HIPCHK(hipMemcpy(c->vcache + o, v, n * sizeof(float), hipMemcpyHostToDevice));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !k || !v) return fail(L2J_E_ARG, "null argument");
+        if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        if (pos0 < 0 || npos < 0 || (int64_t)pos0 + npos > c->cfg.seq_len) return fail(L2J_E_ARG, "positions out of range");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        const uint64_t o = ((uint64_t)layer * c->cfg.seq_len + pos0) * c->kv_dim, n = (uint64_t)npos * c->kv_dim;
+        HIPCHK(hipStreamSynchronize(c->stream));
+        HIPCHK(hipMemcpy(c->kcache + o, k, n * sizeof(float), hipMemcpyHostToDevice));
+        HIPCHK(hipMemcpy(c->vcache + o, v, n * sizeof(float), hipMemcpyHostToDevice));
+        return L2J_OK;
+    }());
 }
 
 int l2j_calibration_copy(l2j_ctx *c, uint64_t nbytes, int32_t rounds)
 {
-    if (!c || nbytes < 16 || rounds <= 0) return fail(L2J_E_ARG, "bad argument");
-    HIPCHK(hipSetDevice(c->cfg.device));
-    uint4 *a = nullptr, *b = nullptr;
-    const long n = (long)(nbytes / 16);
-    HIPCHK(hipMalloc(reinterpret_cast<void **>(&a), (size_t)n * 16));
-    hipError_t e = hipMalloc(reinterpret_cast<void **>(&b), (size_t)n * 16);
-    if (e == hipSuccess) e = hipMemsetAsync(a, 1, (size_t)n * 16, c->stream);
-    for (int r = 0; r < rounds && e == hipSuccess; r++) {
-        hipLaunchKernelGGL(k_copy16, dim3(c->n_cu * 8), dim3(256), 0, c->stream, a, b, n);
-        e = hipGetLastError();
-    }
-    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
-    (void)hipFree(a);
-    (void)hipFree(b);
-    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("calibration copy: ") + hipGetErrorString(e));
-    return L2J_OK;
+    return ctx_rc(c, [&]() -> int {
+        if (!c || nbytes < 16 || rounds <= 0) return fail(L2J_E_ARG, "bad argument");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        uint4 *a = nullptr, *b = nullptr;
+        const long n = (long)(nbytes / 16);
+        HIPCHK(hipMalloc(reinterpret_cast<void **>(&a), (size_t)n * 16));
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&b), (size_t)n * 16);
+        if (e == hipSuccess) e = hipMemsetAsync(a, 1, (size_t)n * 16, c->stream);
+        for (int r = 0; r < rounds && e == hipSuccess; r++) {
+            hipLaunchKernelGGL(k_copy16, dim3(c->n_cu * 8), dim3(256), 0, c->stream, a, b, n);
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        (void)hipFree(a);
+        (void)hipFree(b);
+        if (e != hipSuccess) return fail(L2J_E_HIP, std::string("calibration copy: ") + hipGetErrorString(e));
+        return L2J_OK;
+    }());
 }
 
 uint64_t l2j_bytes_per_token(const l2j_config *g, int32_t pos)
@@ -1259,80 +1402,82 @@ uint64_t l2j_bytes_per_token(const l2j_config *g, int32_t pos)
 
 int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double *mean_us, uint64_t *bytes)
 {
-    std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-    if (!c || !mean_us) return fail(L2J_E_ARG, "null argument");
-    if (kclass < 0 || kclass >= L2J_K_COUNT || rounds <= 0) return fail(L2J_E_ARG, "bad kernel class or rounds");
-    int rc = check_forward_args(c, 1, pos);
-    if (rc) return rc;
-    const l2j_config &g = c->cfg;
-    const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim;
-    uint64_t b = 0;
-    switch (kclass) {
-    case L2J_K_QKV: b = quant_bytes_of(dim * dim + 2 * dim * kvd) + quant_bytes_of(dim); break;
-    case L2J_K_ATTENTION: b = 2ull * (pos + 1) * kvd * 4; break;
-    case L2J_K_WO: b = quant_bytes_of(dim * dim); break;
-    case L2J_K_W13: b = quant_bytes_of(2 * dim * hid) + quant_bytes_of(dim); break;
-    case L2J_K_W2: b = quant_bytes_of(dim * hid); break;
-    case L2J_K_CLASSIFIER: b = (uint64_t)g.vocab_size * dim * 4 + quant_bytes_of(dim); break;
-    case L2J_K_TOKEN: b = l2j_bytes_per_token(&g, pos); break;
-    }
-    if (bytes) *bytes = b;
-    if (kclass == L2J_K_TOKEN) {  // the whole-token kernel, then k_finish (untimed) to reset the barrier counters
-        if (!c->fused) return fail(L2J_E_STATE, "the whole-token kernel is switched off or does not fit this shape");
-        if (rounds > 256) return fail(L2J_E_ARG, "at most 256 rounds of the whole-token kernel");
-        while ((int)c->events.size() < 33 + 2 * rounds) {
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !mean_us) return fail(L2J_E_ARG, "null argument");
+        if (kclass < 0 || kclass >= L2J_K_COUNT || rounds <= 0) return fail(L2J_E_ARG, "bad kernel class or rounds");
+        int rc = check_forward_args(c, 1, pos);
+        if (rc) return rc;
+        const l2j_config &g = c->cfg;
+        const uint64_t dim = g.dim, hid = g.hidden_dim, kvd = c->kv_dim;
+        uint64_t b = 0;
+        switch (kclass) {
+        case L2J_K_QKV: b = quant_bytes_of(dim * dim + 2 * dim * kvd) + quant_bytes_of(dim); break;
+        case L2J_K_ATTENTION: b = 2ull * (pos + 1) * kvd * 4; break;
+        case L2J_K_WO: b = quant_bytes_of(dim * dim); break;
+        case L2J_K_W13: b = quant_bytes_of(2 * dim * hid) + quant_bytes_of(dim); break;
+        case L2J_K_W2: b = quant_bytes_of(dim * hid); break;
+        case L2J_K_CLASSIFIER: b = (uint64_t)g.vocab_size * dim * 4 + quant_bytes_of(dim); break;
+        case L2J_K_TOKEN: b = l2j_bytes_per_token(&g, pos); break;
+        }
+        if (bytes) *bytes = b;
+        if (kclass == L2J_K_TOKEN) {  // the whole-token kernel, then k_finish (untimed) to reset the barrier counters
+            if (!c->fused) return fail(L2J_E_STATE, "the whole-token kernel is switched off or does not fit this shape");
+            if (rounds > 256) return fail(L2J_E_ARG, "at most 256 rounds of the whole-token kernel");
+            while ((int)c->events.size() < 33 + 2 * rounds) {
+                hipEvent_t ev;
+                HIPCHK(hipEventCreate(&ev));
+                c->events.push_back(ev);
+            }
+            // the rounds follow each other on the stream without a host round trip in between, as the tokens of a decode do
+            for (int r = 0; r < rounds; r++) {
+                if ((rc = set_state(c, 1, pos, 0))) return rc;
+                if (c->by_value) {
+                    hipError_t ef = launch_fill_unset(c, c->stream);
+                    if (ef != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(ef));
+                }
+                hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33 + 2 * r], c->events[34 + 2 * r]);
+                if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
+                hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));
+                HIPCHK(hipGetLastError());
+            }
+            HIPCHK(hipStreamSynchronize(c->stream));
+            if ((rc = check_barrier_error(c))) return rc;
+            double total = 0.0;
+            for (int r = 0; r < rounds; r++) {
+                float ms = 0.f;
+                HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * r], c->events[34 + 2 * r]));
+                total += ms;
+            }
+            *mean_us = total * 1e3 / rounds;
+            return L2J_OK;
+        }
+        const int per_round = kclass == L2J_K_CLASSIFIER ? 1 : g.n_layers;
+        while ((int)c->events.size() < 2 * per_round + 33) {
             hipEvent_t ev;
             HIPCHK(hipEventCreate(&ev));
             c->events.push_back(ev);
         }
-        // the rounds follow each other on the stream without a host round trip in between, as the tokens of a decode do
+        // The activations hold whatever the last forward left; timing does not depend on their values.
+        double total_ms = 0.0;
+        long count = 0;
         for (int r = 0; r < rounds; r++) {
             if ((rc = set_state(c, 1, pos, 0))) return rc;
-            if (c->by_value) {
-                hipError_t ef = launch_fill_unset(c, c->stream);
-                if (ef != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(ef));
+            for (int l = 0; l < per_round; l++) {
+                hipError_t e = launch_class(c, kclass, l, c->stream, c->events[33 + 2 * l], c->events[34 + 2 * l]);
+                if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
             }
-            hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33 + 2 * r], c->events[34 + 2 * r]);
-            if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
-            hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));
-            HIPCHK(hipGetLastError());
+            HIPCHK(hipStreamSynchronize(c->stream));
+            for (int l = 0; l < per_round; l++) {
+                float ms = 0.f;
+                HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * l], c->events[34 + 2 * l]));
+                total_ms += ms;
+                count++;
+            }
         }
-        HIPCHK(hipStreamSynchronize(c->stream));
-        if ((rc = check_barrier_error(c))) return rc;
-        double total = 0.0;
-        for (int r = 0; r < rounds; r++) {
-            float ms = 0.f;
-            HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * r], c->events[34 + 2 * r]));
-            total += ms;
-        }
-        *mean_us = total * 1e3 / rounds;
+        *mean_us = total_ms * 1e3 / (double)count;
         return L2J_OK;
-    }
-    const int per_round = kclass == L2J_K_CLASSIFIER ? 1 : g.n_layers;
-    while ((int)c->events.size() < 2 * per_round + 33) {
-        hipEvent_t ev;
-        HIPCHK(hipEventCreate(&ev));
-        c->events.push_back(ev);
-    }
-    // The activations hold whatever the last forward left; timing does not depend on their values.
-    double total_ms = 0.0;
-    long count = 0;
-    for (int r = 0; r < rounds; r++) {
-        if ((rc = set_state(c, 1, pos, 0))) return rc;
-        for (int l = 0; l < per_round; l++) {
-            hipError_t e = launch_class(c, kclass, l, c->stream, c->events[33 + 2 * l], c->events[34 + 2 * l]);
-            if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
-        }
-        HIPCHK(hipStreamSynchronize(c->stream));
-        for (int l = 0; l < per_round; l++) {
-            float ms = 0.f;
-            HIPCHK(hipEventElapsedTime(&ms, c->events[33 + 2 * l], c->events[34 + 2 * l]));
-            total_ms += ms;
-            count++;
-        }
-    }
-    *mean_us = total_ms * 1e3 / (double)count;
-    return L2J_OK;
+    }());
 }
 
 }  // extern "C"

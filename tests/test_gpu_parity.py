@@ -448,6 +448,64 @@ def test_upload_by_layer_and_from_threads(orc):
     np.testing.assert_array_equal(g.forward(3, 0), want)
 
 
+def test_error_text_is_kept_per_context_across_threads(orc):
+    """A failing call on thread A, the message fetched on thread B (a Java virtual thread may be mounted on another
+    carrier thread for its second downcall): l2j_ctx_last_error has it, the thread-local l2j_last_error of B does not."""
+    import threading
+    g = l2j.Transformer(l2j.Config(64, 128, 1, 4, 4, 64, 8, 1))
+    other = l2j.Transformer(l2j.Config(64, 128, 1, 4, 4, 64, 8, 1))
+    L = l2j.lib()
+    rcs, seen = [], {}
+
+    def a():
+        bad = np.zeros(264, np.uint8)
+        rcs.append(L.l2j_upload_quant(g._h, TENSOR.WQ, bad.ctypes.data_as(C.POINTER(C.c_uint8)), bad.size))
+
+    def b():
+        seen["ctx"] = g.last_error()
+        seen["other"] = other.last_error()
+        seen["thread"] = L.l2j_last_error().decode()
+    for f in (a, b):
+        t = threading.Thread(target=f)
+        t.start()
+        t.join()
+    assert rcs == [-2]
+    assert "numberOfBytesByFloatSize" in seen["ctx"]
+    assert seen["other"] == "" and "numberOfBytesByFloatSize" not in seen["thread"]
+    # an option that fixes a launch shape is refused once the shapes are fixed; an unknown one always
+    g.fill_synthetic(1, 0.02)
+    g.set_option("threads", 512)
+    g.finalize()
+    with pytest.raises(l2j.L2JError) as e:
+        g.set_option("threads", 1024)
+    assert e.value.code == -3 and "threads" in str(e.value)
+    with pytest.raises(l2j.L2JError) as e:
+        g.set_option("no_such_option", 1)
+    assert e.value.code == -1
+    g.set_option("sampler_scan", 0)  # allowed at any time
+    g.close(); other.close()
+
+
+def test_options_override_the_process_defaults(orc, monkeypatch):
+    """The same model finalized with the launch mode given per context (no environment involved) computes the same
+    logits on the whole-token path, with grid barriers, and with one launch per phase."""
+    shape = (256, 512, 2, 2, 2, 64, 6, 0)
+    for k in ("L2J_FUSE", "L2J_BY_VALUE", "L2J_GRAPH"):
+        monkeypatch.delenv(k, raising=False)
+    m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
+                  vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
+    m.fill_synth(9, 0.02)
+    want = [m.forward(3 + p, p).copy() for p in range(4)]
+    for opts in ({"fuse": 1}, {"fuse": 1, "by_value": 0}, {"fuse": 0}, {"fuse": 1, "graph": 0}, {"fuse": 0, "graph": 0}):
+        g = l2j.Transformer(l2j.Config(*shape), options=opts)
+        g.fill_synthetic(9, 0.02)
+        g.finalize()
+        for p in range(4):
+            assert rel_err(g.forward(3 + p, p), want[p]) < LOGIT_TOL, (opts, p)
+        g.close()
+    m.close()
+
+
 def test_checkpoint_loader_and_quant_caches(orc, tmp_path):
     from tests.test_oracle_forward import write_bin
     cfg = (64, 96, 2, 4, 2, 30, 8)
@@ -562,7 +620,50 @@ def test_config4_long_context_attention(orc):
     np.testing.assert_array_equal(g.read(BUFFER.VCACHE, layer=1, off=5 * kvd, n=kvd), vc[1, 5])
 
 
+def test_config4_long_context_full_size(orc):
+    """The 32-layer 7B shape deep in its context, on the whole-token path the long-context benchmark times.  The
+    oracle cannot prefill 3584 positions in a test's time, so the GPU decodes the whole sequence (3584 forced prompt
+    ids, then greedy to position 4095), its KV cache is copied into the oracle layer by layer, and the oracle then runs
+    single forwards at chosen positions on that cache: logits within the bar and the same argmax as the token the
+    GPU's own decode loop emitted there."""
+    shape = (4096, 11008, 32, 32, 32, 32000, 4096, 0)
+    L, S, kvd = shape[2], shape[6], 4096
+    say("[C4 full] building")
+    t0 = time.time()
+    m, g = make_pair(orc, shape, seed=104, upload="synthetic")
+    prompt = orc.synth_prompt(104, 3584, shape[5])
+    toks, sec = g.decode_greedy(prompt, S)
+    say("[C4 full] weights + %d GPU steps in %.1fs (%.1f tok/s after the first)" % (len(toks), time.time() - t0, (len(toks) - 1) / sec))
+    assert len(toks) == S, "the decode stopped early (token 1): pick another seed"
+    np.testing.assert_array_equal(toks[:3584], prompt)
+    t0 = time.time()
+    kc, vc = m.buffer(orc.B_KCACHE).reshape(L, S, kvd), m.buffer(orc.B_VCACHE).reshape(L, S, kvd)
+    for l in range(L):
+        kc[l] = g.read(BUFFER.KCACHE, layer=l).reshape(S, kvd)
+        vc[l] = g.read(BUFFER.VCACHE, layer=l).reshape(S, kvd)
+    say("[C4 full] cache copied into the oracle in %.1fs" % (time.time() - t0))
+    worst = 0.0
+    for pos in (3584, 3585, 3840, 4094, 4095):
+        tok = int(toks[pos - 1])
+        want = m.forward(tok, pos).copy()       # reads rows < pos of the GPU's cache, writes its own row pos
+        got = g.forward(tok, pos)               # the whole-token launch replayed at that position
+        e = rel_err(got, want)
+        worst = max(worst, e)
+        top2 = np.partition(want, -2)[-2:]
+        say("[C4 full] pos %d: max|dlogit|/max|logit| = %.3g, relative top-2 gap %.3g" %
+            (pos, e, float(top2[1] - top2[0]) / float(np.abs(want).max())))
+        assert e < LOGIT_TOL, pos
+        assert int(np.argmax(want)) == int(np.argmax(got)) == int(toks[pos]), pos
+        # the row the oracle wrote at pos equals the one the GPU's decode left there
+        for l in (0, L - 1):
+            a = g.read(BUFFER.KCACHE, layer=l, off=pos * kvd, n=kvd)
+            assert np.abs(a - kc[l, pos]).max() <= 2e-5 * max(1.0, float(np.abs(kc[l, pos]).max())), (pos, l)
+    say("[C4 full] worst relative logit error %.3g" % worst)
+    m.close(); g.close()
+
+
 def test_config5_llama2_13b_shape(orc):
-    # the reference's int offsets overflow at this size (J/TransformerWeights.java:89); 64-bit here
-    run_config(orc, "13B", (5120, 13824, 40, 40, 40, 32000, 4096, 0), seed=105, n_prompt=4, n_steps=4 + 8,
-               n_logit_steps=12)
+    # the reference's int offsets overflow at this size (J/TransformerWeights.java:89); 64-bit here.
+    # 32 prompt ids + the first 64 greedy tokens, logits at all 96 steps (the oracle runs at ~3.7 tok/s on 16 cores)
+    run_config(orc, "13B", (5120, 13824, 40, 40, 40, 32000, 4096, 0), seed=105, n_prompt=32, n_steps=32 + 64,
+               n_logit_steps=32 + 64)
