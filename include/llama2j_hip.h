@@ -205,6 +205,13 @@ int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
  * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
  * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
 int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
+/* l2j_running_sums for callers that cannot allocate device memory (code under hipGraph capture, serving loops,
+ * harnesses that forbid it); it has no counterpart in the reference.  Same results, but the terms and sums pass
+ * through a fixed 144 KB device array of the library (one per GPU, held until the process ends) instead of a buffer
+ * allocated per call: n <= 36864, else L2J_E_SIZE.  No hipMalloc / hipFree is made.  Every call on a GPU shares that
+ * GPU's array, so calls that overlapped would race: the library runs them one after the other.  The array keeps the last
+ * call's contents; a call reads none of them (it only reads the n terms it has just copied in). */
+int l2j_running_sums_noalloc(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
 /* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
  * and returns the mean kernel time from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
  * every layer and the classifier in one launch.  The other classes launch one phase of it as a kernel of its

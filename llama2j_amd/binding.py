@@ -105,6 +105,7 @@ def _signatures():
         "l2j_sampler_seed": (C.c_int, [vp, C.c_int64]),
         "l2j_sample": (C.c_int, [vp, fp, C.c_float, C.c_float, C.c_float, i32p]),
         "l2j_running_sums": (C.c_int, [vp, fp, C.c_int32, fp]),
+        "l2j_running_sums_noalloc": (C.c_int, [vp, fp, C.c_int32, fp]),
         "l2j_decode_sample": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, C.c_float, C.c_float, C.c_int64, i32p, i32p,
                                         C.POINTER(C.c_double)]),
         "l2j_read": (C.c_int, [vp, C.c_int, C.c_int, C.c_uint64, fp, C.c_uint64]),
@@ -402,6 +403,14 @@ class Transformer:
             lp = _fp(logits)
         self._check(lib().l2j_sample(self._h, lp, temperature, topp, -1.0 if coin is None else coin, C.byref(nxt)))
         return nxt.value
+
+    def running_sums_noalloc(self, terms):
+        """running_sums through the entry point that allocates nothing (the terms pass through a fixed device buffer
+        of the library: at most 36864)."""
+        terms = np.ascontiguousarray(terms, dtype=np.float32)
+        out = np.empty_like(terms)
+        self._check(lib().l2j_running_sums_noalloc(self._h, _fp(terms), terms.size, _fp(out)))
+        return out
 
     def running_sums(self, terms):
         """The float32 sums terms[0] + ... + terms[i] formed one addition after the other (the order of the reference's

@@ -27,6 +27,10 @@ hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, float *k0, float
                                 int *in_second);
 }  // namespace l2j
 
+// Device memory of l2j_running_sums_noalloc: the terms and their sums of one call.  Every GPU the library runs on holds
+// its own copy of the array until the process ends; in host code the name is only a handle for hipGetSymbolAddress.
+static __device__ __align__(256) float scratch[kSampleMaxVocab];
+
 namespace {
 
 thread_local std::string g_err;
@@ -52,6 +56,26 @@ struct QTensor {
     uint64_t nfloats = 0, ngroups = 0;
     uint64_t groups_loaded = 0;
 };
+
+// The address of `scratch` on each device, looked up by the first l2j_create on that device (with the device current).
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float *g_scratch_ptr[kMaxDevices] = {};
+
+int resolve_scratch(int device)
+{
+    if (device < 0 || device >= kMaxDevices) return fail(L2J_E_ARG, "device ordinal above 63");
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[device]) return L2J_OK;
+    float *p = nullptr;
+    HIPCHK(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    if (!p) return fail(L2J_E_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    // (the largest input needs more than the default 64 KB of dynamic LDS)
+    const int lds = (((kSampleMaxVocab + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
+    HIPCHK(hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    g_scratch_ptr[device] = p;
+    return L2J_OK;
+}
 
 // Launch-shape and algorithm switches of a context.  kAuto = the library picks (by shape, at l2j_finalize).  A context
 // starts from the process defaults (environment variable L2J_<NAME IN CAPITALS>, read once by l2j_create) and
@@ -737,6 +761,7 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
         return fail(L2J_E_HIP, "l2j_create: no HIP device (this library has no CPU fallback)");
     if (cfg->device < 0 || cfg->device >= ndev) return fail(L2J_E_ARG, "l2j_create: device ordinal out of range");
     HIPCHK(hipSetDevice(cfg->device));
+    if ((rc = resolve_scratch(cfg->device))) return rc;
     l2j_ctx *c = new (std::nothrow) l2j_ctx();
     if (!c) return fail(L2J_E_OOM, "l2j_create: host allocation failed");
     c->cfg = *cfg;
@@ -1311,6 +1336,30 @@ int l2j_running_sums(l2j_ctx *c, const float *terms, int32_t n, float *sums)
         if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
         (void)hipFree(d);
         if (e != hipSuccess) return fail(L2J_E_HIP, std::string("running sums: ") + hipGetErrorString(e));
+        return L2J_OK;
+    }());
+}
+
+int l2j_running_sums_noalloc(l2j_ctx *c, const float *terms, int32_t n, float *sums)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !terms || !sums) return fail(L2J_E_ARG, "null argument");
+        if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "l2j_running_sums_noalloc: 1 to 36864 terms (the size of the library's static device buffer)");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        float *d = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(g_scratch_mu);
+            d = g_scratch_ptr[c->cfg.device];
+        }
+        if (!d) return fail(L2J_E_STATE, "l2j_running_sums_noalloc: the static device buffer was not resolved on this device");
+        // The buffer keeps the last call's contents; the kernel reads only the n terms copied in here, so nothing needs clearing.
+        const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
+        HIPCHK(hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream));
+        hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0);
+        HIPCHK(hipGetLastError());
+        HIPCHK(hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+        HIPCHK(hipStreamSynchronize(c->stream));
         return L2J_OK;
     }());
 }
