@@ -29,7 +29,8 @@ struct DevState {
     int token;     // token fed to the next forward
     int pos;       // its position
     int n_prompt;  // positions below this take prompt[pos] as output instead of the argmax
-    int pad;
+    int epoch;     // tokens since the host last set the state: a whole-token kernel that hands its vectors over by value
+                   // alternates between two sets of activation vectors by its parity
 };
 
 // ------------------------------------------------------------------------------------------

@@ -83,7 +83,7 @@ int resolve_scratch(int device)
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -107,6 +107,8 @@ const OptionDef kOptions[OPT_COUNT] = {
     {"sampler_scan", 1, true},         // running sums by the parallel scan (0: one lane, element after element)
     {"sampler_exp_wgs", 32, true},     // workgroups of k_sample_exp (0: the exponentials in k_sample_probs)
     {"graph", 1, false},               // 1: replay a captured hipGraph per token, 0: launch the kernels one by one
+    {"self_contained", 3, false},      // k_token (by value): bit 0 alternates two sets of vectors (no k_fill_unset), bit 1 steps the token loop itself (no k_finish)
+    {"graph_tokens", 32, false},       // tokens per replay of the decode loops' graph (1: only the one-token graph)
 };
 
 int option_from_env(int i)
@@ -139,7 +141,10 @@ struct l2j_ctx {
     // Activations.  Every vector of a token has an address of its own (stride = length rounded up to 256
     // bytes): x holds the 2L+1 versions of the residual stream (version 2l+1 after the attention residual of
     // layer l, 2l+2 after its FFN residual), xb, hb and q one vector per layer.
-    float *x = nullptr, *xb = nullptr, *hb = nullptr, *q = nullptr, *logits = nullptr;
+    // They live in one allocation, twice: a whole-token kernel that hands over by value alternates between the two sets.
+    float *acts = nullptr;
+    uint64_t set_floats = 0;  // floats of one set: x | xb | q | hb | knew | vnew
+    float *x = nullptr, *xb = nullptr, *hb = nullptr, *q = nullptr, *logits = nullptr;  // set 0
     uint64_t sd = 0, sh = 0;  // strides of dim-long and hidden_dim-long vectors, in floats
     float *kcache = nullptr, *vcache = nullptr;
     float2 *rope = nullptr;
@@ -156,8 +161,10 @@ struct l2j_ctx {
 
     // launch shape of the phase kernels and their scratch
     int pk_grid = 0, pk_threads = 1024, attn_threads = 256, attn_grid = 0, attn_nsplit = 1, attn_rows = 32;
-    float *cls_val = nullptr;
-    int *cls_idx = nullptr;
+    unsigned long long *cls_part = nullptr;  // per workgroup: (index, value) of the first maximum of its classifier rows
+    unsigned long long *tstamp = nullptr;    // per position: the device's wall clock at the end of that token
+    unsigned long long *h_tstamp = nullptr;  // pinned
+    double wall_clock_hz = 1e8;
     float *attn_part = nullptr;
     float *rmsw = nullptr;  // dequantized rmsnorm weights: att (L*dim), ffn (L*dim), final (dim)
 
@@ -170,12 +177,17 @@ struct l2j_ctx {
     int *h_fault = nullptr;       // pinned
     int fused_attn_rows = 64;
     bool by_value = false;        // k_token hands activations over by value (no grid barriers)
+    int self_contained = 0;       // ... bit 0: and needs no k_fill_unset before it, bit 1: no k_finish after it
+    bool acts_dirty = false;      // kernels other than a self-contained k_token wrote activation vectors (of set 0) last
     float *knew = nullptr, *vnew = nullptr;  // this token's k and v rows per layer
     uint64_t skv = 0;
     TokenGeom geom{};             // set by l2j_finalize
 
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
+    hipGraph_t graph_n = nullptr;           // graph_tokens tokens in one graph (the decode loops replay it)
+    hipGraphExec_t graph_n_exec = nullptr;
+    int graph_tokens = 1;
     std::vector<hipEvent_t> events;
 
     // device sampler (allocated by its first use): the reference's Sampler object
@@ -287,13 +299,14 @@ void build_geom(l2j_ctx *c)
     t.threads = c->pk_threads;
     t.sd = (long)c->sd; t.sh = (long)c->sh;
     t.emb = c->emb; t.rmsw = c->rmsw; t.silu = c->silu; t.wcls = c->wcls; t.rope = c->rope;
+    t.set_stride = (long)c->set_floats;
     t.x = c->x; t.xb = c->xb; t.hb = c->hb; t.q = c->q; t.kcache = c->kcache; t.vcache = c->vcache; t.logits = c->logits;
     t.wq = qmat(c, L2J_WQ, 0); t.wk = qmat(c, L2J_WK, 0); t.wv = qmat(c, L2J_WV, 0); t.wo = qmat(c, L2J_WO, 0);
     t.w1 = qmat(c, L2J_W1, 0); t.w2 = qmat(c, L2J_W2, 0); t.w3 = qmat(c, L2J_W3, 0);
     t.knew = c->knew; t.vnew = c->vnew; t.skv = (long)c->skv;
     t.attn_part = c->attn_part; t.attn_counters = c->counters; t.attn_nsplit = c->attn_nsplit;
     t.sqrt_hs = sqrtf((float)c->head_size);
-    t.st = c->st; t.cls_val = c->cls_val; t.cls_idx = c->cls_idx; t.prompt = c->prompt; t.out_tokens = c->out_tokens;
+    t.st = c->st; t.cls_part = c->cls_part; t.tstamp = c->tstamp; t.prompt = c->prompt; t.out_tokens = c->out_tokens;
     t.bar_ctr = c->bar_ctr; t.nbar = c->nbar; t.fault = c->fault;
 }
 
@@ -303,7 +316,7 @@ bool geom_complete(const TokenGeom &t)
     const void *ptrs[] = {t.emb, t.rmsw, t.silu, t.wcls, t.rope, t.x, t.xb, t.hb, t.q, t.kcache, t.vcache, t.logits,
                           t.wq.codes, t.wq.gs, t.wk.codes, t.wk.gs, t.wv.codes, t.wv.gs, t.wo.codes, t.wo.gs,
                           t.w1.codes, t.w1.gs, t.w2.codes, t.w2.gs, t.w3.codes, t.w3.gs,
-                          t.knew, t.vnew, t.attn_part, t.attn_counters, t.st, t.cls_val, t.cls_idx, t.prompt, t.out_tokens, t.bar_ctr, t.fault};
+                          t.knew, t.vnew, t.attn_part, t.attn_counters, t.st, t.cls_part, t.tstamp, t.prompt, t.out_tokens, t.bar_ctr, t.fault};
     for (const void *p : ptrs)
         if (!p) return false;
     return true;
@@ -316,14 +329,15 @@ int fused_splits(const l2j_ctx *c)
     return std::max(1, o != kAuto ? o : c->pk_grid / c->cfg.n_heads);
 }
 
-// Marks every activation vector of a token unwritten (before a k_token that hands over by value).
+// Marks the activation vectors unwritten: set 0 before a k_token that hands over by value, both sets (and the
+// per-workgroup classifier results) before a self-contained one whose vectors others have written.
 hipError_t launch_fill_unset(const l2j_ctx *c, hipStream_t s)
 {
-    const uint64_t L = c->cfg.n_layers;
     FillArgs f{};
-    float *p[6] = {c->x, c->xb, c->hb, c->q, c->knew, c->vnew};
-    const uint64_t n[6] = {(2 * L + 1) * c->sd, L * c->sd, L * c->sh, L * c->sd, L * c->skv, L * c->skv};
-    for (int i = 0; i < 6; i++) { f.p[i] = p[i]; f.n[i] = (long)n[i]; }
+    f.p = c->acts;
+    f.n = (long)((c->self_contained & 1) ? 2 * c->set_floats : c->set_floats);
+    f.part = c->cls_part;
+    f.nparts = (c->self_contained & 2) ? c->pk_grid : 0;
     hipLaunchKernelGGL(k_fill_unset, dim3(c->n_cu), dim3(1024), 0, s, f);
     return hipGetLastError();
 }
@@ -355,6 +369,7 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.attn_splits = fused_splits(c);
     a.maxspin = std::max(0, c->opt[OPT_BARRIER_SPINS]);  // each poll is a memory round trip, >= 1 us
     a.by_value = c->by_value ? 1 : 0;
+    a.self_contained = l0 == 0 && l1 == c->cfg.n_layers ? c->self_contained : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
     const size_t smem = layer_smem(c);
     with_token_kernel(c, [&](auto kernel) {
@@ -423,14 +438,16 @@ hipError_t tap_copy(l2j_ctx *c, int which, int l, const float *src, uint64_t n, 
 
 // The launch sequence of one token (J/Run.java:62-169).  With taps, per-layer copies follow each
 // kernel (the pattern of Mode.TEST).
-hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
+hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps, hipEvent_t e0 = nullptr, hipEvent_t e1 = nullptr)
 {
     const l2j_config &g = c->cfg;
     hipError_t e;
     if (c->fused && !taps) {
-        if (c->by_value && (e = launch_fill_unset(c, s)) != hipSuccess) return e;
+        // (a kernel that alternates its sets of vectors marks them itself; whoever launches it marks both first when others wrote them)
+        if (c->by_value && !(c->self_contained & 1) && (e = launch_fill_unset(c, s)) != hipSuccess) return e;
         for (int l = 0; l < g.n_layers; l += c->layers_per_launch)
-            if ((e = launch_layers(c, l, std::min(g.n_layers, l + c->layers_per_launch), s)) != hipSuccess) return e;
+            if ((e = launch_layers(c, l, std::min(g.n_layers, l + c->layers_per_launch), s, e0, e1)) != hipSuccess) return e;
+        if (c->self_contained & 2) return hipSuccess;
         hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, s, cls_phase(c));
         return hipGetLastError();
     }
@@ -459,8 +476,17 @@ hipError_t launch_token(l2j_ctx *c, hipStream_t s, bool taps)
 
 // With option "graph" = 0 the kernels are launched one by one instead of replaying the graph (for tools that do
 // not follow graph launches).
+hipError_t clean_activations(l2j_ctx *c)
+{
+    if (!(c->self_contained & 1) || !c->acts_dirty) return hipSuccess;
+    c->acts_dirty = false;
+    return launch_fill_unset(c, c->stream);
+}
+
 hipError_t launch_one_token(l2j_ctx *c)
 {
+    hipError_t e = clean_activations(c);
+    if (e != hipSuccess) return e;
     return c->graph_exec ? hipGraphLaunch(c->graph_exec, c->stream) : launch_token(c, c->stream, false);
 }
 
@@ -474,9 +500,12 @@ int check_barrier_error(l2j_ctx *c)
     if (!c->fused) return L2J_OK;
     HIPCHK(hipMemcpy(c->h_fault, c->fault, sizeof(int), hipMemcpyDeviceToHost));
     if (*c->h_fault == 0) return L2J_OK;
+    HIPCHK(hipStreamSynchronize(c->stream));  // (tokens enqueued ahead fall through their waits as well)
     *c->h_fault = 0;
     HIPCHK(hipMemcpy(c->fault, c->h_fault, sizeof(int), hipMemcpyHostToDevice));
     HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));  // leave the context usable
+    HIPCHK(hipMemset(c->counters, 0, ((size_t)c->cfg.n_layers * c->cfg.n_heads + 1) * sizeof(unsigned)));
+    c->acts_dirty = true;
     return fail(L2J_E_HIP, "a bounded wait of the whole-token kernel ran out (barrier or input vector; its workgroups were not all resident)");
 }
 
@@ -485,8 +514,8 @@ int set_state(l2j_ctx *c, int token, int pos, int n_prompt)
     c->h_st->token = token;
     c->h_st->pos = pos;
     c->h_st->n_prompt = n_prompt;
-    c->h_st->pad = 0;
-    HIPCHK(hipMemcpyAsync(c->st, c->h_st, sizeof(DevState), hipMemcpyHostToDevice, c->stream));
+    // (the device owns DevState::epoch: every token adds one, and a self-contained k_token picks its set of vectors by it)
+    HIPCHK(hipMemcpyAsync(c->st, c->h_st, offsetof(DevState, epoch), hipMemcpyHostToDevice, c->stream));
     return L2J_OK;
 }
 
@@ -527,8 +556,10 @@ void destroy_graph(l2j_ctx *c)
 {
     if (c->graph_exec) (void)hipGraphExecDestroy(c->graph_exec);
     if (c->graph) (void)hipGraphDestroy(c->graph);
-    c->graph_exec = nullptr;
-    c->graph = nullptr;
+    if (c->graph_n_exec) (void)hipGraphExecDestroy(c->graph_n_exec);
+    if (c->graph_n) (void)hipGraphDestroy(c->graph_n);
+    c->graph_exec = c->graph_n_exec = nullptr;
+    c->graph = c->graph_n = nullptr;
 }
 
 uint64_t quant_bytes_of(uint64_t weights) { return (weights / kGroup) * kGroupBytes + (weights % kGroup ? kGroupBytes : 0); }
@@ -678,42 +709,96 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
     }
     if ((rc = set_state(c, 1, 0, np))) return rc;  // token 1 = BOS at pos 0 (J/Run.java:614)
 
-    // One event after every token of a batch: the stop rule (next == 1) is checked per batch, and the
-    // clock runs from the end of the first token to the end of the token that ended the loop.
-    const int batch = 32;
-    while ((int)c->events.size() < batch + 1) {
-        hipEvent_t ev;
-        HIPCHK(hipEventCreate(&ev));
-        c->events.push_back(ev);
-    }
-    hipEvent_t ev_first = c->events[batch];
+    // The stop rule (next == 1) is checked per batch of tokens, and the clock runs from the end of the first token to
+    // the end of the token that ended the loop.
     float total_ms = 0.f;
     int pos = 0;
     bool stopped = false;
-    while (pos < steps && !stopped) {
-        const int nb = std::min(batch, steps - pos);
-        for (int i = 0; i < nb; i++) {
-            HIPCHK(launch_one_token(c));
-            if (sampled && pos + i >= np) HIPCHK(launch_sampler(c, temperature, topp, -1.0f, true));  // J/Run.java:635-665
-            if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
-            HIPCHK(hipEventRecord(c->events[i], c->stream));
+    if (!sampled) {
+        // Greedy: the last kernel of every token stores the device's wall clock for its position; a full batch is one
+        // replay of the multi-token graph; and the next batch is enqueued before the host waits for the results of
+        // this one, so the GPU does not idle while the host looks for the stop token (a loop that stops has then
+        // run up to one batch too many, whose outputs are dropped).
+        const int batch = std::max(32, c->graph_tokens);
+        while ((int)c->events.size() < 2) {
+            hipEvent_t ev;
+            HIPCHK(hipEventCreate(&ev));
+            c->events.push_back(ev);
         }
-        HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
-        if (sampled) HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream));
-        if ((rc = check_barrier_error(c))) return rc;
-        if (sampled && (rc = check_sampler_status(c))) return rc;
-        int used = nb;
-        for (int i = 0; i < nb; i++) {
-            out_tokens[pos + i] = c->h_tokens[i];
-            if (c->h_tokens[i] == 1) {  // J/Run.java:670-672
-                used = i + 1;
-                stopped = true;
-                break;
+        unsigned long long t_first = 0, t_last = 0;
+        int enq = 0, nbatch = 0, done_batches = 0;  // positions enqueued; batches enqueued and processed
+        auto enqueue = [&]() -> int {
+            const int nb = std::min(batch, steps - enq);
+            if (c->graph_n_exec && nb == c->graph_tokens) {
+                HIPCHK(clean_activations(c));
+                HIPCHK(hipGraphLaunch(c->graph_n_exec, c->stream));
+            } else {
+                for (int i = 0; i < nb; i++) HIPCHK(launch_one_token(c));
             }
+            HIPCHK(hipMemcpyAsync(c->h_tokens + enq, c->out_tokens + enq, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipMemcpyAsync(c->h_tstamp + enq, c->tstamp + enq, (size_t)nb * sizeof(unsigned long long), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipEventRecord(c->events[nbatch & 1], c->stream));
+            enq += nb;
+            nbatch++;
+            return L2J_OK;
+        };
+        while (pos < steps && !stopped) {
+            if (enq == pos && (rc = enqueue())) return rc;
+            const int nb = std::min(batch, steps - pos);  // the batch that starts at pos
+            if (enq < steps && nbatch == done_batches + 1 && (rc = enqueue())) return rc;
+            HIPCHK(hipEventSynchronize(c->events[done_batches & 1]));
+            done_batches++;
+            if ((rc = check_barrier_error(c))) return rc;
+            int used = nb;
+            for (int i = 0; i < nb; i++) {
+                out_tokens[pos + i] = c->h_tokens[pos + i];
+                if (c->h_tokens[pos + i] == 1) {  // J/Run.java:670-672
+                    used = i + 1;
+                    stopped = true;
+                    break;
+                }
+            }
+            if (pos == 0) t_first = c->h_tstamp[0];
+            t_last = c->h_tstamp[pos + used - 1];
+            pos += used;
         }
-        if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
-        pos += used;
+        HIPCHK(hipStreamSynchronize(c->stream));  // a batch enqueued ahead of a stop
+        if ((rc = check_barrier_error(c))) return rc;
+        total_ms = (float)((double)(t_last - t_first) / c->wall_clock_hz * 1e3);
+    } else {
+        // Sampled: the sampler's kernels follow each token's graph, and an event after every token marks its end.
+        const int batch = 32;
+        while ((int)c->events.size() < batch + 1) {
+            hipEvent_t ev;
+            HIPCHK(hipEventCreate(&ev));
+            c->events.push_back(ev);
+        }
+        hipEvent_t ev_first = c->events[batch];
+        while (pos < steps && !stopped) {
+            const int nb = std::min(batch, steps - pos);
+            for (int i = 0; i < nb; i++) {
+                HIPCHK(launch_one_token(c));
+                if (pos + i >= np) HIPCHK(launch_sampler(c, temperature, topp, -1.0f, true));  // J/Run.java:635-665
+                if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
+                HIPCHK(hipEventRecord(c->events[i], c->stream));
+            }
+            HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipStreamSynchronize(c->stream));
+            if ((rc = check_barrier_error(c))) return rc;
+            if ((rc = check_sampler_status(c))) return rc;
+            int used = nb;
+            for (int i = 0; i < nb; i++) {
+                out_tokens[pos + i] = c->h_tokens[i];
+                if (c->h_tokens[i] == 1) {  // J/Run.java:670-672
+                    used = i + 1;
+                    stopped = true;
+                    break;
+                }
+            }
+            if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
+            pos += used;
+        }
     }
     *n_out = pos;
     if (seconds) *seconds = (double)total_ms * 1e-3;
@@ -807,19 +892,27 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
     const uint64_t NL = cfg->n_layers;
     c->sd = ((uint64_t)cfg->dim + 63) / 64 * 64;
     c->sh = ((uint64_t)cfg->hidden_dim + 63) / 64 * 64;
-    TRY(dev_alloc(&c->x, (2 * NL + 1) * c->sd));
-    TRY(dev_alloc(&c->xb, NL * c->sd));
-    TRY(dev_alloc(&c->hb, NL * c->sh));
-    TRY(dev_alloc(&c->q, NL * c->sd));
+    c->skv = ((uint64_t)c->kv_dim + 63) / 64 * 64;
+    c->set_floats = (2 * NL + 1) * c->sd + 2 * NL * c->sd + NL * c->sh + 2 * NL * c->skv;
+    TRY(dev_alloc(&c->acts, 2 * c->set_floats));
+    c->x = c->acts;
+    c->xb = c->x + (2 * NL + 1) * c->sd;
+    c->q = c->xb + NL * c->sd;
+    c->hb = c->q + NL * c->sd;
+    c->knew = c->hb + NL * c->sh;
+    c->vnew = c->knew + NL * c->skv;
     TRY(dev_alloc(&c->logits, cfg->vocab_size));
     TRY(dev_alloc(&c->kcache, kvn));
     TRY(dev_alloc(&c->vcache, kvn));
     TRY(dev_alloc(&c->rope, (uint64_t)cfg->seq_len * (c->head_size / 2)));
     TRY(dev_alloc(&c->silu, kSiluTable));
     TRY(dev_alloc(&c->counters, NL * cfg->n_heads + 1));
-    c->skv = ((uint64_t)c->kv_dim + 63) / 64 * 64;
-    TRY(dev_alloc(&c->knew, NL * c->skv));
-    TRY(dev_alloc(&c->vnew, NL * c->skv));
+    TRY(dev_alloc(&c->tstamp, cfg->seq_len));
+    TRYHIP(hipHostMalloc(reinterpret_cast<void **>(&c->h_tstamp), (size_t)cfg->seq_len * sizeof(unsigned long long), hipHostMallocDefault));
+    {
+        int khz = 0;
+        if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, cfg->device) == hipSuccess && khz > 0) c->wall_clock_hz = 1e3 * khz;
+    }
     TRY(dev_alloc(&c->st, 1));
     TRY(dev_alloc(&c->prompt, cfg->seq_len));
     TRY(dev_alloc(&c->out_tokens, cfg->seq_len));
@@ -841,14 +934,13 @@ int l2j_create(const l2j_config *cfg, l2j_ctx **out)
 static void release_finalize(l2j_ctx *c)
 {
     destroy_graph(c);
-    (void)hipFree(c->cls_val);
-    (void)hipFree(c->cls_idx);
+    (void)hipFree(c->cls_part);
     (void)hipFree(c->attn_part);
     (void)hipFree(c->rmsw);
     (void)hipFree(c->bar_ctr);
     (void)hipFree(c->fault);
     if (c->h_fault) (void)hipHostFree(c->h_fault);
-    c->cls_val = nullptr; c->cls_idx = nullptr; c->attn_part = nullptr; c->rmsw = nullptr; c->bar_ctr = nullptr;
+    c->cls_part = nullptr; c->attn_part = nullptr; c->rmsw = nullptr; c->bar_ctr = nullptr;
     c->fault = nullptr; c->h_fault = nullptr;
 }
 
@@ -869,12 +961,12 @@ void l2j_destroy(l2j_ctx *c)
     }
     if (c->wcls != c->emb) (void)hipFree(c->wcls);
     (void)hipFree(c->emb);
-    float *bufs[] = {c->x, c->xb, c->hb, c->q, c->logits, c->kcache, c->vcache, c->silu};
+    float *bufs[] = {c->acts, c->logits, c->kcache, c->vcache, c->silu};
     for (float *b : bufs) (void)hipFree(b);
     (void)hipFree(c->rope);
     (void)hipFree(c->counters);
-    (void)hipFree(c->knew);
-    (void)hipFree(c->vnew);
+    (void)hipFree(c->tstamp);
+    if (c->h_tstamp) (void)hipHostFree(c->h_tstamp);
     (void)hipFree(c->st);
     (void)hipFree(c->prompt);
     (void)hipFree(c->out_tokens);
@@ -1129,8 +1221,7 @@ int l2j_finalize(l2j_ctx *c)
                 for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
             }
             int rc2;
-            if ((rc2 = dev_alloc(&c->cls_val, c->pk_grid))) return rc2;
-            if ((rc2 = dev_alloc(&c->cls_idx, c->pk_grid))) return rc2;
+            if ((rc2 = dev_alloc(&c->cls_part, c->pk_grid))) return rc2;
             if ((rc2 = dev_alloc(&c->attn_part, (uint64_t)c->cfg.n_layers * c->cfg.n_heads * c->attn_nsplit * (c->head_size + 2)))) return rc2;
             c->nbar = 5 * c->cfg.n_layers;
             if ((rc2 = dev_alloc(&c->bar_ctr, (uint64_t)c->nbar * kBarStride))) return rc2;
@@ -1154,6 +1245,8 @@ int l2j_finalize(l2j_ctx *c)
             }
             c->by_value = c->fused && c->layers_per_launch == c->cfg.n_layers && c->opt[OPT_BY_VALUE] != 0 &&
                           std::max(c->cfg.dim, c->cfg.hidden_dim) <= 4 * kPollWords * c->pk_threads;
+            c->self_contained = c->by_value ? c->opt[OPT_SELF_CONTAINED] & 3 : 0;
+            c->acts_dirty = true;  // marked unwritten ahead of the first token
             build_geom(c);
             if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
         }
@@ -1164,12 +1257,20 @@ int l2j_finalize(l2j_ctx *c)
             c->finalized = true;
             return L2J_OK;
         }
-        HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
-        hipError_t le = launch_token(c, c->stream, false);
-        hipError_t ce = hipStreamEndCapture(c->stream, &c->graph);
-        if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
-        HIPCHK(ce);
-        HIPCHK(hipGraphInstantiate(&c->graph_exec, c->graph, nullptr, nullptr, 0));
+        // One token per replay, and graph_tokens tokens per replay for the decode loops: the kernels read the token, the
+        // position and the prompt from device memory, so the same nodes serve every position.
+        c->graph_tokens = std::max(1, std::min(c->opt[OPT_GRAPH_TOKENS], c->cfg.seq_len));
+        for (int which = 0; which < (c->graph_tokens > 1 ? 2 : 1); which++) {
+            hipGraph_t *gr = which ? &c->graph_n : &c->graph;
+            hipGraphExec_t *ex = which ? &c->graph_n_exec : &c->graph_exec;
+            HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+            hipError_t le = hipSuccess;
+            for (int i = 0; i < (which ? c->graph_tokens : 1) && le == hipSuccess; i++) le = launch_token(c, c->stream, false);
+            hipError_t ce = hipStreamEndCapture(c->stream, gr);
+            if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
+            HIPCHK(ce);
+            HIPCHK(hipGraphInstantiate(ex, *gr, nullptr, nullptr, 0));
+        }
         c->finalized = true;
         return L2J_OK;
     }());
@@ -1252,6 +1353,7 @@ int l2j_forward_taps(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
             if ((rc = dev_alloc(&c->taps[w], L * n))) return rc;
         }
         if ((rc = set_state(c, token, pos, 0))) return rc;
+        c->acts_dirty = true;  // the phases launched one by one leave values in the vectors of set 0
         hipError_t e = launch_token(c, c->stream, true);
         if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
         if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
@@ -1381,11 +1483,19 @@ int l2j_read(l2j_ctx *c, int which, int layer, uint64_t off, float *dst, uint64_
         } else if (which == L2J_B_LOGITS) {
             src = c->logits; len = g.vocab_size;
         } else if (layer < 0) {
+            // the vectors of the last token: set 0, or with a self-contained token kernel the set it picked by the epoch
+            uint64_t so = 0;
+            if ((c->self_contained & 1) && !c->acts_dirty) {
+                int epoch = 0;
+                HIPCHK(hipStreamSynchronize(c->stream));
+                HIPCHK(hipMemcpy(&epoch, &c->st->epoch, sizeof(int), hipMemcpyDeviceToHost));
+                so = ((epoch - 1) & 1) ? c->set_floats : 0;
+            }
             switch (which) {
-            case L2J_B_X: src = c->x + 2ull * g.n_layers * c->sd; len = g.dim; break;  // the last layer's vectors
-            case L2J_B_XB: src = c->xb + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
-            case L2J_B_HB: src = c->hb + (uint64_t)(g.n_layers - 1) * c->sh; len = g.hidden_dim; break;
-            case L2J_B_Q: src = c->q + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
+            case L2J_B_X: src = c->x + so + 2ull * g.n_layers * c->sd; len = g.dim; break;  // the last layer's vectors
+            case L2J_B_XB: src = c->xb + so + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
+            case L2J_B_HB: src = c->hb + so + (uint64_t)(g.n_layers - 1) * c->sh; len = g.hidden_dim; break;
+            case L2J_B_Q: src = c->q + so + (uint64_t)(g.n_layers - 1) * c->sd; len = g.dim; break;
             default: return fail(L2J_E_ARG, "this buffer only exists as a per-layer tap");
             }
         } else {
@@ -1470,7 +1580,7 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
         case L2J_K_TOKEN: b = l2j_bytes_per_token(&g, pos); break;
         }
         if (bytes) *bytes = b;
-        if (kclass == L2J_K_TOKEN) {  // the whole-token kernel, then k_finish (untimed) to reset the barrier counters
+        if (kclass == L2J_K_TOKEN) {  // the whole-token kernel (and, unless it is self-contained, k_finish after it, untimed)
             if (!c->fused) return fail(L2J_E_STATE, "the whole-token kernel is switched off or does not fit this shape");
             if (rounds > 256) return fail(L2J_E_ARG, "at most 256 rounds of the whole-token kernel");
             while ((int)c->events.size() < 33 + 2 * rounds) {
@@ -1481,14 +1591,10 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
             // the rounds follow each other on the stream without a host round trip in between, as the tokens of a decode do
             for (int r = 0; r < rounds; r++) {
                 if ((rc = set_state(c, 1, pos, 0))) return rc;
-                if (c->by_value) {
-                    hipError_t ef = launch_fill_unset(c, c->stream);
-                    if (ef != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(ef));
-                }
-                hipError_t e = launch_layers(c, 0, g.n_layers, c->stream, c->events[33 + 2 * r], c->events[34 + 2 * r]);
+                HIPCHK(clean_activations(c));
+                if (c->layers_per_launch != g.n_layers) return fail(L2J_E_STATE, "the token is split over several launches");
+                hipError_t e = launch_token(c, c->stream, false, c->events[33 + 2 * r], c->events[34 + 2 * r]);
                 if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
-                hipLaunchKernelGGL(k_finish, dim3(1), dim3(256), 0, c->stream, cls_phase(c));
-                HIPCHK(hipGetLastError());
             }
             HIPCHK(hipStreamSynchronize(c->stream));
             if ((rc = check_barrier_error(c))) return rc;
@@ -1501,6 +1607,7 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
             *mean_us = total * 1e3 / rounds;
             return L2J_OK;
         }
+        c->acts_dirty = true;  // a phase launched on its own leaves values in its output vector
         const int per_round = kclass == L2J_K_CLASSIFIER ? 1 : g.n_layers;
         while ((int)c->events.size() < 2 * per_round + 33) {
             hipEvent_t ev;

@@ -46,12 +46,21 @@ __device__ __forceinline__ int ld_coh(const int *p) { return __hip_atomic_load(p
 __device__ __forceinline__ void st_coh(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_coh(unsigned *p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+__device__ __forceinline__ unsigned long long ld_coh(const unsigned long long *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_coh(unsigned long long *p, unsigned long long v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
 // ---- hand-over by value ---------------------------------------------------------------------------------
 // Instead of a barrier, a consumer can wait for the data itself: before a token every activation vector is
 // filled with kUnset (a NaN bit pattern no computation produces), producers overwrite it with write-through
 // stores, and consumers re-read their part of the vector with device-coherent 16-byte loads until no kUnset
 // word is left.  The wait is bounded like the barrier's.
 constexpr unsigned kUnset = 0x7FC0DEADu;
+constexpr unsigned long long kUnset64 = 0x7FC0DEAD7FC0DEADull;
+
+// A workgroup's classifier result, (index, value) in one 64-bit word so that it is stored and read whole.
+__device__ __forceinline__ unsigned long long pack_max(float v, int i) { return ((unsigned long long)(unsigned)i << 32) | __float_as_uint(v); }
+__device__ __forceinline__ float max_val(unsigned long long w) { return __uint_as_float((unsigned)w); }
+__device__ __forceinline__ int max_idx(unsigned long long w) { return (int)(unsigned)(w >> 32); }
 
 __device__ __forceinline__ float4 ld_coh16(const float *p)
 {
@@ -950,8 +959,7 @@ struct ClsPhase {
     const float *w;      // (vocab, dim) fp32
     int n, vocab;
     float *logits;
-    float *part_val;     // one per workgroup
-    int *part_idx;
+    unsigned long long *part;  // one (index, value) per workgroup: the first maximum of its rows
     int nparts;
     DevState *st;
     const int *prompt;   // seq_len
@@ -960,6 +968,9 @@ struct ClsPhase {
     int nbar;
     int threads;         // workgroup size of the classifier
     Poll poll;           // how the input vector is read
+    unsigned long long *tstamp;  // seq_len: the device's wall clock at the end of the token of each position
+    float4 *unset_p;     // self-contained k_token: vectors to mark unwritten for the next token (nothing touches them
+    long unset_n4;       // during this launch), unset_n4 16-byte words; 0: none
 };
 
 constexpr int kCU = 8;
@@ -1004,6 +1015,18 @@ struct ClsRun {
         }
     }
 
+    // This thread's share of the vectors to mark unwritten.  The stores are written through to memory: left dirty in the
+    // caches, 4.6 MB of marks (7B shape) made the write-back at the end of the launch 13 us longer.
+    __device__ __forceinline__ void mark_unset()
+    {
+        const float u = __uint_as_float(kUnset);
+        v4f uv;
+        uv.x = uv.y = uv.z = uv.w = u;
+        const long step = (long)G * a.threads;
+        for (long i = (long)blockIdx.x * a.threads + 64 * wave + lane; i < a.unset_n4; i += step)
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(a.unset_p + i), "v"(uv) : "memory");
+    }
+
     // smem: as for a matvec phase, then 16 floats and 16 ints for the per-wave maxima
     __device__ __forceinline__ void run(float4 *smem4)
     {
@@ -1020,6 +1043,7 @@ struct ClsRun {
 
         float best_v = -__builtin_inff();
         int best_i = 0x7fffffff;
+        bool marked = a.unset_n4 == 0;
         for (; row < a.vocab; row += W * G) {
             float acc = 0.0f;
             for (int base = 0; base < n4; base += 64 * kCU) {
@@ -1039,14 +1063,18 @@ struct ClsRun {
                 a.logits[row] = acc;
                 if (better(acc, row, best_v, best_i)) { best_v = acc; best_i = row; }
             }
+            if (!marked) {  // between two rows, where the stores hide among the row loads
+                marked = true;
+                mark_unset();
+            }
         }
+        if (!marked) mark_unset();
         if (lane == 0) { bval[wave] = best_v; bidx[wave] = best_i; }
         __syncthreads();
         if (threadIdx.x == 0) {
             for (int w = 1; w < W; w++)
                 if (better(bval[w], bidx[w], best_v, best_i)) { best_v = bval[w]; best_i = bidx[w]; }
-            a.part_val[blockIdx.x] = best_v;
-            a.part_idx[blockIdx.x] = best_i;
+            st_coh(a.part + blockIdx.x, pack_max(best_v, best_i));  // written through: workgroup 0 may wait for it in this launch
         }
     }
 };
@@ -1072,7 +1100,8 @@ struct TokenGeom {
     long sd, sh;  // strides of dim-long and hidden-long activation vectors, in floats
     const float *emb, *rmsw, *silu, *wcls;
     const float2 *rope;
-    float *x, *xb, *hb, *q, *kcache, *vcache, *logits;
+    float *x, *xb, *hb, *q, *kcache, *vcache, *logits;  // x, xb, hb, q, knew, vnew: set 0 of two, `set_stride` floats apart
+    long set_stride;
     QMat wq, wk, wv, wo, w1, w2, w3;  // off = 0: layer 0
     float *knew, *vnew;  // this token's k and v rows per layer (stride skv), for the hand-over by value
     long skv;
@@ -1081,8 +1110,8 @@ struct TokenGeom {
     int attn_nsplit;
     float sqrt_hs;
     DevState *st;
-    float *cls_val;
-    int *cls_idx;
+    unsigned long long *cls_part;
+    unsigned long long *tstamp;
     const int *prompt;
     int *out_tokens;
     unsigned *bar_ctr;
@@ -1103,43 +1132,47 @@ __host__ __device__ inline QMat at_layer(const M &m, long floats_per_layer, int 
 }
 
 // Arguments of the phases of layer l (J/Run.java:76-159).
+// `set`: which of the two sets of activation vectors (always 0 outside a whole-token kernel that alternates them).
 template <class G>
-__host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, int l)
+__host__ __device__ inline MatvecPhase matvec_phase_of(const G &g, int kclass, int l, int set = 0)
 {
     const long dim = g.dim, hid = g.hidden, kvd = g.kv_dim;
     const long kvoff = (long)l * g.seq_len * kvd;
+    const long so = set * g.set_stride;
+    float *const x = g.x + so, *const xb = g.xb + so, *const hb = g.hb + so, *const q = g.q + so;
     MatvecPhase d{};
     d.emb = g.emb; d.rope = g.rope; d.silu = g.silu; d.st = g.st;
     d.head_size = g.head_size; d.kv_dim = g.kv_dim; d.exact_silu = g.exact_silu; d.threads = g.threads;
     switch (kclass) {
     case K_QKV:
-        d.n = g.dim; d.from_emb = l == 0; d.xin = g.x + 2 * l * g.sd; d.rmsw = g.rmsw + l * dim;
+        d.n = g.dim; d.from_emb = l == 0; d.xin = x + 2 * l * g.sd; d.rmsw = g.rmsw + l * dim;
         d.d0 = g.dim; d.d1 = d.d2 = g.kv_dim;
         d.m0 = at_layer(g.wq, dim * dim, l); d.m1 = at_layer(g.wk, dim * kvd, l); d.m2 = at_layer(g.wv, dim * kvd, l);
-        d.out0 = g.q + l * g.sd; d.out1 = g.kcache + kvoff; d.out2 = g.vcache + kvoff;
+        d.out0 = q + l * g.sd; d.out1 = g.kcache + kvoff; d.out2 = g.vcache + kvoff;
         break;
     case K_WO:
-        d.n = g.dim; d.xin = g.xb + l * g.sd; d.d0 = g.dim; d.m0 = at_layer(g.wo, dim * dim, l);
-        d.out0 = g.x + (2 * l + 1) * g.sd; d.res_src = g.x + 2 * l * g.sd; d.res_emb = l == 0;
+        d.n = g.dim; d.xin = xb + l * g.sd; d.d0 = g.dim; d.m0 = at_layer(g.wo, dim * dim, l);
+        d.out0 = x + (2 * l + 1) * g.sd; d.res_src = x + 2 * l * g.sd; d.res_emb = l == 0;
         break;
     case K_W13:
-        d.n = g.dim; d.xin = g.x + (2 * l + 1) * g.sd; d.rmsw = g.rmsw + (g.n_layers + l) * dim; d.d0 = g.hidden;
-        d.m0 = at_layer(g.w1, dim * hid, l); d.m1 = at_layer(g.w3, dim * hid, l); d.out0 = g.hb + l * g.sh;
+        d.n = g.dim; d.xin = x + (2 * l + 1) * g.sd; d.rmsw = g.rmsw + (g.n_layers + l) * dim; d.d0 = g.hidden;
+        d.m0 = at_layer(g.w1, dim * hid, l); d.m1 = at_layer(g.w3, dim * hid, l); d.out0 = hb + l * g.sh;
         break;
     default:  // K_W2
-        d.n = g.hidden; d.xin = g.hb + l * g.sh; d.d0 = g.dim; d.m0 = at_layer(g.w2, dim * hid, l);
-        d.out0 = g.x + (2 * l + 2) * g.sd; d.res_src = g.x + (2 * l + 1) * g.sd;
+        d.n = g.hidden; d.xin = hb + l * g.sh; d.d0 = g.dim; d.m0 = at_layer(g.w2, dim * hid, l);
+        d.out0 = x + (2 * l + 2) * g.sd; d.res_src = x + (2 * l + 1) * g.sd;
         break;
     }
     return d;
 }
 
 template <class G>
-__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split, int threads, int max_splits)
+__host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_per_split, int threads, int max_splits, int set = 0)
 {
     const long kvoff = (long)l * g.seq_len * g.kv_dim;
+    const long so = set * g.set_stride;
     AttnPhase t{};
-    t.q = g.q + l * g.sd; t.kc = g.kcache + kvoff; t.vc = g.vcache + kvoff; t.out = g.xb + l * g.sd;
+    t.q = g.q + so + l * g.sd; t.kc = g.kcache + kvoff; t.vc = g.vcache + kvoff; t.out = g.xb + so + l * g.sd;
     t.part = g.attn_part + (long)l * g.n_heads * g.attn_nsplit * (g.head_size + 2); t.counters = g.attn_counters + l * g.n_heads; t.st = g.st;
     t.n_heads = g.n_heads; t.kv_mul = g.kv_mul; t.head_size = g.head_size; t.kv_dim = g.kv_dim;
     t.nsplit = g.attn_nsplit; t.rows_per_split = rows_per_split; t.threads = threads;
@@ -1149,12 +1182,13 @@ __host__ __device__ inline AttnPhase attn_phase_of(const G &g, int l, int rows_p
 }
 
 template <class G>
-__host__ __device__ inline ClsPhase cls_phase_of(const G &g, int nparts)
+__host__ __device__ inline ClsPhase cls_phase_of(const G &g, int nparts, int set = 0)
 {
     ClsPhase a{};
-    a.xin = g.x + 2L * g.n_layers * g.sd; a.rmsw = g.rmsw + 2L * g.n_layers * g.dim; a.w = g.wcls;
-    a.n = g.dim; a.vocab = g.vocab; a.logits = g.logits; a.part_val = g.cls_val; a.part_idx = g.cls_idx; a.nparts = nparts;
+    a.xin = g.x + set * g.set_stride + 2L * g.n_layers * g.sd; a.rmsw = g.rmsw + 2L * g.n_layers * g.dim; a.w = g.wcls;
+    a.n = g.dim; a.vocab = g.vocab; a.logits = g.logits; a.part = g.cls_part; a.nparts = nparts;
     a.st = g.st; a.prompt = g.prompt; a.out_tokens = g.out_tokens; a.bar_ctr = g.bar_ctr; a.nbar = g.nbar; a.threads = g.threads;
+    a.tstamp = g.tstamp;
     return a;
 }
 
@@ -1182,23 +1216,28 @@ struct TokenArgs {
     int attn_splits;        // at most this many splits per head: one (head, split) item per workgroup
     int maxspin;
     int by_value;           // 1: consumers wait for the data itself (activations pre-filled with kUnset); 0: grid barriers
+    int self_contained;     // (with by_value, the whole token in this launch) bit 0: the kernel alternates between two sets of
+                            // activation vectors and marks the other one unwritten for the next token (no k_fill_unset
+                            // before it); bit 1: it does the token-loop step itself (no k_finish after it)
 };
 
-// Before a token whose phases hand over by value: every activation vector of the token is marked unwritten.
+// Before a token whose phases hand over by value: the activation vectors it will write (n floats at p, a multiple of
+// 4) and, for a self-contained token, the per-workgroup classifier results (nparts words) are marked unwritten.
 struct FillArgs {
-    float *p[6];
-    long n[6];  // floats, multiples of 4
+    float *p;
+    long n;
+    unsigned long long *part;
+    int nparts;
 };
 
 __global__ void k_fill_unset(const FillArgs a)
 {
     const float u = __uint_as_float(kUnset);
     const float4 u4 = make_float4(u, u, u, u);
-    for (int b = 0; b < 6; b++) {
-        float4 *p = reinterpret_cast<float4 *>(a.p[b]);
-        const long nq = a.n[b] >> 2;
-        for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < nq; i += (long)gridDim.x * blockDim.x) p[i] = u4;
-    }
+    float4 *p = reinterpret_cast<float4 *>(a.p);
+    const long nq = a.n >> 2;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < nq; i += (long)gridDim.x * blockDim.x) p[i] = u4;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < a.nparts; i += gridDim.x * blockDim.x) a.part[i] = kUnset64;
 }
 
 // Between two phases: every wave waits for its own stores to be acknowledged, the workgroup arrives at the
@@ -1239,21 +1278,21 @@ __device__ __forceinline__ Poll token_poll()
 }
 
 // A matvec phase of k_token: the arguments of layer l plus how its input arrives.
-__device__ __forceinline__ MatvecPhase token_phase(int kclass, int l)
+__device__ __forceinline__ MatvecPhase token_phase(int kclass, int l, int set)
 {
-    MatvecPhase d = matvec_phase_of(token_args()->g, kclass, l);
+    MatvecPhase d = matvec_phase_of(token_args()->g, kclass, l, set);
     d.poll = token_poll();
     if (d.poll.on && kclass == K_QKV) {
-        d.knew = token_args()->g.knew + l * token_args()->g.skv;
-        d.vnew = token_args()->g.vnew + l * token_args()->g.skv;
+        d.knew = token_args()->g.knew + set * token_args()->g.set_stride + l * token_args()->g.skv;
+        d.vnew = token_args()->g.vnew + set * token_args()->g.set_stride + l * token_args()->g.skv;
     }
     return d;
 }
 
 template <int W2_MODE, int TU = (W2_MODE == PH_ROW6 ? 6 : kTU)>
-__device__ __forceinline__ void token_w2(const GridBar &b, int l, float4 *smem4, int token, int pos)
+__device__ __forceinline__ void token_w2(const GridBar &b, int l, int set, float4 *smem4, int token, int pos)
 {
-    MatvecRun<W2_MODE, TU> w2(token_phase(K_W2, l));
+    MatvecRun<W2_MODE, TU> w2(token_phase(K_W2, l, set));
     handoff(b, 5 * l + 3, w2);
     w2.template run<true>(smem4, token, pos);
 }
@@ -1287,12 +1326,12 @@ struct TakeRegisters {   // a takes over what LendRegisters requested into b's r
 // the others request their first W13 item already when the Wo phase begins (the attention and Wo phases leave the
 // memory system two thirds idle), so that only half of W13's first items remain to be requested at its hand-over.
 template <int WO_MODE, int TUD = kTU, bool LEND = true>
-__device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, float4 *smem4, int token, int pos)
+__device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, int set, float4 *smem4, int token, int pos)
 {
     typedef MatvecRun<WO_MODE, (WO_MODE == PH_RES ? TUD : WO_MODE == PH_ROW6 ? 6 : kTU)> WoRun;
     typedef MatvecRun<PH_W13, TUD> W13Run;
-    WoRun wo(token_phase(K_WO, l));
-    W13Run w13(token_phase(K_W13, l));
+    WoRun wo(token_phase(K_WO, l, set));
+    W13Run w13(token_phase(K_W13, l, set));
     bool lend = false;
     if constexpr (WO_MODE == PH_RES && LEND) {
         // only in workgroups that had no attention item: the others come late, and their wait for the attention
@@ -1317,6 +1356,50 @@ __device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, float4 *sm
     w13.template run<true>(smem4, token, pos);
 }
 
+// The end of a self-contained token, in workgroup 0 once its own rows are done: it waits for the maximum of every
+// workgroup by value (the words were marked unwritten before the launch; bounded like the other waits), folds them
+// (first index of the strict maximum, J/Sampler.java:46-57), steps the token loop (J/Run.java:635-642, 668, 680)
+// as k_finish does, and marks the words unwritten again.
+__device__ __forceinline__ void token_finish(const ClsPhase &a, float4 *smem4)
+{
+    float *bval = reinterpret_cast<float *>(smem4);
+    int *bidx = reinterpret_cast<int *>(smem4) + 16;
+    __syncthreads();  // the classifier is done with its LDS
+    float bv = -__builtin_inff();
+    int bi = 0x7fffffff;
+    for (int b = threadIdx.x; b < a.nparts; b += blockDim.x) {
+        unsigned long long w = ld_coh(a.part + b);
+        int spins = 0;
+        while (w == kUnset64) {
+            if (++spins > a.poll.maxspin || ((spins & 63) == 0 && ld_coh(a.poll.fault) != 0)) { st_coh(a.poll.fault, 1); break; }
+            __builtin_amdgcn_s_sleep(4);
+            w = ld_coh(a.part + b);
+        }
+        if (better(max_val(w), max_idx(w), bv, bi)) { bv = max_val(w); bi = max_idx(w); }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off);
+        const int oi = __shfl_xor(bi, off);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bval[threadIdx.x >> 6] = bv; bidx[threadIdx.x >> 6] = bi; }
+    __syncthreads();  // every word has been read
+    for (int b = threadIdx.x; b < a.nparts; b += blockDim.x) a.part[b] = kUnset64;
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++)
+            if (better(bval[w], bidx[w], bv, bi)) { bv = bval[w]; bi = bidx[w]; }
+        if (bi == 0x7fffffff) bi = 0;  // all NaN: the reference's scan never leaves index 0
+        const int pos = a.st->pos;
+        const int next = pos < a.st->n_prompt ? a.prompt[pos] : bi;
+        a.out_tokens[pos] = next;
+        a.tstamp[pos] = wall_clock64();
+        a.st->token = next;
+        a.st->pos = pos + 1;
+        a.st->epoch = a.st->epoch + 1;
+    }
+}
+
 // TUD, TUH: chunks per lane and sub-row for the phases whose rows are dim and hidden codes long (tu_for); kTU is
 // the general case, in which the Wo and W2 phases pick their mode by the row length (row_mode).
 template <int LPR, int TUD = kTU, int TUH = kTU>
@@ -1325,49 +1408,55 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     extern __shared__ float4 smem4[];
     TokenArgsPtr t = token_args();
     const int token = t->g.st->token, pos = t->g.st->pos;
+    const int set = (t->self_contained & 1) ? t->g.st->epoch & 1 : 0;  // the other set is marked unwritten for the next token
     const int l0 = t->l0, l1 = t->l1;
     const int wo_mode = row_mode(t->g.dim), w2_mode = row_mode(t->g.hidden);
     GridBar b;
     b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
     for (int l = l0; l < l1; l++) {
         {
-            MatvecRun<PH_QKV, TUD> qkv(token_phase(K_QKV, l));
+            MatvecRun<PH_QKV, TUD> qkv(token_phase(K_QKV, l, set));
             if (l == l0) qkv.preload();             // launch order guarantees the input
             else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
             qkv.template run<true>(smem4, token, pos);
         }
         {
-            AttnPhase ap = attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads, token_args()->attn_splits);
+            AttnPhase ap = attn_phase_of(token_args()->g, l, token_args()->attn_rows, token_args()->g.threads, token_args()->attn_splits, set);
             ap.poll = token_poll();
-            ap.knew = token_args()->g.knew + l * token_args()->g.skv;
-            ap.vnew = token_args()->g.vnew + l * token_args()->g.skv;
+            ap.knew = token_args()->g.knew + set * token_args()->g.set_stride + l * token_args()->g.skv;
+            ap.vnew = token_args()->g.vnew + set * token_args()->g.set_stride + l * token_args()->g.skv;
             AttnRun<LPR> att(ap, pos);
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
         if constexpr (TUD < kTU) {  // the host picked TUD so that a row of dim codes is one step
-            token_wo_w13<PH_RES, TUD>(b, l, smem4, token, pos);
+            token_wo_w13<PH_RES, TUD>(b, l, set, smem4, token, pos);
         } else if constexpr (TUD > kTU) {  // without lending (measured at the 13B shape: 2.77 with, 2.74 ms without)
-            token_wo_w13<PH_RES, TUD, false>(b, l, smem4, token, pos);
+            token_wo_w13<PH_RES, TUD, false>(b, l, set, smem4, token, pos);
         } else {
-            if (wo_mode == PH_ROW6) token_wo_w13<PH_ROW6>(b, l, smem4, token, pos);
-            else if (wo_mode == PH_ROW) token_wo_w13<PH_ROW>(b, l, smem4, token, pos);
-            else token_wo_w13<PH_RES>(b, l, smem4, token, pos);
+            if (wo_mode == PH_ROW6) token_wo_w13<PH_ROW6>(b, l, set, smem4, token, pos);
+            else if (wo_mode == PH_ROW) token_wo_w13<PH_ROW>(b, l, set, smem4, token, pos);
+            else token_wo_w13<PH_RES>(b, l, set, smem4, token, pos);
         }
         if constexpr (TUH != kTU) {  // likewise for a row of hidden codes
-            token_w2<PH_RES, TUH>(b, l, smem4, token, pos);
+            token_w2<PH_RES, TUH>(b, l, set, smem4, token, pos);
         } else {
-            if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, smem4, token, pos);
-            else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, smem4, token, pos);
-            else token_w2<PH_RES>(b, l, smem4, token, pos);
+            if (w2_mode == PH_ROW6) token_w2<PH_ROW6>(b, l, set, smem4, token, pos);
+            else if (w2_mode == PH_ROW) token_w2<PH_ROW>(b, l, set, smem4, token, pos);
+            else token_w2<PH_RES>(b, l, set, smem4, token, pos);
         }
     }
     if (token_args()->with_cls) {
-        ClsPhase cp = cls_phase_of(token_args()->g, gridDim.x);
+        ClsPhase cp = cls_phase_of(token_args()->g, gridDim.x, set);
         cp.poll = token_poll();
+        if (token_args()->self_contained & 1) {  // the other set, for the token after this one
+            cp.unset_p = reinterpret_cast<float4 *>(token_args()->g.x + (1 - set) * token_args()->g.set_stride);
+            cp.unset_n4 = token_args()->g.set_stride >> 2;
+        }
         ClsRun cls(cp);
         handoff(b, 5 * (l1 - 1) + 4, cls);
         cls.run(smem4);
+        if ((token_args()->self_contained & 2) && blockIdx.x == 0) token_finish(cp, smem4);
     }
 }
 
@@ -1382,9 +1471,8 @@ __global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
     for (int i = threadIdx.x; i < a.nbar * (1 + kBarGroups); i += blockDim.x)
         st_coh(a.bar_ctr + (long)(i / (1 + kBarGroups)) * kBarStride + 64 * (i % (1 + kBarGroups)), 0u);
     for (int b = threadIdx.x; b < a.nparts; b += blockDim.x) {
-        const float v = a.part_val[b];
-        const int i = a.part_idx[b];
-        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+        const unsigned long long w = a.part[b];
+        if (better(max_val(w), max_idx(w), bv, bi)) { bv = max_val(w); bi = max_idx(w); }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -1401,8 +1489,10 @@ __global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
         const int pos = a.st->pos;
         const int next = pos < a.st->n_prompt ? a.prompt[pos] : bi;
         a.out_tokens[pos] = next;
+        a.tstamp[pos] = wall_clock64();
         a.st->token = next;
         a.st->pos = pos + 1;
+        a.st->epoch = a.st->epoch + 1;
     }
 }
 

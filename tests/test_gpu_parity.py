@@ -255,10 +255,14 @@ def test_kernel_timing_entry_point(orc, launch_mode):
     np.testing.assert_array_equal(after, want)
 
 
-@pytest.mark.parametrize("env", [{"L2J_BY_VALUE": "0"}, {"L2J_LAYERS_PER_LAUNCH": "1"}, {"L2J_BY_VALUE": "1"}])
+@pytest.mark.parametrize("env", [{"L2J_BY_VALUE": "0"}, {"L2J_LAYERS_PER_LAUNCH": "1"}, {"L2J_BY_VALUE": "1"},
+                                 {"L2J_SELF_CONTAINED": "0"}, {"L2J_SELF_CONTAINED": "1"}, {"L2J_SELF_CONTAINED": "2"},
+                                 {"L2J_GRAPH_TOKENS": "1"}, {"L2J_GRAPH_TOKENS": "7"}, {"L2J_GRAPH": "0"}])
 def test_whole_token_kernel_hand_over_variants(orc, monkeypatch, env):
     # the whole-token kernel with grid barriers instead of the hand-over by value, with one launch per layer (which
-    # implies barriers), and by value: same tokens as the oracle, deep enough that attention runs in several splits
+    # implies barriers), by value (the default: the kernel alternates two sets of vectors and steps the token loop
+    # itself), by value with k_fill_unset before and / or k_finish after every token, with other numbers of tokens per
+    # graph replay and without graphs: same tokens as the oracle, deep enough that attention runs in several splits
     monkeypatch.setenv("L2J_FUSE", "1")
     for k, v in env.items():
         monkeypatch.setenv(k, v)
@@ -280,6 +284,50 @@ def test_general_token_kernel_on_shapes_that_have_an_instance_of_their_own(orc, 
     rng = np.random.default_rng(6)
     for pos, tok in enumerate(rng.integers(0, shape[5], size=shape[6])):
         assert rel_err(g.forward(int(tok), pos), m.forward(int(tok), pos)) < 1e-4, pos
+
+
+def test_whole_token_kernel_between_other_launches(orc, monkeypatch):
+    """The self-contained whole-token kernel keeps its own book on which activation vectors read 'unwritten'.  Launches
+    that write those vectors behind its back (per-layer taps, phases timed on their own) must not confuse it: tokens
+    and logits of forwards mixed with such launches equal the oracle's, and the live taps name the set the last token used."""
+    monkeypatch.setenv("L2J_FUSE", "1")
+    shape = (256, 512, 3, 2, 2, 64, 40, 0)
+    m, g = make_pair(orc, shape, seed=71, realistic=True)
+    m.enable_taps()
+    tok = 1
+    for pos in range(24):
+        want = m.forward(tok, pos).copy()
+        if pos % 5 == 3:
+            got = g.forward_taps(tok, pos)            # per-phase launches: they leave values in set 0
+        elif pos % 5 == 4:
+            g.time_kernel(l2j.KERNEL.W13, pos, 1)     # a phase on its own, then the whole-token kernel again
+            got = g.forward(tok, pos)
+        else:
+            got = g.forward(tok, pos)                 # consecutive whole-token launches alternate the sets
+            x, ref = g.read(BUFFER.X), m.tap(orc.TAP_X_FFN, shape[2] - 1)   # the residual stream the classifier read
+            assert np.abs(x - ref).max() <= 2e-5 * max(1.0, float(np.abs(ref).max())), pos
+        assert rel_err(got, want) < LOGIT_TOL, pos
+        tok = int(np.argmax(want))
+    m.close(); g.close()
+
+
+def test_decode_stops_inside_a_replayed_batch(orc, monkeypatch):
+    """The decode loop replays several tokens per graph launch and enqueues the next batch before it has looked at
+    this one's tokens; a sequence that emits token 1 in the middle of a batch still ends there (J/Run.java:670-672)."""
+    monkeypatch.setenv("L2J_FUSE", "1")
+    monkeypatch.setenv("L2J_GRAPH_TOKENS", "8")
+    shape = (64, 96, 2, 4, 4, 3, 200, 1)   # a vocabulary of three: token 1 comes up within a few steps
+    for seed in range(40, 48):
+        m, g = make_pair(orc, shape, seed=seed, realistic=True)
+        want, _, _ = m.generate_greedy(np.array([2, 0, 2, 2, 0], np.int32), 200)
+        got, sec = g.decode_greedy(np.array([2, 0, 2, 2, 0], np.int32), 200)
+        np.testing.assert_array_equal(got, want)
+        assert sec >= 0.0
+        # and the context is usable afterwards: a fresh decode gives the same tokens
+        g.reset()
+        got2, _ = g.decode_greedy(np.array([2, 0, 2, 2, 0], np.int32), 200)
+        np.testing.assert_array_equal(got2, want)
+        m.close(); g.close()
 
 
 def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
