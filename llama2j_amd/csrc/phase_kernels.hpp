@@ -646,6 +646,10 @@ struct MatvecRun {
         int cur = item, cur_which = which, cur_r = r, base = 0;
         float resv0, resv1, acc0 = 0.0f, acc1 = 0.0f;
         residual(res, resv0, resv1);
+        // Everything requested so far has arrived before the loop is entered (the first step is needed at once anyway).
+        // With requests pending from the several paths that lead here, the compiler's wait insertion loses their order
+        // inside the loop and waits for all of them (vmcnt(0)) at the top of every step instead of chunk by chunk.
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         while (true) {
             int nbase = base + kStep, nitem = cur;
             const bool last_step = nbase >= nch;
