@@ -83,7 +83,7 @@ int resolve_scratch(int device)
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -109,6 +109,7 @@ const OptionDef kOptions[OPT_COUNT] = {
     {"graph", 1, false},               // 1: replay a captured hipGraph per token, 0: launch the kernels one by one
     {"self_contained", 3, false},      // k_token (by value): bit 0 alternates two sets of vectors (no k_fill_unset), bit 1 steps the token loop itself (no k_finish)
     {"graph_tokens", 32, false},       // tokens per replay of the decode loops' graph (1: only the one-token graph)
+    {"fast_steps", 1, false},          // k_token folds rows of dim codes without clamping when they are exactly one step
 };
 
 int option_from_env(int i)
@@ -350,6 +351,10 @@ auto with_token_kernel(const l2j_ctx *c, F f)
     const int lpr = attn_lpr(c);
     const int tud = tu_for(c->cfg.dim), tuh = tu_for(c->cfg.hidden_dim);
     const bool special = c->opt[OPT_TOKEN_SPECIAL] != 0;
+    if (special && c->opt[OPT_FAST_STEPS] != 0 && lpr == 32 && c->cfg.dim == 1024 * tud && c->cfg.dim % 256 == 0) {
+        if (tud == kTU) return f(k_token<32, kTU, kTU, true>);
+        if (tud == 5) return f(k_token<32, 5, kTU, true>);
+    }
     if (special && lpr == 16 && tud == 1 && tuh == 1) return f(k_token<16, 1, 1>);
     if (special && lpr == 16 && tud == 1 && tuh == 2) return f(k_token<16, 1, 2>);
     if (special && lpr == 32 && tud == 5) return f(k_token<32, 5, kTU>);
@@ -1217,7 +1222,8 @@ int l2j_finalize(l2j_ctx *c)
                                     reinterpret_cast<const void *>(k_classifier), reinterpret_cast<const void *>(k_token<16>),
                                     reinterpret_cast<const void *>(k_token<32>), reinterpret_cast<const void *>(k_token<64>),
                                     reinterpret_cast<const void *>(k_token<16, 1, 1>), reinterpret_cast<const void *>(k_token<16, 1, 2>),
-                                    reinterpret_cast<const void *>(k_token<32, 5, kTU>)};
+                                    reinterpret_cast<const void *>(k_token<32, 5, kTU>),
+                                    reinterpret_cast<const void *>(k_token<32, kTU, kTU, true>), reinterpret_cast<const void *>(k_token<32, 5, kTU, true>)};
                 for (const void *k : ks) HIPCHK(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)need));
             }
             int rc2;

@@ -348,8 +348,13 @@ constexpr int kTU = 4;  // 16-byte chunks in flight per lane per sub-row
 // workgroups, so that a wave may use 256 registers, was measured: 1.82 against 1.78 ms per 7B token.)
 // TU_ = 16-byte chunks per lane and sub-row that a wave holds at a time (64 * TU_ chunks are one step of a sub-row):
 // rows of up to 64 * TU_ chunks are one step, and a phase whose rows are shorter than its step folds empty chunks.
-template <int MODE, int TU_ = (MODE == PH_ROW6 ? 6 : kTU)>
+// FAST (row pairs whose rows are exactly one step: n == 16 * 64 * TU codes): no lane ever falls outside a row, so fold()
+// neither clamps nor masks and reads the staged vector at constant distances from one per-lane address: 20 vector
+// instructions fewer per step of 380 (7B shape: 13 us per token).  The requests keep their general form: with the scale
+// loads issued from a scalar base at constant offsets the token took 35 us longer, without the clamps 2 us longer.
+template <int MODE, int TU_ = (MODE == PH_ROW6 ? 6 : kTU), bool FAST = false>
 struct MatvecRun {
+    static_assert(!FAST || (MODE != PH_ROW && MODE != PH_ROW6), "whole-step streaming is for row pairs");
     // PH_ROW streams one row with 2*kTU chunks in flight: "sub-row 1" is the same row kTU*64 chunks further on.
     // PH_ROW6 holds six chunks per lane and sub-row instead of four: a row of 513..768 chunks (11008 codes are 688) is
     // then one step, requested whole ahead of the hand-over, where PH_ROW would request its tail only after the first
@@ -544,6 +549,25 @@ struct MatvecRun {
     template <bool REFILL>
     __device__ __forceinline__ void fold(int base, const float4 *xs, const float *sumx, float &acc0, float &acc1, int nbase)
     {
+        if constexpr (FAST) {
+            const float4 *xp = xs + lane;
+            const float *sp = sumx + lane;
+#pragma unroll
+            for (int u = 0; u < TU; u++) {
+                const uint4 a0 = w0[u], a1 = w1[u];
+                const float2 g0 = s0[u], g1 = s1[u];
+                const float4 x0 = xp[64 * u], x1 = xp[nch + 64 * u], x2 = xp[2 * nch + 64 * u], x3 = xp[3 * nch + 64 * u];
+                const float sx = sp[64 * u];
+                acc0 += fmaf(g0.x, dot16(a0, x0, x1, x2, x3), g0.y * sx);
+                acc1 += fmaf(g1.x, dot16(a1, x0, x1, x2, x3), g1.y * sx);
+                if (REFILL) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    issue_chunk(nbase, u);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < TU; u++) {
             const uint4 a0 = w0[u], a1 = w1[u];
@@ -1329,11 +1353,11 @@ struct TakeRegisters {   // a takes over what LendRegisters requested into b's r
 // Wo + residual, then rmsnorm + W1,W3 + SwiGLU.  With Wo in row pairs only half the waves of the 7B shape have a Wo item;
 // the others request their first W13 item already when the Wo phase begins (the attention and Wo phases leave the
 // memory system two thirds idle), so that only half of W13's first items remain to be requested at its hand-over.
-template <int WO_MODE, int TUD = kTU, bool LEND = true>
+template <int WO_MODE, int TUD = kTU, bool LEND = true, bool FAST = false>
 __device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, int set, float4 *smem4, int token, int pos)
 {
-    typedef MatvecRun<WO_MODE, (WO_MODE == PH_RES ? TUD : WO_MODE == PH_ROW6 ? 6 : kTU)> WoRun;
-    typedef MatvecRun<PH_W13, TUD> W13Run;
+    typedef MatvecRun<WO_MODE, (WO_MODE == PH_RES ? TUD : WO_MODE == PH_ROW6 ? 6 : kTU), FAST && WO_MODE == PH_RES> WoRun;
+    typedef MatvecRun<PH_W13, TUD, FAST> W13Run;
     WoRun wo(token_phase(K_WO, l, set));
     W13Run w13(token_phase(K_W13, l, set));
     bool lend = false;
@@ -1406,7 +1430,9 @@ __device__ __forceinline__ void token_finish(const ClsPhase &a, float4 *smem4)
 
 // TUD, TUH: chunks per lane and sub-row for the phases whose rows are dim and hidden codes long (tu_for); kTU is
 // the general case, in which the Wo and W2 phases pick their mode by the row length (row_mode).
-template <int LPR, int TUD = kTU, int TUH = kTU>
+// FASTD: a row of dim codes is exactly one step of TUD chunks per lane (dim == 1024 * TUD, checked on the host): the
+// phases whose rows are dim long (QKV, Wo, W1/W3) fold it without clamping (MatvecRun).
+template <int LPR, int TUD = kTU, int TUH = kTU, bool FASTD = false>
 __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
 {
     extern __shared__ float4 smem4[];
@@ -1419,7 +1445,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
     for (int l = l0; l < l1; l++) {
         {
-            MatvecRun<PH_QKV, TUD> qkv(token_phase(K_QKV, l, set));
+            MatvecRun<PH_QKV, TUD, FASTD> qkv(token_phase(K_QKV, l, set));
             if (l == l0) qkv.preload();             // launch order guarantees the input
             else handoff(b, 5 * (l - 1) + 4, qkv);  // after W2 of the previous layer
             qkv.template run<true>(smem4, token, pos);
@@ -1433,7 +1459,9 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
             handoff(b, 5 * l, att);
             att.template run<true>(reinterpret_cast<float *>(smem4));
         }
-        if constexpr (TUD < kTU) {  // the host picked TUD so that a row of dim codes is one step
+        if constexpr (FASTD) {  // (lending as below: only with four chunks per lane)
+            token_wo_w13<PH_RES, TUD, TUD == kTU, true>(b, l, set, smem4, token, pos);
+        } else if constexpr (TUD < kTU) {  // the host picked TUD so that a row of dim codes is one step
             token_wo_w13<PH_RES, TUD>(b, l, set, smem4, token, pos);
         } else if constexpr (TUD > kTU) {  // without lending (measured at the 13B shape: 2.77 with, 2.74 ms without)
             token_wo_w13<PH_RES, TUD, false>(b, l, set, smem4, token, pos);
