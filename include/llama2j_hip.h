@@ -2,8 +2,8 @@
  * libllama2j_hip.so - C ABI of the MI355X (gfx950) mode of llama2j's per-token forward pass.
  *
  * The library owns every device buffer (weights, activations, KV cache), takes llama2j's own
- * weight formats, and runs the whole token as one hand-written gfx950 kernel (plus a one-workgroup
- * argmax/step kernel), captured in a hipGraph and replayed on one GPU.  It is the
+ * weight formats, and runs the whole token, argmax and token-loop step included, as one hand-written
+ * gfx950 kernel, captured in a hipGraph and replayed on one GPU.  It is the
  * seam a `Mode.HIP` plugs into beside the reference's CPU and CUDA modes: each entry point
  * names the reference interface it replaces (paths relative to the reference root,
  * J/ = src/main/java/com/lastbot/llama2j/, K/ = J/kernel/).
@@ -87,9 +87,14 @@ int l2j_device_count(void);
  * defaults (environment variable L2J_<NAME>, read once by l2j_create; unset: the built-in value), this call overrides
  * one of them, and the library never reads the environment afterwards.  Before l2j_finalize: "threads", "grid",
  * "attn_threads", "attn_rows", "attn_nsplit", "fused_attn_rows", "fused_attn_splits", "barrier_spins", "fuse" (1 whole-token
- * kernel, 0 one launch per phase, -1 by model size), "layers_per_launch", "by_value", "token_special", "graph" (0: launch
- * kernel by kernel instead of replaying a captured hipGraph).  At any time: "sampler_scan", "sampler_exp_wgs". */
+ * kernel, 0 one launch per phase, -1 by model size), "layers_per_launch", "by_value", "self_contained", "fast_steps",
+ * "token_special", "graph" (0: launch kernel by kernel instead of replaying captured hipGraphs), "graph_tokens" (tokens per
+ * replay in the decode loops).  At any time: "sampler_scan", "sampler_exp_wgs", "fallback" (1: when a bounded wait of the
+ * whole-token kernel runs out, because something else holds compute units of the GPU, the context switches to one launch
+ * per phase for good and repeats the call; 0: the call returns L2J_E_HIP).  l2j_get_option reads the value in force
+ * ("fuse" reads 0 after such a switch). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
+int l2j_get_option(l2j_ctx *ctx, const char *name, int32_t *value);
 
 /* = allocateQuantAndCopyToDevice (J/ContextCUDA.java:138-158, J/TransformerWeights.java:238-257).
  * `ref_bytes` is the exact payload of a .quant cache: ceil(n/256) groups of 264 bytes

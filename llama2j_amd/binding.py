@@ -89,6 +89,7 @@ def _signatures():
         "l2j_last_error": (C.c_char_p, []),
         "l2j_ctx_last_error": (C.c_int, [vp, C.c_char_p, C.c_int32]),
         "l2j_set_option": (C.c_int, [vp, C.c_char_p, C.c_int32]),
+        "l2j_get_option": (C.c_int, [vp, C.c_char_p, i32p]),
         "l2j_device_count": (C.c_int, []),
         "l2j_upload_quant": (C.c_int, [vp, C.c_int, u8p, C.c_uint64]),
         "l2j_upload_quant_layer": (C.c_int, [vp, C.c_int, C.c_int, u8p, C.c_uint64]),
@@ -300,6 +301,11 @@ class Transformer:
         buf = C.create_string_buffer(1024)
         self._check(lib().l2j_ctx_last_error(self._h, buf, len(buf)))
         return buf.value.decode(errors="replace")
+
+    def get_option(self, name):
+        v = C.c_int32(0)
+        self._check(lib().l2j_get_option(self._h, name.encode(), C.byref(v)))
+        return v.value
 
     def set_option(self, name, value):
         self._check(lib().l2j_set_option(self._h, name.encode(), int(value)))

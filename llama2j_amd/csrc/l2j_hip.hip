@@ -83,7 +83,7 @@ int resolve_scratch(int device)
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -110,6 +110,7 @@ const OptionDef kOptions[OPT_COUNT] = {
     {"self_contained", 3, false},      // k_token (by value): bit 0 alternates two sets of vectors (no k_fill_unset), bit 1 steps the token loop itself (no k_finish)
     {"graph_tokens", 32, false},       // tokens per replay of the decode loops' graph (1: only the one-token graph)
     {"fast_steps", 1, false},          // k_token folds rows of dim codes without clamping when they are exactly one step
+    {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
 };
 
 int option_from_env(int i)
@@ -499,7 +500,43 @@ hipError_t launch_one_token(l2j_ctx *c)
 // of this process take turns (each entry point synchronizes before it returns).
 std::mutex g_forward_mu;
 
-// After a synchronize: a workgroup whose bounded wait at a grid barrier ran out has set the flag.
+void destroy_graph(l2j_ctx *c)
+{
+    if (c->graph_exec) (void)hipGraphExecDestroy(c->graph_exec);
+    if (c->graph) (void)hipGraphDestroy(c->graph);
+    if (c->graph_n_exec) (void)hipGraphExecDestroy(c->graph_n_exec);
+    if (c->graph_n) (void)hipGraphDestroy(c->graph_n);
+    c->graph_exec = c->graph_n_exec = nullptr;
+    c->graph = c->graph_n = nullptr;
+}
+
+// One token per replay, and graph_tokens tokens per replay for the decode loops: the kernels read the token, the
+// position and the prompt from device memory, so the same nodes serve every position.
+int capture_graphs(l2j_ctx *c)
+{
+    destroy_graph(c);
+    if (c->opt[OPT_GRAPH] == 0) return L2J_OK;
+    c->graph_tokens = std::max(1, std::min(c->opt[OPT_GRAPH_TOKENS], c->cfg.seq_len));
+    for (int which = 0; which < (c->graph_tokens > 1 ? 2 : 1); which++) {
+        hipGraph_t *gr = which ? &c->graph_n : &c->graph;
+        hipGraphExec_t *ex = which ? &c->graph_n_exec : &c->graph_exec;
+        HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+        hipError_t le = hipSuccess;
+        for (int i = 0; i < (which ? c->graph_tokens : 1) && le == hipSuccess; i++) le = launch_token(c, c->stream, false);
+        hipError_t ce = hipStreamEndCapture(c->stream, gr);
+        if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
+        HIPCHK(ce);
+        HIPCHK(hipGraphInstantiate(ex, *gr, nullptr, nullptr, 0));
+    }
+    return L2J_OK;
+}
+
+constexpr int kRepeatToken = 1;  // check_barrier_error: the context now launches phase by phase; run the token(s) again
+
+// After a synchronize: a workgroup whose bounded wait ran out has set the flag.  The whole-token kernel needs all its
+// workgroups resident at once; when something else holds compute units (another process on the GPU) its waits run
+// out.  With the "fallback" option the context then gives the whole-token kernel up for good: one launch per phase
+// needs no residency, and the caller repeats what failed (kRepeatToken).
 int check_barrier_error(l2j_ctx *c)
 {
     if (!c->fused) return L2J_OK;
@@ -511,6 +548,15 @@ int check_barrier_error(l2j_ctx *c)
     HIPCHK(hipMemset(c->bar_ctr, 0, (size_t)c->nbar * kBarStride * sizeof(unsigned)));  // leave the context usable
     HIPCHK(hipMemset(c->counters, 0, ((size_t)c->cfg.n_layers * c->cfg.n_heads + 1) * sizeof(unsigned)));
     c->acts_dirty = true;
+    if (c->opt[OPT_FALLBACK] != 0) {
+        c->fused = false;
+        c->by_value = false;
+        c->self_contained = 0;
+        c->opt[OPT_FUSE] = 0;
+        int rc = capture_graphs(c);
+        if (rc) return rc;
+        return kRepeatToken;
+    }
     return fail(L2J_E_HIP, "a bounded wait of the whole-token kernel ran out (barrier or input vector; its workgroups were not all resident)");
 }
 
@@ -557,15 +603,6 @@ int unpack_into(l2j_ctx *c, QTensor &t, uint64_t group0, const uint8_t *ref_byte
     return rc;
 }
 
-void destroy_graph(l2j_ctx *c)
-{
-    if (c->graph_exec) (void)hipGraphExecDestroy(c->graph_exec);
-    if (c->graph) (void)hipGraphDestroy(c->graph);
-    if (c->graph_n_exec) (void)hipGraphExecDestroy(c->graph_n_exec);
-    if (c->graph_n) (void)hipGraphDestroy(c->graph_n);
-    c->graph_exec = c->graph_n_exec = nullptr;
-    c->graph = c->graph_n = nullptr;
-}
 
 uint64_t quant_bytes_of(uint64_t weights) { return (weights / kGroup) * kGroupBytes + (weights % kGroup ? kGroupBytes : 0); }
 
@@ -999,6 +1036,20 @@ int l2j_set_option(l2j_ctx *c, const char *name, int32_t value)
     }());
 }
 
+int l2j_get_option(l2j_ctx *c, const char *name, int32_t *value)
+{
+    return ctx_rc(c, [&]() -> int {
+        if (!c || !name || !value) return fail(L2J_E_ARG, "null argument");
+        for (int i = 0; i < OPT_COUNT; i++) {
+            if (strcmp(name, kOptions[i].name) != 0) continue;
+            std::lock_guard<std::mutex> lock(c->upload_mu);
+            *value = c->opt[i];
+            return L2J_OK;
+        }
+        return fail(L2J_E_ARG, std::string("unknown option '") + name + "'");
+    }());
+}
+
 int l2j_get_config(l2j_ctx *c, l2j_config *cfg)
 {
     return ctx_rc(c, [&]() -> int {
@@ -1257,26 +1308,9 @@ int l2j_finalize(l2j_ctx *c)
             if (!geom_complete(c->geom)) return fail(L2J_E_STATE, "internal: a device buffer of the forward pass was not allocated");
         }
 
-        // capture one token
         HIPCHK(hipStreamSynchronize(c->stream));
-        if (c->opt[OPT_GRAPH] == 0) {
-            c->finalized = true;
-            return L2J_OK;
-        }
-        // One token per replay, and graph_tokens tokens per replay for the decode loops: the kernels read the token, the
-        // position and the prompt from device memory, so the same nodes serve every position.
-        c->graph_tokens = std::max(1, std::min(c->opt[OPT_GRAPH_TOKENS], c->cfg.seq_len));
-        for (int which = 0; which < (c->graph_tokens > 1 ? 2 : 1); which++) {
-            hipGraph_t *gr = which ? &c->graph_n : &c->graph;
-            hipGraphExec_t *ex = which ? &c->graph_n_exec : &c->graph_exec;
-            HIPCHK(hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
-            hipError_t le = hipSuccess;
-            for (int i = 0; i < (which ? c->graph_tokens : 1) && le == hipSuccess; i++) le = launch_token(c, c->stream, false);
-            hipError_t ce = hipStreamEndCapture(c->stream, gr);
-            if (le != hipSuccess) return fail(L2J_E_HIP, std::string("capture launch: ") + hipGetErrorString(le));
-            HIPCHK(ce);
-            HIPCHK(hipGraphInstantiate(ex, *gr, nullptr, nullptr, 0));
-        }
+        const int rcg = capture_graphs(c);
+        if (rcg) return rcg;
         c->finalized = true;
         return L2J_OK;
     }());
@@ -1321,11 +1355,13 @@ int l2j_forward(l2j_ctx *c, int32_t token, int32_t pos, float *logits)
         std::lock_guard<std::mutex> forward_lock(g_forward_mu);
         int rc = check_forward_args(c, token, pos);
         if (rc) return rc;
-        if ((rc = set_state(c, token, pos, 0))) return rc;
-        HIPCHK(launch_one_token(c));
-        if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream));
-        return check_barrier_error(c);
+        do {  // (a second time, phase by phase, when the whole-token kernel's waits ran out)
+            if ((rc = set_state(c, token, pos, 0))) return rc;
+            HIPCHK(launch_one_token(c));
+            if (logits) HIPCHK(hipMemcpyAsync(logits, c->logits, (size_t)c->cfg.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipStreamSynchronize(c->stream));
+        } while ((rc = check_barrier_error(c)) == kRepeatToken);
+        return rc;
     }());
 }
 
@@ -1336,12 +1372,14 @@ int l2j_forward_argmax(l2j_ctx *c, int32_t token, int32_t pos, int32_t *next)
         if (!next) return fail(L2J_E_ARG, "null argument");
         int rc = check_forward_args(c, token, pos);
         if (rc) return rc;
-        if ((rc = set_state(c, token, pos, 0))) return rc;
-        HIPCHK(launch_one_token(c));
-        HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
-        HIPCHK(hipStreamSynchronize(c->stream));
-        *next = c->h_tokens[0];
-        return check_barrier_error(c);
+        do {
+            if ((rc = set_state(c, token, pos, 0))) return rc;
+            HIPCHK(launch_one_token(c));
+            HIPCHK(hipMemcpyAsync(c->h_tokens, &c->st->token, sizeof(int), hipMemcpyDeviceToHost, c->stream));
+            HIPCHK(hipStreamSynchronize(c->stream));
+            *next = c->h_tokens[0];
+        } while ((rc = check_barrier_error(c)) == kRepeatToken);
+        return rc;
     }());
 }
 
@@ -1373,7 +1411,9 @@ int l2j_decode_greedy(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32
 {
     return ctx_rc(c, [&]() -> int {
         std::lock_guard<std::mutex> forward_lock(g_forward_mu);
-        return decode_loop(c, prompt, n_prompt, steps, false, 0.0f, 0.0f, 0, out_tokens, n_out, seconds);
+        int rc;  // (the whole loop once more, phase by phase, when the whole-token kernel's waits ran out)
+        while ((rc = decode_loop(c, prompt, n_prompt, steps, false, 0.0f, 0.0f, 0, out_tokens, n_out, seconds)) == kRepeatToken) {}
+        return rc;
     }());
 }
 
@@ -1384,7 +1424,9 @@ int l2j_decode_sample(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32
         std::lock_guard<std::mutex> forward_lock(g_forward_mu);
         int rc = check_sampler_args(temperature, topp);
         if (rc) return rc;
-        return decode_loop(c, prompt, n_prompt, steps, temperature != 0.0f, temperature, topp, rng_seed, out_tokens, n_out, seconds);
+        while ((rc = decode_loop(c, prompt, n_prompt, steps, temperature != 0.0f, temperature, topp, rng_seed, out_tokens, n_out, seconds)) ==
+               kRepeatToken) {}
+        return rc;
     }());
 }
 
@@ -1603,7 +1645,8 @@ int l2j_time_kernel(l2j_ctx *c, int kclass, int32_t pos, int32_t rounds, double 
                 if (e != hipSuccess) return fail(L2J_E_HIP, std::string("launch: ") + hipGetErrorString(e));
             }
             HIPCHK(hipStreamSynchronize(c->stream));
-            if ((rc = check_barrier_error(c))) return rc;
+            if ((rc = check_barrier_error(c)))
+                return rc == kRepeatToken ? fail(L2J_E_HIP, "a bounded wait of the whole-token kernel ran out; the context now launches phase by phase") : rc;
             double total = 0.0;
             for (int r = 0; r < rounds; r++) {
                 float ms = 0.f;

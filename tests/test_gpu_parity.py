@@ -336,13 +336,14 @@ def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
     shape = (64, 96, 2, 4, 2, 40, 32, 1)
     monkeypatch.setenv("L2J_FUSE", "1")
     monkeypatch.setenv("L2J_BARRIER_SPINS", "0")
+    monkeypatch.setenv("L2J_FALLBACK", "0")
     m, bad = make_pair(orc, shape, seed=50)
     failures = 0
     for pos in range(8):
         try:
             bad.forward(3, pos)
         except l2j.L2JError as e:
-            assert e.code == -4 and "barrier" in str(e)
+            assert e.code == -4 and "bounded wait" in str(e)
             failures += 1
     assert failures > 0
     monkeypatch.setenv("L2J_BARRIER_SPINS", "20000")
@@ -351,6 +352,32 @@ def test_barrier_time_out_is_reported_not_hung(orc, monkeypatch):
         assert rel_err(good.forward(3, pos), m2.forward(3, pos)) < 1e-4
     # the context whose waits expired works again once the stale state is gone
     bad.close()
+
+
+def test_waits_that_run_out_fall_back_to_one_launch_per_phase(orc, monkeypatch):
+    """The whole-token kernel needs every workgroup resident; when its bounded waits run out (forced here by a spin limit of
+    zero; in the field by another process holding compute units) the context switches to one launch per phase for good
+    and repeats the call: the caller sees correct results, not an error."""
+    shape = (64, 96, 2, 4, 2, 40, 32, 1)
+    monkeypatch.setenv("L2J_FUSE", "1")
+    monkeypatch.setenv("L2J_BARRIER_SPINS", "0")
+    for entry in ("forward", "forward_argmax", "decode_greedy", "decode_sample"):
+        m, g = make_pair(orc, shape, seed=51, realistic=True)
+        assert g.get_option("fuse") == 1 and g.get_option("fallback") == 1
+        prompt = orc.synth_prompt(51, 3, shape[5])
+        if entry == "forward":
+            assert rel_err(g.forward(3, 0), m.forward(3, 0)) < 1e-4
+        elif entry == "forward_argmax":
+            assert g.forward_argmax(3, 0) == int(np.argmax(m.forward(3, 0)))
+        elif entry == "decode_greedy":
+            np.testing.assert_array_equal(g.decode_greedy(prompt, 24)[0], m.generate_greedy(prompt, 24)[0])
+        else:
+            np.testing.assert_array_equal(g.decode_sample(prompt, 24, 0.0, 0.9, 7)[0], m.generate_greedy(prompt, 24)[0])
+        assert g.get_option("fuse") == 0          # the switch is for good
+        m.reset()
+        for pos in range(4):                      # and the context goes on working, phase by phase
+            assert rel_err(g.forward(5, pos), m.forward(5, pos)) < 1e-4
+        m.close(); g.close()
 
 
 def test_two_contexts_decode_from_two_threads(orc, launch_mode):
