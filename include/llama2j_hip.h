@@ -138,7 +138,8 @@ int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int
 /* ---- sampling on the device: J/Sampler.java and the sampling branch of J/Run.java:643-665 ----
  * The context holds one sampler = the reference's Sampler object: a java.util.Random and the ProbIndex
  * array that sample_topp sorts whole, so that entries of earlier calls take part in later ones
- * (J/Sampler.java:17-18, 92-97).  vocab_size is limited to 36864 (the probabilities are kept in LDS). */
+ * (J/Sampler.java:17-18, 92-97).  Any vocab_size >= 2: up to 36864 probabilities are kept in LDS, larger vocabularies are
+ * sampled where they lie in device memory (same results, slower). */
 /* = new Sampler(rngSeed, vocab_size) (J/Sampler.java:24-31, J/Run.java:620). */
 int l2j_sampler_seed(l2j_ctx *ctx, int64_t rng_seed);
 /* One sampling step (J/Run.java:643-665): temperature 0 = Sampler.argmax; else logits /= temperature,
@@ -206,7 +207,7 @@ int l2j_get_config(l2j_ctx *ctx, l2j_config *cfg);
  *  - 131070) * (sigma / 37837.2265625f), stream 0 = embedding, 1..10 = quant tensors in file
  * order, 11 = classifier, and quantizes the ten quant tensors with the reference's encoder. */
 int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
-/* Measurement and test: the running float32 sums of n <= 36864 non-negative terms in element order, as the reference's
+/* Measurement and test: the running float32 sums of n <= 16777216 non-negative terms in element order, as the reference's
  * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
  * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
 int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);

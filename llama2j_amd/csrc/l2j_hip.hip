@@ -72,7 +72,7 @@ int resolve_scratch(int device)
     if (!p) return fail(L2J_E_HIP, "hipGetSymbolAddress(scratch) returned a null address");
     // (the largest input needs more than the default 64 KB of dynamic LDS)
     const int lds = (((kSampleMaxVocab + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
-    HIPCHK(hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    HIPCHK(hipFuncSetAttribute((const void *)k_running_sums<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     g_scratch_ptr[device] = p;
     return L2J_OK;
 }
@@ -626,23 +626,31 @@ void free_sampler(l2j_ctx *c)
     c->h_ss = nullptr;
 }
 
+// dynamic LDS of the sampler's one-workgroup kernels: the terms, padded to whole steps of the single-lane sum plus one
+size_t sampler_lds_bytes(int n)
+{
+    return n <= kSampleMaxVocab ? (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float) : 0;
+}
+
 int alloc_sampler(l2j_ctx *c)
 {
     const int n = c->cfg.vocab_size;
     int rc;
     for (int i = 0; i < 2; i++) {
-        if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n))) return rc;
+        if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n + 4))) return rc;   // (read in 16-byte words: stage_terms)
         if ((rc = dev_alloc(&c->pi_idx[i], (uint64_t)n))) return rc;
     }
     size_t bytes = 0;
     HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream, nullptr));
     c->sort_temp_bytes = bytes;
     HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
-    if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n))) return rc;
+    if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n + 4))) return rc;
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
-    const int lds = (((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * (int)sizeof(float);
-    HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    if (n <= kSampleMaxVocab) {
+        const int lds = (int)sampler_lds_bytes(n);
+        HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    }
     return dev_alloc(&c->ss, 1);   // last: its presence says that the sampler is complete
 }
 
@@ -650,7 +658,6 @@ int ensure_sampler(l2j_ctx *c)
 {
     if (c->ss) return L2J_OK;
     const int n = c->cfg.vocab_size;
-    if (n > kSampleMaxVocab) return fail(L2J_E_SIZE, "device sampler: vocab_size above 36864 does not fit the LDS");
     if (n < 2) return fail(L2J_E_SIZE, "device sampler: vocab_size below 2");
     const int rc = alloc_sampler(c);
     if (rc) free_sampler(c);
@@ -690,15 +697,17 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     a.st = in_loop ? c->st : nullptr;
     a.out_tokens = c->out_tokens;
     a.scan = c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0;
-    const int exp_wgs = std::min(1024, std::max(0, c->opt[OPT_SAMPLER_EXP_WGS]));   // 0: the exponentials in k_sample_probs' one workgroup
+    const bool in_lds = n <= kSampleMaxVocab;   // else the kernels work in device memory, where k_sample_exp leaves the exponentials
+    const int exp_wgs = std::min(1024, std::max(in_lds ? 0 : 1, c->opt[OPT_SAMPLER_EXP_WGS]));   // 0: the exponentials in k_sample_probs' one workgroup
     a.expbuf = exp_wgs > 0 ? c->sample_exp : nullptr;
     if (a.expbuf) {
         hipLaunchKernelGGL(k_sample_exp, dim3(exp_wgs), dim3(1024), 0, c->stream, a);
         hipError_t ee = hipGetLastError();
         if (ee != hipSuccess) return ee;
     }
-    const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
-    hipLaunchKernelGGL(k_sample_probs, dim3(1), dim3(1024), lds, c->stream, a);
+    const size_t lds = sampler_lds_bytes(n);
+    if (in_lds) hipLaunchKernelGGL(k_sample_probs<true>, dim3(1), dim3(1024), lds, c->stream, a);
+    else hipLaunchKernelGGL(k_sample_probs<false>, dim3(1), dim3(1024), 0, c->stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.plain) return e;
     size_t bytes = c->sort_temp_bytes;
@@ -709,7 +718,8 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     const int sorted = in_second ? other : cur;   // the array stays there until the next call
     a.sorted_prob = c->pi_prob[sorted]; a.sorted_idx = c->pi_idx[sorted];
     c->pi_cur = sorted;
-    hipLaunchKernelGGL(k_topp_pick, dim3(1), dim3(1024), lds, c->stream, a);
+    if (in_lds) hipLaunchKernelGGL(k_topp_pick<true>, dim3(1), dim3(1024), lds, c->stream, a);
+    else hipLaunchKernelGGL(k_topp_pick<false>, dim3(1), dim3(1024), 0, c->stream, a);
     return hipGetLastError();
 }
 
@@ -1471,15 +1481,16 @@ int l2j_running_sums(l2j_ctx *c, const float *terms, int32_t n, float *sums)
     return ctx_rc(c, [&]() -> int {
         std::lock_guard<std::mutex> forward_lock(g_forward_mu);
         if (!c || !terms || !sums) return fail(L2J_E_ARG, "null argument");
-        if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "1 to 36864 terms");
+        if (n <= 0 || n > (1 << 24)) return fail(L2J_E_SIZE, "1 to 16777216 terms");
         HIPCHK(hipSetDevice(c->cfg.device));
         float *d = nullptr;
         HIPCHK(hipMalloc(reinterpret_cast<void **>(&d), (size_t)n * sizeof(float)));
-        const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
-        hipError_t e = hipFuncSetAttribute((const void *)k_running_sums, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e == hipSuccess) e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        const size_t lds = sampler_lds_bytes(n);
+        hipError_t e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
-            hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0);
+            const int scan_on = c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0;
+            if (n <= kSampleMaxVocab) hipLaunchKernelGGL(k_running_sums<true>, dim3(1), dim3(1024), lds, c->stream, d, n, scan_on);
+            else hipLaunchKernelGGL(k_running_sums<false>, dim3(1), dim3(1024), 0, c->stream, d, n, 1);
             e = hipGetLastError();
         }
         if (e == hipSuccess) e = hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream);
@@ -1504,9 +1515,9 @@ int l2j_running_sums_noalloc(l2j_ctx *c, const float *terms, int32_t n, float *s
         }
         if (!d) return fail(L2J_E_STATE, "l2j_running_sums_noalloc: the static device buffer was not resolved on this device");
         // The buffer keeps the last call's contents; the kernel reads only the n terms copied in here, so nothing needs clearing.
-        const size_t lds = (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float);
+        const size_t lds = sampler_lds_bytes(n);
         HIPCHK(hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream));
-        hipLaunchKernelGGL(k_running_sums, dim3(1), dim3(1024), lds, c->stream, d, n, c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0);
+        hipLaunchKernelGGL(k_running_sums<true>, dim3(1), dim3(1024), lds, c->stream, d, n, c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0);
         HIPCHK(hipGetLastError());
         HIPCHK(hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream));
         HIPCHK(hipStreamSynchronize(c->stream));

@@ -5,11 +5,11 @@
 // The reference adds the probabilities one by one into a float (the softmax denominator, the CDF of
 // sample, the cumulative probability of sample_topp); float addition is not associative, so the order
 // matters.  As one dependent chain in a single lane such a sum costs 3.4 ns per element (the eight-cycle
-// latency of a dependent v_add_f32, measured; 0.11 ms for 32000 probabilities): chain_sums, kept for the head
-// of every sum and as a switch (SampleArgs::scan = 0).  By default the sums are formed by chain_scan, which
-// reproduces the sequential sums bit for bit from integer prefix sums inside each binade of the running sum
-// (about 0.045 ms for 32000 probabilities).  Everything else (divide, max, exp, normalize, candidate filter,
-// the search in the running sums) is spread over the workgroup.  The probabilities live in LDS.
+// latency of a dependent v_add_f32, measured; 0.11 ms for 32000 probabilities): chain_sums, kept as a switch
+// (SampleArgs::scan = 0).  By default the sums are formed by spec_sums, which reproduces the sequential sums bit
+// for bit from integer prefix sums inside each binade of the running sum.  Everything else (divide, max, exp,
+// normalize, candidate filter, the search in the running sums) is spread over the workgroup.  Up to kSampleMaxVocab
+// probabilities live in LDS; larger vocabularies are worked on where they are, in device memory.
 //
 // sample_topp sorts its whole ProbIndex array, not just the candidates of the call: entries of earlier calls
 // stay behind them and take part (J/Sampler.java:92-97).  The array therefore lives in device memory between
@@ -21,7 +21,7 @@
 
 namespace l2j {
 
-constexpr int kSampleMaxVocab = 36864;  // the probabilities of one call in LDS: 144 KB
+constexpr int kSampleMaxVocab = 36864;  // the most probabilities of one call that fit in LDS: 144 KB
 constexpr unsigned long long kJavaRandMult = 0x5DEECE66DULL, kJavaRandMask = (1ULL << 48) - 1;
 
 struct SamplerState {        // the reference's Sampler object, device resident
@@ -45,7 +45,7 @@ struct SampleArgs {
     const int *sorted_idx;
     DevState *st;            // token loop (null outside it): the sampled token replaces the argmax
     int *out_tokens;         //   that k_finish stored for position st->pos - 1
-    int scan;                // 1: the running sums by windows of equal exponent (chain_scan), 0: one lane adds them all
+    int scan;                // 1: the running sums by spec_sums, 0: one lane adds them all (vocabularies that fit in LDS only)
     float *expbuf;           // not null: k_sample_exp has left exp(x / temperature - max) here (n floats)
 };
 
@@ -162,166 +162,233 @@ __device__ __forceinline__ int first_past(const float *p, const float *ends, int
 // a = floor(e / u), by the fraction e / u - a alone (below, above or equal to 1/2; a tie goes to the even sum, so it
 // depends on the parity of S + a).  Inside a binade the sequential float sum is therefore an integer prefix sum whose
 // steps depend on nothing but the parity of what came before, which composes: a run of terms maps an incoming parity to
-// an increment, (inc0, inc1), and two runs combine as (x0 + y[x0 & 1], x1 + y[(1 + x1) & 1]).  The workgroup scans a tile
-// of terms that way, finds the first term whose sum reaches 2^24 * u (it leaves the binade), adds that one term with a real
-// float addition and starts over behind it in the new binade.  The results are the reference's sums bit for bit.  A sum
-// grows through a binade per doubling, so after a short head that one lane adds (where the sum doubles every few terms)
-// a few rounds per tile remain; an input that leaves binades faster than that falls back to the single lane.
-constexpr int kScanHead = 1024;      // terms added by one lane before the scan starts
-constexpr int kScanPer = 9;          // terms per thread and round; odd: the lanes of a wave then read different LDS banks
-                                     // (measured per sampled 7B token: 7: 1.729, 8: 1.740, 9: 1.730, 13: 1.741 ms)
-constexpr int kScanMaxRounds = 48;
-constexpr int kScanBig = 1 << 25;    // an increment that leaves any binade; sums saturate here
+// an increment, (inc0, inc1), and two runs combine as (x0 + y[x0 & 1], x1 + y[(1 + x1) & 1]).
+//
+// Which binade the sum is in when it reaches a term is not known in advance, but it can be guessed well: every thread
+// takes a contiguous run of terms, a double-precision prefix sum over the threads (any order: it is only a guess) gives
+// the sum at both ends of the run, and when both ends lie in one binade the thread reduces its run to (inc0, inc1) for
+// that binade ("clean"); else ("dirty": a binade boundary inside the run, zero, denormal, infinite or NaN sums) it
+// reduces nothing.  Each wave combines the pairs of its clean threads between one dirty thread and the next (a
+// segmented scan).  Then one wave walks the sequence with the real float sum F in hand: a stretch of clean threads whose
+// guessed binade is the binade of F, and whose increment keeps F inside it, advances F by integer arithmetic, exactly as
+// the additions would have; anything else (a dirty thread, a wrong guess) is added term by term.  A guess is never
+// trusted: it only decides how fast F moves.  Sums of 32000 probabilities have about a dozen dirty threads (one per
+// doubling of the sum), so the walk has some forty steps; in the worst case (every thread dirty) it is the sequential
+// sum.  The results are the reference's sums bit for bit.
+constexpr int kSpecThreads = 1024;
+constexpr int kSpecBig = 1 << 25;        // an increment that leaves any binade; sums saturate here
+constexpr int kSpecIdentity = 254;       // binade code of a stretch of zeros (or of no terms): leaves any sum as it is
+constexpr int kSpecNoStop = 1 << 30;
 
-struct ScanShared {
-    float sum;
-    int i0, cross, send, rounds;
-    int w0[16], w1[16];
+struct SpecShared {
+    int x0[kSpecThreads], x1[kSpecThreads];   // per thread: increments of its stretch up to and including it (even / odd sum before)
+    float fst[kSpecThreads];                  // the sum before a thread's terms, where the walk has stored it
+    unsigned char mm[kSpecThreads];           // binade code of that stretch: 1..253 exponent field, 254 zeros, 0 unusable
+    unsigned char took[kSpecThreads];         // at the first thread of a stretch: the walk advanced over it by integers
+    double wsum[16];
+    unsigned dirty_lo[16], dirty_hi[16];      // per wave: its dirty threads
+    float total;                              // the sum of all terms (when the walk did not stop early)
+    int t_stop;                               // last thread whose starting sum is known (kSpecNoStop: all)
 };
 
-__device__ __forceinline__ int sat_add(int a, int b) { return min(a + b, kScanBig); }
+struct SpecThread {
+    int lo, hi;      // this thread's terms
+    float start;     // the running sum before them
+    bool valid;
+};
 
-// increments of the integer sum for a term e in the binade E, for an even / odd sum before it
-__device__ __forceinline__ void scan_quant(float e, int E, int &inc0, int &inc1)
+__device__ __forceinline__ int sat_add(int a, int b) { return min(a + b, kSpecBig); }
+
+// F advanced by the increments (c0, c1) guessed for the binade with exponent field m; false when the guess does not
+// hold (F is in another binade, or leaves this one on the way): F is then unchanged.
+__device__ __forceinline__ bool spec_apply(float &F, int c0, int c1, int m)
 {
-    const unsigned b = __float_as_uint(e), ef = (b >> 23) & 0xffu, m = b & 0x7fffffu;
-    if (ef == 0xffu) { inc0 = inc1 = kScanBig; return; }
-    const int Ee = ef ? (int)ef - 127 : -126;
-    const unsigned M = ef ? (m | 0x800000u) : m;
-    const int d = E - Ee;
-    if (M == 0u || d >= 25) { inc0 = inc1 = 0; return; }
-    if (d < 0) { inc0 = inc1 = kScanBig; return; }
-    if (d == 0) { inc0 = inc1 = (int)M; return; }
-    const unsigned a = M >> d, rem = M & ((1u << d) - 1u), half = 1u << (d - 1);
-    if (rem < half) { inc0 = inc1 = (int)a; }
-    else if (rem > half) { inc0 = inc1 = (int)a + 1; }
-    else { inc0 = (int)(a + (a & 1u)); inc1 = (int)(a + ((a + 1u) & 1u)); }
+    const unsigned b = __float_as_uint(F);
+    if ((int)(b >> 23) != m) return false;
+    const int S = (int)((b & 0x7fffffu) | 0x800000u);
+    const int Sn = S + ((S & 1) ? c1 : c0);
+    if (Sn >= (1 << 24)) return false;
+    F = __uint_as_float(((unsigned)m << 23) | ((unsigned)Sn & 0x7fffffu));
+    return true;
 }
 
-// S * 2^(E-23) for S < 2^24 (S >= 2^23 unless E = -126)
-__device__ __forceinline__ float scan_value(int S, int E)
+__device__ __forceinline__ int spec_merge(int a, int b)   // binade code of two stretches in a row
 {
-    return __uint_as_float(S >= (1 << 23) ? (((unsigned)(E + 127) << 23) | ((unsigned)S & 0x7fffffu)) : (unsigned)S);
+    return a == kSpecIdentity ? b : (b == kSpecIdentity || a == b) ? a : 0;
 }
 
-// Running sums of p[0..n) in element order (all threads of a 1024-thread workgroup call; p in LDS).  With STORE every
-// p[i] is replaced by the sum up to and including it.  Returns the total.
-template <bool STORE>
-__device__ __forceinline__ float chain_scan(float *p, int n, ScanShared &sh, float *ends)
+__device__ __forceinline__ float spec_uniform(float F)
+{
+    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(F)));
+}
+
+// F + p[lo] + ... + p[hi - 1], one after the other (every lane of the wave the same)
+__device__ __forceinline__ float spec_add_terms(float F, const float *p, int lo, int hi)
+{
+#pragma unroll 8
+    for (int i = lo; i < hi; i++) F = __fadd_rn(F, p[i]);
+    return spec_uniform(F);
+}
+
+// Starting sums of every thread's terms of p[0..n), in element order (all threads of a 1024-thread workgroup call).
+// With `bounded` the walk stops behind the first stretch or thread at whose end the sum exceeds `limit`; later threads
+// come back invalid.  sh.total = the whole sum when it did not stop.
+__device__ __forceinline__ SpecThread spec_sums(const float *p, int n, SpecShared &sh, float limit, bool bounded)
 {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int h = min(n, kScanHead);
-    if (tid == 0) {   // the head: one lane, with the sum after every 32 terms kept
-        float acc;
-        chain_sums<true>(p, h, ends, 0.0f, false, false, &acc);
-        sh.sum = acc; sh.i0 = h; sh.cross = 0x7fffffff; sh.send = 0; sh.rounds = 0;
+    const int T = ((n + kSpecThreads - 1) / kSpecThreads) | 1;   // odd: the lanes of a wave read different LDS banks
+    SpecThread me;
+    me.lo = min(n, tid * T);
+    me.hi = min(n, me.lo + T);
+    // the guess: double-precision sums at both ends of the thread's terms
+    double loc = 0.0;
+#pragma unroll 4
+    for (int i = me.lo; i < me.hi; i++) loc += (double)p[i];
+    double inc = loc;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const double l = __shfl_up(inc, off);
+        if (lane >= off) inc += l;
     }
-    if (STORE) {      // the sums inside each step of 32, one thread per step, from the step's exact starting sum
-        __syncthreads();
-        if (tid * kChainStep < h) {
-            float acc = tid ? ends[tid - 1] : 0.0f;
-            for (int i = tid * kChainStep; i < min(h, (tid + 1) * kChainStep); i++) {
-                acc = __fadd_rn(acc, p[i]);
-                p[i] = acc;
+    if (lane == 63) sh.wsum[wave] = inc;
+    __syncthreads();
+    double before = 0.0;
+    for (int w = 0; w < wave; w++) before += sh.wsum[w];
+    const double p_end = before + inc, p_start = p_end - loc;
+    const unsigned bs = __float_as_uint((float)p_start) >> 23, be = __float_as_uint((float)p_end) >> 23;
+    int m = 0, x0 = 0, x1 = 0;
+    if (me.lo >= me.hi || loc == 0.0) {
+        m = kSpecIdentity;
+    } else if (p_start > 0.0 && bs == be && bs >= 1u && bs <= 253u) {
+        m = (int)bs;
+        const int shift = 23 - ((int)bs - 127);
+#pragma unroll 4
+        for (int i = me.lo; i < me.hi; i++) {
+            // e / u (NaN becomes the large increment too); off a tie the increment is the nearest integer, whatever the parity
+            const float t = fminf(ldexpf(p[i], shift), 33554432.0f);
+            const float fl = floorf(t);
+            int i0 = (int)rintf(t), i1 = i0;
+            if (t - fl == 0.5f) {
+                const int a = (int)fl;
+                i0 = a + (a & 1);
+                i1 = a + (~a & 1);
             }
+            x0 = sat_add(x0, (x0 & 1) ? i1 : i0);
+            x1 = sat_add(x1, ((1 + x1) & 1) ? i1 : i0);
         }
     }
-    while (true) {
-        __syncthreads();
-        const int i0 = sh.i0, rounds = sh.rounds;
-        const float s = sh.sum;
-        if (i0 >= n) break;
-        const unsigned sb = __float_as_uint(s), sef = (sb >> 23) & 0xffu;
-        if (rounds >= kScanMaxRounds || s == 0.0f || sef == 0xffu) {  // the single lane takes the rest
-            __syncthreads();
-            if (tid == 0) {
-                float acc = s;
-                for (int i = i0; i < n; i++) {
-                    acc = __fadd_rn(acc, p[i]);
-                    if (STORE) p[i] = acc;
+    // inclusive scan over the wave, started anew behind every dirty thread
+    const unsigned long long dirty = __ballot(m == 0);
+    int brk = (lane == 0 || ((dirty >> (lane - 1)) & 1ull) || m == 0) ? 1 : 0;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int l0 = __shfl_up(x0, off), l1 = __shfl_up(x1, off), lmb = __shfl_up(m * 2 + brk, off);
+        if (lane >= off && !brk) {
+            const int n0 = sat_add(l0, (l0 & 1) ? x1 : x0), n1 = sat_add(l1, ((1 + l1) & 1) ? x1 : x0);
+            x0 = n0; x1 = n1;
+            m = spec_merge(lmb >> 1, m);
+            brk = lmb & 1;
+        }
+    }
+    sh.x0[tid] = x0;
+    sh.x1[tid] = x1;
+    sh.mm[tid] = (unsigned char)m;
+    if (lane == 0) {
+        sh.dirty_lo[wave] = (unsigned)dirty;
+        sh.dirty_hi[wave] = (unsigned)(dirty >> 32);
+    }
+    if (tid == 0) sh.t_stop = kSpecNoStop;
+    __syncthreads();
+    // the walk
+    if (wave == 0) {
+        float F = 0.0f;
+        bool stopped = false;
+        for (int w = 0; w < kSpecThreads / 64 && !stopped; w++) {
+            unsigned long long mask = ((unsigned long long)sh.dirty_hi[w] << 32) | sh.dirty_lo[w];
+            const int wx0 = sh.x0[w * 64 + lane], wx1 = sh.x1[w * 64 + lane], wmm = sh.mm[w * 64 + lane];
+            int first = 0;   // first thread of the stretch at hand
+            while (true) {
+                const int d = mask ? __ffsll((long long)mask) - 1 : 64;   // the dirty thread behind it
+                if (d > first) {
+                    const int t0 = w * 64 + first, t1 = w * 64 + d - 1;
+                    const int sm = __builtin_amdgcn_readlane(wmm, d - 1);
+                    const float before = F;
+                    bool took = sm == kSpecIdentity;
+                    if (!took && sm != 0)
+                        took = spec_apply(F, __builtin_amdgcn_readlane(wx0, d - 1), __builtin_amdgcn_readlane(wx1, d - 1), sm);
+                    sh.fst[t0] = before;   // (every lane the same value)
+                    sh.took[t0] = took ? 1 : 0;
+                    if (!took) {   // thread by thread, term by term
+                        for (int t = t0; t <= t1; t++) {
+                            sh.fst[t] = F;
+                            F = spec_add_terms(F, p, min(n, t * T), min(n, t * T + T));
+                        }
+                    }
+                    if (bounded && F > limit) {
+                        sh.t_stop = t1;
+                        stopped = true;
+                        break;
+                    }
                 }
-                sh.sum = acc; sh.i0 = n;
-            }
-            continue;
-        }
-        const int E = sef ? (int)sef - 127 : -126;
-        const int S0 = (int)(sef ? ((sb & 0x7fffffu) | 0x800000u) : (sb & 0x7fffffu));
-        const int tile_end = min(n, i0 + 1024 * kScanPer), base = i0 + tid * kScanPer;
-        int inc0[kScanPer], inc1[kScanPer], t0 = 0, t1 = 0;
-#pragma unroll
-        for (int k = 0; k < kScanPer; k++) {
-            inc0[k] = inc1[k] = 0;
-            if (base + k < tile_end) scan_quant(p[base + k], E, inc0[k], inc1[k]);
-            t0 = sat_add(t0, (t0 & 1) ? inc1[k] : inc0[k]);
-            t1 = sat_add(t1, ((1 + t1) & 1) ? inc1[k] : inc0[k]);
-        }
-        // inclusive scan of the compositions over the wave, then over the waves
-        int x0 = t0, x1 = t1;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int l0 = __shfl_up(x0, off), l1 = __shfl_up(x1, off);
-            if (lane >= off) {
-                const int n0 = sat_add(l0, (l0 & 1) ? x1 : x0), n1 = sat_add(l1, ((1 + l1) & 1) ? x1 : x0);
-                x0 = n0; x1 = n1;
-            }
-        }
-        if (lane == 63) { sh.w0[wave] = x0; sh.w1[wave] = x1; }
-        int e0 = __shfl_up(x0, 1), e1 = __shfl_up(x1, 1);   // exclusive within the wave
-        if (lane == 0) { e0 = 0; e1 = 0; }
-        __syncthreads();
-        int q0 = 0, q1 = 0;   // everything before this wave
-        for (int w = 0; w < wave; w++) {
-            const int y0 = sh.w0[w], y1 = sh.w1[w];
-            const int n0 = sat_add(q0, (q0 & 1) ? y1 : y0), n1 = sat_add(q1, ((1 + q1) & 1) ? y1 : y0);
-            q0 = n0; q1 = n1;
-        }
-        const int pre = (S0 & 1) ? q1 : q0;                       // increment up to this wave for the actual parity
-        const int Sw = sat_add(S0, pre);
-        int S = sat_add(Sw, (Sw & 1) ? e1 : e0);                   // the sum before this thread's terms
-        int my_cross = 0x7fffffff, my_pre = 0;
-#pragma unroll
-        for (int k = 0; k < kScanPer; k++) {
-            if (base + k < tile_end && S < (1 << 24)) {
-                const int Sn = sat_add(S, (S & 1) ? inc1[k] : inc0[k]);
-                if (Sn >= (1 << 24)) {
-                    my_cross = base + k; my_pre = S;
-                } else {
-                    if (STORE) p[base + k] = scan_value(Sn, E);
-                    if (base + k == tile_end - 1) sh.send = Sn;
+                if (d == 64) break;
+                const int t = w * 64 + d;
+                sh.fst[t] = F;
+                F = spec_add_terms(F, p, min(n, t * T), min(n, t * T + T));
+                if (bounded && F > limit) {
+                    sh.t_stop = t;
+                    stopped = true;
+                    break;
                 }
-                S = Sn;
+                first = d + 1;
+                mask &= mask - 1ull;
             }
         }
-        if (my_cross != 0x7fffffff) atomicMin(&sh.cross, my_cross);
-        __syncthreads();
-        const int cross = sh.cross;
-        __syncthreads();
-        if (cross != 0x7fffffff) {
-            if (my_cross == cross) {   // the term that leaves the binade: a real addition, then on from the term behind it
-                const float v = __fadd_rn(scan_value(my_pre, E), p[cross]);
-                if (STORE) p[cross] = v;
-                sh.sum = v; sh.i0 = cross + 1; sh.cross = 0x7fffffff; sh.rounds = rounds + 1;
-            }
-        } else if (tid == 0) {
-            sh.sum = scan_value(sh.send, E); sh.i0 = tile_end; sh.rounds = rounds + 1;
-        }
+        sh.total = F;
     }
     __syncthreads();
-    return sh.sum;
+    me.valid = tid <= sh.t_stop;
+    me.start = 0.0f;
+    // a thread of a stretch that was taken whole: the sum before the stretch, advanced by the threads before it
+    const int e0 = __shfl_up(x0, 1), e1 = __shfl_up(x1, 1), em = __shfl_up(m, 1);
+    if (me.valid) {
+        const unsigned long long below = dirty & ((1ull << lane) - 1ull);
+        const int first = below ? 64 - __clzll((long long)below) : 0;
+        const int t0 = wave * 64 + first;
+        if (((dirty >> lane) & 1ull) || !sh.took[t0]) {
+            me.start = sh.fst[tid];
+        } else {
+            float F = sh.fst[t0];
+            if (lane > first && em != kSpecIdentity) spec_apply(F, e0, e1, em);
+            me.start = F;
+        }
+    }
+    return me;
 }
 
-// The first i < m with (above ? p[i] > limit : limit < p[i]) in a non-decreasing p (m if none).  All threads call.
-__device__ __forceinline__ int first_over(const float *p, int m, float limit, bool above, int *slot)
+// The first i < m whose running sum exceeds `limit` (m if none), *sum_at = that running sum.  All threads call; the
+// runs up to that element must be valid.  slot and fslot are LDS words.
+__device__ __forceinline__ int spec_first_over(const float *p, const SpecThread &me, int m, float limit, int *slot, float *fslot,
+                                               float *sum_at)
 {
-    if (threadIdx.x == 0) *slot = m;
+    if (threadIdx.x == 0) { *slot = m; *fslot = 0.0f; }
     __syncthreads();
-    const int per = ((m + blockDim.x - 1) / blockDim.x) | 1, lo = min(m, (int)threadIdx.x * per), hi = min(m, lo + per);
-    for (int i = lo; i < hi; i++) {
-        const float s = p[i];
-        if (above ? s > limit : limit < s) { atomicMin(slot, i); break; }
+    int found = m;
+    float at = 0.0f;
+    if (me.valid) {
+        float acc = me.start;
+        const int hi = min(me.hi, m);
+#pragma unroll 4
+        for (int i = me.lo; i < hi; i++) {   // (no early exit: the loads of an unrolled loop can then go out together)
+            acc = __fadd_rn(acc, p[i]);
+            if (found == m && acc > limit) { found = i; at = acc; }
+        }
+        if (found < m) atomicMin(slot, found);
     }
     __syncthreads();
     const int r = *slot;
+    if (found < m && found == r) *fslot = at;
+    __syncthreads();
+    *sum_at = *fslot;
     __syncthreads();
     return r;
 }
@@ -335,7 +402,16 @@ __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
     float mx = -__builtin_inff();
     int bad = 0;
-    for (int i = tid; i < n; i += nt) {
+    const int n4 = n & ~3;   // (16-byte loads, several in flight: the loop is bound by their latency)
+#pragma unroll 4
+    for (int i = 4 * tid; i < n4; i += 4 * nt) {
+        const float4 x = *reinterpret_cast<const float4 *>(a.logits + i);
+        const float v0 = __fdiv_rn(x.x, a.temperature), v1 = __fdiv_rn(x.y, a.temperature);
+        const float v2 = __fdiv_rn(x.z, a.temperature), v3 = __fdiv_rn(x.w, a.temperature);
+        bad |= (v0 != v0) | (v1 != v1) | (v2 != v2) | (v3 != v3);
+        mx = fmaxf(fmaxf(fmaxf(mx, v0), fmaxf(v1, v2)), v3);
+    }
+    for (int i = n4 + tid; i < n; i += nt) {
         const float v = __fdiv_rn(a.logits[i], a.temperature);
         bad |= v != v;
         mx = fmaxf(mx, v);
@@ -347,44 +423,72 @@ __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
     if (bad && blockIdx.x == 0) atomicOr(&a.ss->nan, 1);
 }
 
+// dst[0..np) in LDS = src[0..n) followed by zeros; src is 16-byte aligned and readable up to n rounded up to 4, np a
+// multiple of 4.  All threads call.
+__device__ __forceinline__ void stage_terms(float *dst, const float *src, int n, int np)
+{
+#pragma unroll 4
+    for (int i = 4 * threadIdx.x; i < np; i += 4 * blockDim.x) {
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (i < n) v = *reinterpret_cast<const float4 *>(src + i);
+        if (i + 1 >= n) v.y = 0.0f;
+        if (i + 2 >= n) v.z = 0.0f;
+        if (i + 3 >= n) v.w = 0.0f;
+        *reinterpret_cast<float4 *>(dst + i) = v;
+    }
+}
+
+// What the sampler's one-workgroup kernels keep in LDS besides the probabilities; the members are used one after the other.
+union SamplerShared {
+    SpecShared spec;
+    float ends[kChainMaxSteps];
+    int cnt[16];
+};
+
 // J/Run.java:645-659 (divide by the temperature, FindMax, ExpSumNormalize), then either J/Sampler.java:33-44
-// (plain) or the candidate filter of J/Sampler.java:85-96.  One workgroup; dynamic LDS: (n rounded up to 32) + 32 floats.
+// (plain) or the candidate filter of J/Sampler.java:85-96.  One workgroup.  IN_LDS: the probabilities live in LDS
+// (dynamic LDS: (n rounded up to 32) + 32 floats, n <= kSampleMaxVocab); else in a.expbuf, where k_sample_exp has
+// left the exponentials (any n).
+template <bool IN_LDS>
 __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
 {
-    extern __shared__ __align__(16) float sp[];
-    __shared__ float ends[kChainMaxSteps];
+    extern __shared__ __align__(16) float lds_sp[];
+    __shared__ SamplerShared u;
     __shared__ float red[16];
-    __shared__ int cnt[1024];
     __shared__ float s_sum, s_coin, s_f;
     __shared__ int s_slot, s_m;
-    __shared__ ScanShared scan;
-    const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
-    const int np = (n + kChainStep - 1) & ~(kChainStep - 1);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = a.n, nt = blockDim.x;
+    float *sp;
+    if constexpr (IN_LDS) sp = lds_sp; else sp = a.expbuf;
 
     int bad = 0;
-    if (a.expbuf) {
-        for (int i = tid; i < np; i += nt) sp[i] = i < n ? a.expbuf[i] : 0.0f;
-    } else {
-        // logits[q] /= temperature; max
-        float mx = -__builtin_inff();
-        for (int i = tid; i < np; i += nt) {
-            float v = 0.0f;
-            if (i < n) {
-                v = __fdiv_rn(a.logits[i], a.temperature);
-                bad |= v != v;
-                mx = fmaxf(mx, v);
+    if constexpr (IN_LDS) {
+        const int np = (n + kChainStep - 1) & ~(kChainStep - 1);
+        if (a.expbuf) {
+            stage_terms(sp, a.expbuf, n, np);
+        } else {
+            // logits[q] /= temperature; max
+            float mx = -__builtin_inff();
+            for (int i = tid; i < np; i += nt) {
+                float v = 0.0f;
+                if (i < n) {
+                    v = __fdiv_rn(a.logits[i], a.temperature);
+                    bad |= v != v;
+                    mx = fmaxf(mx, v);
+                }
+                sp[i] = v;
             }
-            sp[i] = v;
+            mx = block_max(mx, red);
+            // x = (float) Math.exp(x - max)
+            for (int i = tid; i < n; i += nt) sp[i] = (float)exp((double)__fsub_rn(sp[i], mx));
         }
-        mx = block_max(mx, red);
-        // x = (float) Math.exp(x - max)
-        for (int i = tid; i < n; i += nt) sp[i] = (float)exp((double)__fsub_rn(sp[i], mx));
+        __syncthreads();
     }
-    __syncthreads();
     // sum += x, in element order
-    if (a.scan) {
-        const float t = chain_scan<false>(sp, n, scan, ends);
-        if (tid == 0) s_sum = t;
+    const bool scan = !IN_LDS || a.scan;
+    if (scan) {
+        spec_sums(sp, n, u.spec, 0.0f, false);
+        if (tid == 0) s_sum = u.spec.total;
     } else if (tid == 0) {
         float t;
         chain_sums<false>(sp, n, nullptr, 0.0f, false, false, &t);
@@ -393,6 +497,7 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
     __syncthreads();
     const float sum = s_sum;
     // if (sum != 0) x /= sum; the probabilities replace the logits
+#pragma unroll 4
     for (int i = tid; i < n; i += nt) {
         float v = sp[i];
         if (sum != 0.0f) v = __fdiv_rn(v, sum);
@@ -409,19 +514,19 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
             float r = a.coin;
             if (r < 0.0f) r = java_next_float(&a.ss->rng);
             s_coin = r;
-            if (!a.scan) {
+            if (!scan) {
                 float t;
-                s_m = chain_sums<true>(sp, n, ends, r, false, true, &t);
+                s_m = chain_sums<true>(sp, n, u.ends, r, false, true, &t);
             }
         }
         __syncthreads();
         int pick;
-        if (a.scan) {
-            chain_scan<true>(sp, n, scan, ends);   // the probabilities are in a.logits by now: sp becomes the cdf
-            pick = first_over(sp, n, s_coin, false, &s_slot);
+        float at;
+        if (scan) {
+            const SpecThread me = spec_sums(sp, n, u.spec, s_coin, true);
+            pick = spec_first_over(sp, me, n, s_coin, &s_slot, &s_f, &at);
         } else {
-            float at;
-            pick = first_past(sp, ends, s_m, n, s_coin, false, &s_slot, &s_f, &at);
+            pick = first_past(sp, u.ends, s_m, n, s_coin, false, &s_slot, &s_f, &at);
         }
         if (pick >= n) pick = n - 1;
         if (tid == 0) {
@@ -436,40 +541,47 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
 
     // J/Sampler.java:85-96: candidates in index order into the front of the ProbIndex array
     const float cutoff = __fdiv_rn(__fsub_rn(1.0f, a.topp), (float)(n - 1));
-    // (an odd number of elements per thread: the lanes of a wave then read different LDS banks)
-    const int per = ((n + nt - 1) / nt) | 1, lo = min(n, tid * per), hi = min(n, lo + per);
+    // every wave takes a contiguous part of the indices and goes through it 64 at a time, so that the candidates of a
+    // step go out to consecutive addresses
+    const int per_wave = (((n + nt - 1) / nt) * 64 + 63) & ~63, w_lo = min(n, wave * per_wave), w_hi = min(n, w_lo + per_wave);
     int c = 0;
-    for (int i = lo; i < hi; i++) c += sp[i] >= cutoff;
-    cnt[tid] = c;
+#pragma unroll 4
+    for (int i = w_lo + lane; i < w_hi; i += 64) c += sp[i] >= cutoff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+    if (lane == 0) u.cnt[wave] = c;
     __syncthreads();
-    for (int off = 1; off < nt; off <<= 1) {   // inclusive scan of the per-thread counts
-        const int v = tid >= off ? cnt[tid - off] : 0;
-        __syncthreads();
-        cnt[tid] += v;
-        __syncthreads();
+    int at = 0, total = 0;
+    for (int w = 0; w < nt / 64; w++) {
+        const int cw = u.cnt[w];
+        if (w < wave) at += cw;
+        total += cw;
     }
-    int at = cnt[tid] - c;
-    for (int i = lo; i < hi; i++) {
-        const float v = sp[i];
-        if (v >= cutoff) {
-            a.cand_prob[at] = v;
-            a.cand_idx[at] = i;
-            at++;
+    if (tid == 0) a.ss->n0 = total;
+    for (int i0 = w_lo; i0 < w_hi; i0 += 64) {
+        const int i = i0 + lane;
+        const float v = i < w_hi ? sp[i] : 0.0f;
+        const bool is = i < w_hi && v >= cutoff;
+        const unsigned long long m = __ballot(is);
+        if (is) {
+            const int r = at + __popcll(m & ((1ull << lane) - 1ull));
+            a.cand_prob[r] = v;
+            a.cand_idx[r] = i;
         }
+        at += __popcll(m);
     }
-    if (tid == nt - 1) a.ss->n0 = cnt[tid];
 }
 
-// J/Sampler.java:99-119 on the sorted ProbIndex array.  One workgroup; dynamic LDS: (n rounded up to 32) + 32 floats,
-// n0 <= n.
+// J/Sampler.java:99-119 on the sorted ProbIndex array.  One workgroup.  IN_LDS: the candidates are copied to LDS first
+// (dynamic LDS as above, n0 <= n <= kSampleMaxVocab); else they are read where they are.
+template <bool IN_LDS>
 __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
 {
-    extern __shared__ __align__(16) float sp[];
-    __shared__ float ends[kChainMaxSteps];
+    extern __shared__ __align__(16) float lds_sp[];
+    __shared__ SamplerShared u;
     __shared__ float s_cum, s_r, s_f;
     __shared__ int s_slot, s_m;
-    __shared__ ScanShared scan;
-    const int tid = threadIdx.x, nt = blockDim.x;
+    const int tid = threadIdx.x;
     const int n0 = a.ss->n0;
     if (n0 <= 0) {   // no probability reaches the cutoff (NaNs, or topp near 0 on a flat distribution): the reference
         if (tid == 0) {   // indexes probIndex[-1] and throws; the host reports the call as failed
@@ -478,22 +590,33 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
         }
         return;
     }
-    const int np = (n0 + kChainStep - 1) & ~(kChainStep - 1);
-    for (int i = tid; i < np; i += nt) sp[i] = i < n0 ? a.sorted_prob[i] : 0.0f;
-    __syncthreads();
-    if (a.scan) {
-        // sp becomes the running sums; cumulative_prob is the first of them above topp (else the last), and the cdf of
-        // the pick below runs over the same terms from zero again: the same sums
-        chain_scan<true>(sp, n0, scan, ends);
-        int last = first_over(sp, n0, a.topp, true, &s_slot);
-        if (last >= n0) last = n0 - 1;
+    const float *sp;
+    if constexpr (IN_LDS) {
+        const int np = (n0 + kChainStep - 1) & ~(kChainStep - 1);
+        stage_terms(lds_sp, a.sorted_prob, n0, np);
+        __syncthreads();
+        sp = lds_sp;
+    } else {
+        sp = a.sorted_prob;
+    }
+    if (!IN_LDS || a.scan) {
+        // cumulative_prob is the first running sum above topp (else the last), and the cdf of the pick below runs over
+        // the same terms from zero again: the same sums
+        const SpecThread me = spec_sums(sp, n0, u.spec, a.topp, true);
+        float cum;
+        int last = spec_first_over(sp, me, n0, a.topp, &s_slot, &s_f, &cum);
+        if (last >= n0) {   // never exceeded: all candidates, cumulative_prob = their sum
+            last = n0 - 1;
+            cum = u.spec.total;
+        }
         if (tid == 0) {
             float coin = a.coin;
             if (coin < 0.0f) coin = java_next_float(&a.ss->rng);
-            s_r = __fmul_rn(coin, sp[last]);
+            s_r = __fmul_rn(coin, cum);
         }
         __syncthreads();
-        int pick = first_over(sp, last + 1, s_r, false, &s_slot);
+        float at;
+        int pick = spec_first_over(sp, me, last + 1, s_r, &s_slot, &s_f, &at);
         if (pick > last) pick = last;
         if (tid == 0) {
             const int token = a.sorted_idx[pick];
@@ -508,13 +631,13 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
     // cumulative_prob += prob until it exceeds topp
     if (tid == 0) {
         float t;
-        s_m = chain_sums<true>(sp, n0, ends, a.topp, true, true, &t);
+        s_m = chain_sums<true>(sp, n0, u.ends, a.topp, true, true, &t);
         s_cum = t;
     }
     __syncthreads();
     const int steps = s_m;
     float cum;
-    int last = first_past(sp, ends, steps, n0, a.topp, true, &s_slot, &s_f, &cum);
+    int last = first_past(sp, u.ends, steps, n0, a.topp, true, &s_slot, &s_f, &cum);
     if (last >= n0) {   // never exceeded: all candidates, cumulative_prob = their sum
         last = n0 - 1;
         cum = s_cum;
@@ -527,7 +650,7 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
     __syncthreads();
     // the first i <= last_idx with r < cdf(i), else last_idx
     float at;
-    int pick = first_past(sp, ends, min(steps, last / kChainStep + 1), last + 1, s_r, false, &s_slot, &s_f, &at);
+    int pick = first_past(sp, u.ends, min(steps, last / kChainStep + 1), last + 1, s_r, false, &s_slot, &s_f, &at);
     if (pick > last) pick = last;
     if (tid == 0) {
         const int token = a.sorted_idx[pick];
@@ -539,26 +662,34 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
     }
 }
 
-// The running sums of x[0..n) by the sampler's routine (scan: chain_scan, else one lane).  One workgroup; dynamic LDS as above.
+// The running sums of x[0..n) by the sampler's routine (scan_on: spec_sums, else one lane).  One workgroup.  IN_LDS: the
+// terms are staged in LDS (dynamic LDS as above, n <= kSampleMaxVocab); else they are read where they are (any n).
+template <bool IN_LDS>
 __global__ void __launch_bounds__(1024) k_running_sums(float *x, int n, int scan_on)
 {
-    extern __shared__ __align__(16) float sp[];
-    __shared__ float ends[kChainMaxSteps];
-    __shared__ ScanShared scan;
-    const int np = ((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep;
-    for (int i = threadIdx.x; i < np; i += blockDim.x) sp[i] = i < n ? x[i] : 0.0f;
-    __syncthreads();
-    if (scan_on) {
-        chain_scan<true>(sp, n, scan, ends);
+    extern __shared__ __align__(16) float lds_sp[];
+    __shared__ SamplerShared u;
+    const float *sp = x;
+    if constexpr (IN_LDS) {
+        const int np = ((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep;
+        for (int i = threadIdx.x; i < np; i += blockDim.x) lds_sp[i] = i < n ? x[i] : 0.0f;
+        __syncthreads();
+        sp = lds_sp;
+    }
+    if (!IN_LDS || scan_on) {
+        const SpecThread me = spec_sums(sp, n, u.spec, 0.0f, false);
+        float acc = me.start;
+        for (int i = me.lo; i < me.hi; i++) {
+            acc = __fadd_rn(acc, sp[i]);
+            x[i] = acc;
+        }
     } else if (threadIdx.x == 0) {
         float acc = 0.0f;
         for (int i = 0; i < n; i++) {
             acc = __fadd_rn(acc, sp[i]);
-            sp[i] = acc;
+            x[i] = acc;
         }
     }
-    __syncthreads();
-    for (int i = threadIdx.x; i < n; i += blockDim.x) x[i] = sp[i];
 }
 
 // J/Sampler.java:46-57 on an array given by the caller: first index of the strict maximum.  One workgroup.

@@ -98,8 +98,24 @@ def running_sum_cases():
     yield "leading zeros", np.concatenate([np.zeros(5000), rng.random(5000)])
     yield "every term leaves the binade", np.ldexp(1.0, np.arange(-100, 100))
     yield "a large term late", np.concatenate([rng.random(20000) * 1e-3, [1e6], rng.random(5000)])
-    for m in (1, 2, 31, 32, 33, 1023, 1024, 1025, 1024 + 8192, 1024 + 8193, 36864):
+    for m in (1, 2, 31, 32, 33, 63, 64, 65, 1023, 1024, 1025, 3071, 3072, 3073, 1024 + 8192, 1024 + 8193, 36863, 36864):
         yield "n = %d" % m, rng.random(m)
+    # sums that stay next to a power of two for thousands of terms, where a guessed binade is easily wrong
+    for k in range(3):
+        x = rng.standard_normal(n) * (1 + 3 * k)
+        x[rng.integers(0, n)] += 8 + 4 * k
+        e = np.exp((x - x.max()).astype(np.float32).astype(np.float64)).astype(np.float32)
+        pr = e / np.cumsum(e, dtype=np.float32)[-1]
+        yield "peaked exponentials %d" % k, e
+        yield "peaked probabilities %d" % k, pr
+        yield "peaked probabilities, sorted descending %d" % k, np.sort(pr)[::-1]
+    yield "one, then tiny terms", np.concatenate([[1.0], np.full(n - 1, 1e-9)])
+    yield "just below one, then terms of 3e-8", np.concatenate([rng.random(500) * 1e-3, [0.75], np.full(31000, 3e-8)])
+    yield "an infinity", np.concatenate([rng.random(700), [np.inf], rng.random(700)])
+    # more terms than fit in LDS: the sums are formed in device memory
+    for m in (36865, 50257, 131072, 200003):
+        yield "n = %d" % m, rng.random(m)
+    yield "n = 151936, peaked", np.exp(rng.standard_normal(151936) * 5 - 12)
 
 
 @pytest.mark.parametrize("scan", ["1", "0"])
@@ -108,8 +124,9 @@ def test_running_sums_are_the_sequential_float32_sums(orc, monkeypatch, scan):
     monkeypatch.setenv("L2J_SAMPLER_SCAN", scan)
     g = small_transformer(64)
     for name, terms in running_sum_cases():
-        terms = np.asarray(terms, dtype=np.float32)
-        want = np.cumsum(terms, dtype=np.float32)
+        with np.errstate(over="ignore", invalid="ignore"):
+            terms = np.asarray(terms, dtype=np.float32)
+            want = np.cumsum(terms, dtype=np.float32)
         got = g.running_sums(terms)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (name, int(np.argmax(got != want)))
 
@@ -161,10 +178,18 @@ def test_largest_vocabulary_the_sampler_takes(orc):
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
-def test_sampler_rejects_a_vocabulary_that_does_not_fit(orc):
-    g = small_transformer(40000)
-    with pytest.raises(L2JError):
-        g.sampler_seed(1)
+@pytest.mark.parametrize("vocab", [36865, 50257, 131072])
+def test_vocabularies_beyond_the_lds(orc, vocab):
+    """Above 36864 entries the probabilities stay in device memory; the tokens are still the reference's."""
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(vocab)
+    g.sampler_seed(11)
+    o = orc.Sampler(11, vocab)
+    for kind, topp in (("flat", 0.9), ("peaked", 0.95), ("mid", 1.0), ("peaked", 0.5), ("flat", 1.0), ("mid", 0.99)):
+        lg = logits_of(rng, vocab, kind)
+        want, probs = o.step(lg, 0.9, topp)
+        assert g.sample(0.9, topp, logits=lg) == want, (kind, topp)
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
 @pytest.mark.parametrize("shape,steps,t,topp", [
