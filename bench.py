@@ -23,6 +23,8 @@ WORKLOADS = {
     # name: (dim, hidden, layers, heads, kv_heads, vocab, seq_len, shared), seed, prompt ids
     "llama2-7b-shape": ((4096, 11008, 32, 32, 32, 32000, 4096, 0), 103, 32),
     "llama2-13b-shape": ((5120, 13824, 40, 40, 40, 32000, 4096, 0), 105, 32),
+    # grouped-query attention (8 kv heads), 72 GB of weights and scales: one GPU's HBM holds it whole
+    "llama2-70b-shape": ((8192, 28672, 80, 64, 8, 32000, 4096, 0), 107, 32),
     # 3584 forced prompt ids, then 512 generated: the timed region is positions 3584..4095 only
     "llama2-7b-long-context": ((4096, 11008, 32, 32, 32, 32000, 4096, 0), 104, 3584),
     "stories110m-shape": ((768, 2048, 12, 12, 12, 32000, 1024, 1), 102, 16),

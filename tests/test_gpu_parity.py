@@ -737,6 +737,20 @@ def test_config4_long_context_full_size(orc):
     m.close(); g.close()
 
 
+def test_llama2_70b_width_grouped_query(orc):
+    # the 70B geometry (dim 8192, hidden 28672, 64 heads sharing 8 kv heads) at 4 layers: rows of two and seven steps,
+    # 32 prompt ids + the first 64 greedy tokens, logits at all 96 steps
+    run_config(orc, "70B width", (8192, 28672, 4, 64, 8, 32000, 4096, 0), seed=106, n_prompt=32, n_steps=32 + 64,
+               n_logit_steps=32 + 64)
+
+
+def test_llama2_70b_shape_full_depth(orc):
+    # all 80 layers (72 GB of weights on the one GPU, the same again on the host for the oracle, which runs at
+    # ~0.7 tok/s on 16 cores): 4 prompt ids + 12 greedy tokens, logits at all 16 steps
+    run_config(orc, "70B", (8192, 28672, 80, 64, 8, 32000, 4096, 0), seed=107, n_prompt=4, n_steps=4 + 12,
+               n_logit_steps=4 + 12)
+
+
 def test_config5_llama2_13b_shape(orc):
     # the reference's int offsets overflow at this size (J/TransformerWeights.java:89); 64-bit here.
     # 32 prompt ids + the first 64 greedy tokens, logits at all 96 steps (the oracle runs at ~3.7 tok/s on 16 cores)
