@@ -135,6 +135,19 @@ int l2j_forward_taps(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_
 int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps,
                       int32_t *out_tokens, int32_t *n_out, double *seconds);
 
+/* Sixteen sequences at once, every weight read once per step for all of them (the reference has no counterpart:
+ * "parallel processing of multiple queries" is on its wish-list, README.md:347).  Every sequence runs the token loop
+ * of l2j_decode_greedy (BOS first, its own prompt ids forced, first-maximum argmax afterwards) for exactly `steps`
+ * positions; a sequence that emits token 1 keeps running and the caller cuts it there.  prompts: 16 rows of
+ * prompt_stride ids, n_prompt[b] of them used; out_tokens: 16 rows of `steps` ids.  The matrix products run on the
+ * matrix cores in fp32 (fp32 activations and sums as in K/MatMul.java:117-151; sums are formed in another order
+ * than in the single-sequence path, so logits agree to rounding, not bit for bit).  The call allocates its own
+ * activation buffers and a KV cache of 16 x steps rows per layer and frees them when it returns; the context's
+ * cache is not touched.  Needs dim and hidden_dim in whole groups of 256 and head_size 64, 128 or 256.
+ * *seconds (may be NULL): GPU time from the end of the first step to the end of the last. */
+int l2j_decode_greedy_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t prompt_stride,
+                            int32_t steps, int32_t *out_tokens, double *seconds);
+
 /* ---- sampling on the device: J/Sampler.java and the sampling branch of J/Run.java:643-665 ----
  * The context holds one sampler = the reference's Sampler object: a java.util.Random and the ProbIndex
  * array that sample_topp sorts whole, so that entries of earlier calls take part in later ones
@@ -218,6 +231,14 @@ int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
  * GPU's array, so calls that overlapped would race: the library runs them one after the other.  The array keeps the last
  * call's contents; a call reads none of them (it only reads the n terms it has just copied in). */
 int l2j_running_sums_noalloc(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
+/* Measurement and test of the matrix-core kernel for several sequences at once (the reference has none: "parallel
+ * processing of multiple queries" is on its wish-list, README.md:347): y[b][r] = sum_k dequant(W[r][k]) * x[b][k] for
+ * sixteen activation vectors x (16 x K floats) against one layer's matrix of a quantized matrix tensor (L2J_WQ..L2J_W3;
+ * K a multiple of 256), in the arithmetic of K/MatMul.java:117-151 (fp32 products and sums, group scale and offset).
+ * y: 16 x rows floats.  groups_per_slice: groups of 256 codes per slice of K (a workgroup stages that slice of the
+ * activations in LDS).  *mean_us (may be NULL): mean time of `rounds` launches of the product kernel. */
+int l2j_batch_matmul(l2j_ctx *ctx, int tensor, int layer, const float *x, float *y, int32_t groups_per_slice,
+                     int32_t rounds, double *mean_us);
 /* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
  * and returns the mean kernel time from the start/stop events of each launch.  L2J_K_TOKEN is the kernel the forward pass runs: every phase of
  * every layer and the classifier in one launch.  The other classes launch one phase of it as a kernel of its

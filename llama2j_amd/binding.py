@@ -114,6 +114,8 @@ def _signatures():
         "l2j_sync": (C.c_int, [vp]),
         "l2j_time_kernel": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
+        "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
+        "l2j_batch_matmul": (C.c_int, [vp, C.c_int, C.c_int, fp, fp, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
         "l2j_bytes_per_token": (C.c_uint64, [cfgp, C.c_int32]),
         "l2j_quant_nbytes": (C.c_uint64, [C.c_uint64]),
         "l2j_quant_encode": (C.c_int, [fp, C.c_uint64, u8p]),
@@ -417,6 +419,31 @@ class Transformer:
         out = np.empty_like(terms)
         self._check(lib().l2j_running_sums_noalloc(self._h, _fp(terms), terms.size, _fp(out)))
         return out
+
+    def decode_greedy_batch(self, prompts, steps):
+        """Sixteen greedy token loops at once (l2j_decode_greedy_batch).  prompts: up to sixteen id sequences (missing
+        ones run without a prompt); returns (tokens of shape (16, steps), seconds after the first step)."""
+        assert len(prompts) <= 16
+        stride = max([len(p) for p in prompts] + [1])
+        ids = np.zeros((16, stride), dtype=np.int32)
+        n = np.zeros(16, dtype=np.int32)
+        for b, p in enumerate(prompts):
+            ids[b, :len(p)] = p
+            n[b] = len(p)
+        out = np.zeros((16, steps), dtype=np.int32)
+        sec = C.c_double(0.0)
+        self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), stride, steps, _i32(out), C.byref(sec)))
+        return out, sec.value
+
+    def batch_matmul(self, tensor, layer, x, rows, groups_per_slice=2, rounds=1):
+        """y[b] = W x[b] for sixteen activation vectors against one layer's matrix of a quantized tensor, by the
+        matrix-core kernel of the batched path; returns (y of shape (16, rows), mean microseconds per launch)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        assert x.ndim == 2 and x.shape[0] == 16
+        y = np.empty((16, rows), dtype=np.float32)
+        us = C.c_double(0.0)
+        self._check(lib().l2j_batch_matmul(self._h, int(tensor), layer, _fp(x), _fp(y), groups_per_slice, rounds, C.byref(us)))
+        return y, us.value
 
     def running_sums(self, terms):
         """The float32 sums terms[0] + ... + terms[i] formed one addition after the other (the order of the reference's

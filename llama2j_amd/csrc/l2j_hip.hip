@@ -4,6 +4,7 @@
 #include "kernels.hpp"
 #include "phase_kernels.hpp"
 #include "sampler_kernels.hpp"
+#include "batch_kernels.hpp"
 
 #include <hip/hip_ext.h>
 
@@ -1522,6 +1523,241 @@ int l2j_running_sums_noalloc(l2j_ctx *c, const float *terms, int32_t n, float *s
         HIPCHK(hipMemcpyAsync(sums, d, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, c->stream));
         HIPCHK(hipStreamSynchronize(c->stream));
         return L2J_OK;
+    }());
+}
+
+// rows and row length of one layer's matrix of a quantized matrix tensor (false: not one)
+static bool matrix_shape(const l2j_config &cf, int tensor, int *rows, int *K)
+{
+    const int kvd = cf.dim / cf.n_heads * cf.n_kv_heads;
+    switch (tensor) {
+    case L2J_WQ: case L2J_WO: *rows = cf.dim; *K = cf.dim; return true;
+    case L2J_WK: case L2J_WV: *rows = kvd; *K = cf.dim; return true;
+    case L2J_W1: case L2J_W3: *rows = cf.hidden_dim; *K = cf.dim; return true;
+    case L2J_W2: *rows = cf.dim; *K = cf.hidden_dim; return true;
+    default: return false;
+    }
+}
+
+int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y, int32_t groups_per_slice, int32_t rounds,
+                     double *mean_us)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !x || !y) return fail(L2J_E_ARG, "null argument");
+        int rows = 0, K = 0;
+        if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
+        if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        if (K % 256 || rows % 16) return fail(L2J_E_SIZE, "the batched matrix product needs rows of whole groups (K % 256 == 0) and rows % 16 == 0");
+        const QTensor &t = c->qt[tensor];
+        if (t.groups_loaded != t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
+        const int ngroups = K / 256, gps = std::max(1, std::min(ngroups, (int)groups_per_slice));
+        const int slices = (ngroups + gps - 1) / gps;
+        const size_t lds = (size_t)kBatch * (gps * 256 + kXPad) * sizeof(float);
+        if (lds > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        float *dx = nullptr, *dsx = nullptr, *dpart = nullptr, *dy = nullptr;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        auto release = [&]() {
+            (void)hipFree(dx); (void)hipFree(dsx); (void)hipFree(dpart); (void)hipFree(dy);
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+        };
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&dx), (size_t)kBatch * K * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dsx), (size_t)kBatch * ngroups * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dpart), (size_t)slices * kBatch * rows * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
+        if (e == hipSuccess) e = hipEventCreate(&e0);
+        if (e == hipSuccess) e = hipEventCreate(&e1);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        if (e == hipSuccess) {
+            BGemm a{};
+            a.m = qmat(c, tensor, (uint64_t)layer * rows * K);
+            a.rows = rows; a.K = K; a.x = dx; a.sx = dsx; a.part = dpart; a.gps = gps;
+            hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * ngroups + 3) / 4), dim3(256), 0, c->stream, dx, dsx, K);
+            const dim3 grid((rows + kBgRowsPerWG - 1) / kBgRowsPerWG, slices);
+            const int n = std::max(1, (int)rounds);
+            hipLaunchKernelGGL(k_bgemm, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
+            (void)hipEventRecord(e0, c->stream);
+            for (int i = 0; i < n; i++) hipLaunchKernelGGL(k_bgemm, grid, dim3(kBgThreads), lds, c->stream, a);
+            (void)hipEventRecord(e1, c->stream);
+            hipLaunchKernelGGL(k_breduce, dim3(256), dim3(256), 0, c->stream, dpart, dy, rows, slices);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipMemcpyAsync(y, dy, (size_t)kBatch * rows * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+            float ms = 0.0f;
+            if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+            if (mean_us) *mean_us = (double)ms * 1e3 / n;
+        }
+        release();
+        if (e != hipSuccess) return fail(L2J_E_HIP, std::string("batch matmul: ") + hipGetErrorString(e));
+        return L2J_OK;
+    }());
+}
+
+// ---- several sequences at once ----------------------------------------------------------------------------------
+
+namespace {
+
+struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
+    float *x = nullptr, *xn = nullptr, *sx = nullptr, *q = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
+    float *part[3] = {nullptr, nullptr, nullptr};
+    float *kc = nullptr, *vc = nullptr;
+    BatchState *st = nullptr;
+    int *prompts = nullptr, *out = nullptr;
+    unsigned *done = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    void release()
+    {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+        void *ps[] = {x, xn, sx, q, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
+        for (void *p : ps) (void)hipFree(p);
+    }
+};
+
+constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
+
+int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
+size_t batch_lds() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }
+
+void launch_bgemm(l2j_ctx *c, int tensor, int layer, const float *x, const float *sx, float *part)
+{
+    int rows = 0, K = 0;
+    matrix_shape(c->cfg, tensor, &rows, &K);
+    BGemm a{};
+    a.m = qmat(c, tensor, (uint64_t)layer * rows * K);
+    a.rows = rows; a.K = K; a.x = x; a.sx = sx; a.part = part; a.gps = kBatchGps;
+    hipLaunchKernelGGL(k_bgemm, dim3((rows + kBgRowsPerWG - 1) / kBgRowsPerWG, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
+}
+
+// One position of all sequences: embedding, the layers, the classifier, the next tokens.
+void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
+{
+    const l2j_config &cf = c->cfg;
+    const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim;
+    const int sd = batch_slices(dim), sh = batch_slices(hidden);
+    hipStream_t s = c->stream;
+    hipLaunchKernelGGL(k_bembed, dim3(kBatch), dim3(256), 0, s, c->emb, b.st, b.x, dim);
+    for (int l = 0; l < L; l++) {
+        hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)l * dim, b.xn, b.sx, dim);
+        launch_bgemm(c, L2J_WQ, l, b.xn, b.sx, b.part[0]);
+        launch_bgemm(c, L2J_WK, l, b.xn, b.sx, b.part[1]);
+        launch_bgemm(c, L2J_WV, l, b.xn, b.sx, b.part[2]);
+        BQkv e{};
+        e.pq = b.part[0]; e.pk = b.part[1]; e.pv = b.part[2]; e.sq = sd; e.sk = sd;
+        e.dim = dim; e.kv_dim = kvd; e.head_size = hs; e.rope = c->rope; e.st = b.st; e.q = b.q;
+        e.kc = b.kc + (size_t)l * max_pos * kvd; e.vc = b.vc + (size_t)l * max_pos * kvd;
+        e.seq_stride = (long)L * max_pos;
+        hipLaunchKernelGGL(k_bepi_qkv, dim3(((dim + 2 * kvd) / 2 + 255) / 256, kBatch), dim3(256), 0, s, e);
+        BAttn t{};
+        t.q = b.q; t.kc = e.kc; t.vc = e.vc; t.seq_stride = e.seq_stride; t.out = b.xb; t.st = b.st;
+        t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
+        t.sqrt_hs = sqrtf((float)hs);
+        const dim3 ag(cf.n_heads, kBatch);
+        if (hs == 64) hipLaunchKernelGGL(k_battn<16>, ag, dim3(256), 0, s, t);
+        else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
+        else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
+        hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * (dim / 256) + 3) / 4), dim3(256), 0, s, b.xb, b.sx, dim);
+        launch_bgemm(c, L2J_WO, l, b.xb, b.sx, b.part[0]);
+        hipLaunchKernelGGL(k_bepi_res, dim3((kBatch * dim + 255) / 256), dim3(256), 0, s, b.part[0], sd, b.x, dim);
+        hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, b.sx, dim);
+        launch_bgemm(c, L2J_W1, l, b.xn, b.sx, b.part[0]);
+        launch_bgemm(c, L2J_W3, l, b.xn, b.sx, b.part[1]);
+        hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, kBatch), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
+                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb, b.sx);
+        launch_bgemm(c, L2J_W2, l, b.hb, b.sx, b.part[0]);
+        hipLaunchKernelGGL(k_bepi_res, dim3((kBatch * dim + 255) / 256), dim3(256), 0, s, b.part[0], sh, b.x, dim);
+    }
+    hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)2 * L * dim, b.xn, b.sx, dim);
+    BGemmF32 g{};
+    g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
+    hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds(), s, g);
+    BNext n{};
+    n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
+    n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
+    hipLaunchKernelGGL(k_bnext, dim3(kBatch), dim3(1024), 0, s, n, b.done);
+}
+
+}  // namespace
+
+int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t prompt_stride, int32_t steps,
+                            int32_t *out_tokens, double *seconds)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !n_prompt || !out_tokens || (prompt_stride > 0 && !prompts) || prompt_stride < 0) return fail(L2J_E_ARG, "bad argument");
+        if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
+        const l2j_config &cf = c->cfg;
+        const int hs = c->head_size;
+        if (cf.dim % 256 || cf.hidden_dim % 256 || c->kv_dim % 16 || cf.vocab_size % 16 || (hs != 64 && hs != 128 && hs != 256))
+            return fail(L2J_E_SIZE, "batched decode needs dim and hidden_dim in whole groups of 256, kv_dim and vocab_size multiples of 16, "
+                                    "head_size 64, 128 or 256");
+        if (steps <= 0 || steps > cf.seq_len) return fail(L2J_E_ARG, "steps must be 1..seq_len");
+        for (int b = 0; b < kBatch; b++) {
+            if (n_prompt[b] < 0 || n_prompt[b] > prompt_stride) return fail(L2J_E_ARG, "n_prompt out of range");
+            for (int i = 0; i < n_prompt[b]; i++)
+                if (prompts[(size_t)b * prompt_stride + i] < 0 || prompts[(size_t)b * prompt_stride + i] >= cf.vocab_size)
+                    return fail(L2J_E_ARG, "prompt id out of range");
+        }
+        HIPCHK(hipSetDevice(cf.device));
+        const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, kvd = c->kv_dim, vocab = cf.vocab_size;
+        const int sd = batch_slices(dim), sh = batch_slices(hidden);
+        const size_t part_floats = (size_t)kBatch * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
+        const size_t cache_floats = (size_t)kBatch * L * steps * kvd;
+        const int pstride = std::max(1, (int)prompt_stride);
+        BatchBufs b;
+        auto done = [&](int rc) { b.release(); return rc; };
+        hipError_t e = hipSuccess;
+        auto alloc = [&](auto **p, size_t n) {
+            if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
+        };
+        alloc(&b.x, (size_t)kBatch * dim); alloc(&b.xn, (size_t)kBatch * std::max(dim, hidden));
+        alloc(&b.sx, (size_t)kBatch * (std::max(dim, hidden) / 256)); alloc(&b.q, (size_t)kBatch * dim);
+        alloc(&b.xb, (size_t)kBatch * dim); alloc(&b.hb, (size_t)kBatch * hidden); alloc(&b.logits, (size_t)kBatch * vocab);
+        for (int i = 0; i < 3; i++) alloc(&b.part[i], part_floats);
+        alloc(&b.kc, cache_floats); alloc(&b.vc, cache_floats);
+        alloc(&b.st, 1); alloc(&b.prompts, (size_t)kBatch * pstride); alloc(&b.out, (size_t)kBatch * steps); alloc(&b.done, 1);
+        if (e == hipSuccess) e = hipEventCreate(&b.e0);
+        if (e == hipSuccess) e = hipEventCreate(&b.e1);
+        if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: ") + hipGetErrorString(e)));
+        BatchState h{};
+        h.pos = 0;
+        for (int i = 0; i < kBatch; i++) { h.token[i] = 1; h.n_prompt[i] = n_prompt[i]; }   // BOS first (J/Run.java:612)
+        if (hipMemcpyAsync(b.st, &h, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+            (prompt_stride > 0 && hipMemcpyAsync(b.prompts, prompts, (size_t)kBatch * prompt_stride * sizeof(int), hipMemcpyHostToDevice, c->stream) != hipSuccess) ||
+            hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
+            hipStreamSynchronize(c->stream) != hipSuccess)
+            return done(fail(L2J_E_HIP, "batched decode: set-up failed"));
+        // one position as a graph: every kernel reads the position and the tokens from device memory
+        e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            launch_batch_step(c, b, steps, pstride);
+            const hipError_t le = hipGetLastError();
+            e = hipStreamEndCapture(c->stream, &b.graph);
+            if (e == hipSuccess) e = le;
+        }
+        if (e == hipSuccess) e = hipGraphInstantiate(&b.exec, b.graph, nullptr, nullptr, 0);
+        if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: graph capture: ") + hipGetErrorString(e)));
+        for (int pos = 0; pos < steps && e == hipSuccess; pos++) {
+            e = hipGraphLaunch(b.exec, c->stream);
+            if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
+        }
+        if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(out_tokens, b.out, (size_t)kBatch * steps * sizeof(int), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        float ms = 0.0f;
+        if (e == hipSuccess && steps > 1) e = hipEventElapsedTime(&ms, b.e0, b.e1);
+        if (seconds) *seconds = (double)ms * 1e-3;
+        if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: ") + hipGetErrorString(e)));
+        return done(L2J_OK);
     }());
 }
 

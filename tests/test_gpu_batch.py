@@ -1,0 +1,91 @@
+"""Sixteen sequences at once (l2j_decode_greedy_batch, l2j_batch_matmul): the matrix-core path must give every sequence
+what it gets alone.  Checked through the C ABI against the single-sequence path (itself pinned against the CPU oracle
+in test_gpu_parity.py), against the oracle directly, and against float64 products of the dequantized weights."""
+import numpy as np
+import pytest
+
+import llama2j_amd as l2j
+from llama2j_amd import TENSOR
+from llama2j_amd.binding import L2JError
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    (512, 1024, 4, 8, 8, 1008, 64, 1),      # head 64, shared classifier
+    (512, 1024, 2, 8, 2, 1008, 64, 0),      # grouped-query attention: 8 heads on 2 kv heads
+    (1024, 2816, 2, 8, 4, 2000, 96, 0),     # head 128, rows of 4 and 11 groups (an odd number of groups: a last slice of one)
+    (512, 768, 2, 2, 2, 512, 40, 1),        # head 256
+]
+
+
+def dequantized(g, tensor, layer, rows, K):
+    """One layer's matrix as float64, from the .quant bytes the library serialises (min, max big-endian, 256 codes)."""
+    per = rows * K // 256
+    raw = g.read_quant(tensor, layer * per, per).reshape(per, 264)
+    hdr = raw[:, :8].copy().view(">f4").astype(np.float32)
+    mn, mx = hdr[:, 0], hdr[:, 1]
+    rm = ((mx - mn) / np.float32(255.0)).astype(np.float32)          # K/MatMul.java:137
+    w = raw[:, 8:].astype(np.float32) * rm[:, None] + mn[:, None]    # K/MatMul.java:141
+    return w.reshape(rows, K).astype(np.float64)
+
+
+def test_matrix_core_product_matches_float64():
+    shape = (1024, 2816, 2, 8, 4, 2000, 96, 0)
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(7, 0.02)
+    g.finalize()
+    rng = np.random.default_rng(0)
+    kvd = 1024 * 4 // 8
+    for tensor, rows, K in ((TENSOR.WQ, 1024, 1024), (TENSOR.WK, kvd, 1024), (TENSOR.W1, 2816, 1024), (TENSOR.W2, 1024, 2816)):
+        x = (rng.standard_normal((16, K)) * np.exp(rng.uniform(-3, 3, (16, 1)))).astype(np.float32)
+        want = x.astype(np.float64) @ dequantized(g, tensor, 1, rows, K).T
+        for gps in (1, 2, 3, 8):
+            got, _ = g.batch_matmul(tensor, 1, x, rows, groups_per_slice=gps)
+            err = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)      # per sequence
+            assert err.max() < 5e-6, (int(tensor), gps, float(err.max()))
+    g.close()
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_every_sequence_gets_what_it_gets_alone(orc, shape):
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(9, 0.02)
+    g.finalize()
+    rng = np.random.default_rng(shape[0] + shape[4])
+    steps = shape[6]
+    prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 9))).astype(np.int32) for _ in range(13)]   # three without a prompt
+    got, sec = g.decode_greedy_batch(prompts, steps)
+    assert got.shape == (16, steps) and sec > 0
+    for b in range(16):
+        p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
+        g.reset()
+        want, _ = g.decode_greedy(p, steps)          # stops after token 1; the batch runs on
+        np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d" % b)
+        np.testing.assert_array_equal(got[b, :len(p)], p)
+    # two of them against the oracle as well
+    m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
+                  vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
+    m.fill_synth(9, 0.02)
+    for b in (0, 15):
+        p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
+        m.reset()
+        want, _, _ = m.generate_greedy(p, steps)
+        np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d against the oracle" % b)
+    # the context's own cache and loop state are untouched: a single decode after the batch is what it was before
+    g.reset()
+    again, _ = g.decode_greedy(prompts[0], steps)
+    np.testing.assert_array_equal(again, got[0, :len(again)])
+    m.close(); g.close()
+
+
+def test_shapes_the_batched_path_does_not_take_are_an_error():
+    g = l2j.Transformer(l2j.Config(288, 768, 1, 6, 6, 320, 16, 1))   # rows of 288 codes: groups straddle rows
+    g.fill_synthetic(1, 0.02)
+    g.finalize()
+    with pytest.raises(L2JError) as e:
+        g.decode_greedy_batch([np.array([5, 6], dtype=np.int32)], 8)
+    assert e.value.code == -2
+    with pytest.raises(L2JError):
+        g.batch_matmul(TENSOR.WQ, 0, np.zeros((16, 288), dtype=np.float32), 288)
+    assert len(g.decode_greedy(np.array([5, 6], dtype=np.int32), 8)[0]) > 0     # the context stays usable
+    g.close()
