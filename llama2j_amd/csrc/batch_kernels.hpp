@@ -17,15 +17,21 @@ constexpr int kXPad = 4;            // floats between the slices of two sequence
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
 
-// y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].
+// y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].  Up to three matrices that
+// share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
+constexpr int kBgMaxMat = 3;
 struct BGemm {
-    QMat m;            // m.off: the layer's matrix (a multiple of 256), rows of K codes
-    int rows, K;       // rows % 16 == 0, K % 256 == 0
-    const float *x;    // (kBatch, K)
-    const float *sx;   // (kBatch, K / 256): sum of x over each group
-    float *part;       // (slices, kBatch, rows)
-    int gps;           // groups of 256 codes per slice
+    QMat m[kBgMaxMat];        // m.off: the layer's matrix (a multiple of 256), rows of K codes
+    int rows[kBgMaxMat];      // rows % 16 == 0
+    float *part[kBgMaxMat];   // (slices, kBatch, rows)
+    int nmat;
+    int K;                    // K % 256 == 0
+    const float *x;           // (kBatch, K)
+    const float *sx;          // (kBatch, K / 256): sum of x over each group
+    int gps;                  // groups of 256 codes per slice
 };
+
+__host__ __device__ inline int bg_row_blocks(int rows) { return (rows + 127) / 128; }
 
 __device__ __forceinline__ float code_f(const uint4 &w, int j)
 {
@@ -43,13 +49,18 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngroups = a.K >> 8;
     const int g0 = blockIdx.y * a.gps, g1 = min(ngroups, g0 + a.gps), nk = (g1 - g0) << 8;
-    const int row0 = min(blockIdx.x * kBgRowsPerWG + wave * kBgRowsPerWave, a.rows - 16);   // (a wave past the end repeats the last tile)
-    const bool live = blockIdx.x * kBgRowsPerWG + wave * kBgRowsPerWave < a.rows;
+    int mi = 0, rb = blockIdx.x;   // which matrix, which of its row blocks
+    while (mi + 1 < a.nmat && rb >= bg_row_blocks(a.rows[mi])) { rb -= bg_row_blocks(a.rows[mi]); mi++; }
+    const QMat mat = a.m[mi];
+    const int rows = a.rows[mi];
+    float *const part = a.part[mi];
+    const int row0 = min(rb * kBgRowsPerWG + wave * kBgRowsPerWave, rows - 16);   // (a wave past the end repeats the last tile)
+    const bool live = rb * kBgRowsPerWG + wave * kBgRowsPerWave < rows;
     const int r = lane & 15, s = lane >> 4;
-    const bool two = row0 + 16 < a.rows;
-    const uint4 *c0 = reinterpret_cast<const uint4 *>(a.m.codes + a.m.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
+    const bool two = row0 + 16 < rows;
+    const uint4 *c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
     const uint4 *c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
-    const float2 *gs0 = a.m.gs + ((a.m.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
+    const float2 *gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
     const float2 *gs1 = gs0 + (two ? 16L * ngroups : 0L);
     const float *sxp = a.sx + (long)r * ngroups + g0;   // this lane's column is sequence r
     v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
@@ -118,7 +129,7 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         gs0++; gs1++; sxp++;
     }
     // lane holds rows row0 + 4 s + (0..3) of sequence r
-    float *p = a.part + ((long)blockIdx.y * kBatch + r) * a.rows + row0 + 4 * s;
+    float *p = part + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;
     *reinterpret_cast<v4f32 *>(p) = y0;
     if (two) *reinterpret_cast<v4f32 *>(p + 16) = y1;
 }
@@ -258,6 +269,50 @@ __global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, cons
     }
 }
 
+// x[b] += the slices of a product summed in order (K/Accum.java:26-30), then xn[b] and its group sums as k_brms does: the
+// hand-over from Wo to W1/W3 and from W2 to the next layer's Wq/Wk/Wv (or to the classifier) in one kernel.
+__global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ part, int slices, float *__restrict__ x, const float *__restrict__ w,
+                                                   float *__restrict__ xn, float *__restrict__ sx, int n)
+{
+    __shared__ float red[16];
+    const int b = blockIdx.x, tid = threadIdx.x, n4 = n >> 2;
+    const long stride4 = (long)kBatch * n4;   // 16-byte words between two slices
+    const float4 *pp = reinterpret_cast<const float4 *>(part) + (long)b * n4;
+    float4 *xp = reinterpret_cast<float4 *>(x + (long)b * n);
+    float ssq = 0.0f;
+    for (int i = tid; i < n4; i += 1024) {
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int s = 0; s < slices; s++) {
+            const float4 v = pp[(long)s * stride4 + i];
+            t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+        }
+        float4 v = xp[i];
+        v.x = __fadd_rn(v.x, t.x); v.y = __fadd_rn(v.y, t.y); v.z = __fadd_rn(v.z, t.z); v.w = __fadd_rn(v.w, t.w);
+        xp[i] = v;
+        ssq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+    }
+    ssq = block_sum(ssq, red, 16);   // (its barriers also order the stores above before the loads below)
+    const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
+    const float4 *wp = reinterpret_cast<const float4 *>(w);
+    float4 *op = reinterpret_cast<float4 *>(xn + (long)b * n);
+    for (int i0 = 0; i0 < n4; i0 += 1024) {
+        const int i = i0 + tid;
+        float t = 0.0f;
+        if (i < n4) {
+            float4 v = xp[i];   // (written by this same thread)
+            const float4 wv = wp[i];
+            v.x = __fmul_rn(wv.x, __fmul_rn(ss, v.x));
+            v.y = __fmul_rn(wv.y, __fmul_rn(ss, v.y));
+            v.z = __fmul_rn(wv.z, __fmul_rn(ss, v.z));
+            v.w = __fmul_rn(wv.w, __fmul_rn(ss, v.w));
+            op[i] = v;
+            t = (v.x + v.y) + (v.z + v.w);
+        }
+        t = wave_sum(t);
+        if ((tid & 63) == 0 && i < n4) sx[(long)b * (n >> 8) + (i >> 6)] = t;
+    }
+}
+
 struct BQkv {
     const float *pq, *pk, *pv;   // partial products (slices, kBatch, dim | kv_dim)
     int sq, sk;                  // slices of q, of k and v
@@ -294,17 +349,6 @@ __global__ void __launch_bounds__(256) k_bepi_qkv(const BQkv a)
     float *dst = which == 0 ? a.q + (long)b * a.dim + rr
                             : (which == 1 ? a.kc : a.vc) + ((long)b * a.seq_stride + pos) * a.kv_dim + rr;
     *reinterpret_cast<float2 *>(dst) = make_float2(v0, v1);
-}
-
-// x[b][r] += the slices of a product summed in order (K/Accum.java:26-30)
-__global__ void __launch_bounds__(256) k_bepi_res(const float *__restrict__ part, int slices, float *__restrict__ x, int rows)
-{
-    const long n = (long)kBatch * rows;
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    float t = 0.0f;
-    for (int s = 0; s < slices; s++) t += part[(long)s * n + i];
-    x[i] = __fadd_rn(x[i], t);
 }
 
 // hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74) and the group sums of hb.

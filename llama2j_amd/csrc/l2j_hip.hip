@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -1573,8 +1574,8 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             BGemm a{};
-            a.m = qmat(c, tensor, (uint64_t)layer * rows * K);
-            a.rows = rows; a.K = K; a.x = dx; a.sx = dsx; a.part = dpart; a.gps = gps;
+            a.m[0] = qmat(c, tensor, (uint64_t)layer * rows * K);
+            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.sx = dsx; a.gps = gps;
             hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * ngroups + 3) / 4), dim3(256), 0, c->stream, dx, dsx, K);
             const dim3 grid((rows + kBgRowsPerWG - 1) / kBgRowsPerWG, slices);
             const int n = std::max(1, (int)rounds);
@@ -1607,6 +1608,7 @@ struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
     BatchState *st = nullptr;
     int *prompts = nullptr, *out = nullptr;
     unsigned *done = nullptr;
+    int *h_pin = nullptr;   // pinned: every transfer of the call goes through it, as in the single-sequence loops
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -1618,22 +1620,45 @@ struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
         if (e1) (void)hipEventDestroy(e1);
         void *ps[] = {x, xn, sx, q, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
         for (void *p : ps) (void)hipFree(p);
+        if (h_pin) (void)hipHostFree(h_pin);
     }
 };
+
+#ifdef L2J_BATCH_TIMES
+struct BtRec { std::string name; hipEvent_t e0, e1; };
+static std::vector<BtRec> g_bt;
+static bool g_bt_on = false;
+struct BtScope {
+    hipStream_t s; bool on; BtRec r;
+    BtScope(const char *n, hipStream_t st) : s(st), on(g_bt_on) { if (on) { r.name = n; (void)hipEventCreate(&r.e0); (void)hipEventCreate(&r.e1); (void)hipEventRecord(r.e0, s); } }
+    ~BtScope() { if (on) { (void)hipEventRecord(r.e1, s); g_bt.push_back(r); } }
+};
+#define BT(name) BtScope bt_scope_(name, c->stream)
+#else
+#define BT(name)
+#endif
 
 constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
 
 int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
 size_t batch_lds() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }
 
-void launch_bgemm(l2j_ctx *c, int tensor, int layer, const float *x, const float *sx, float *part)
+// The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
+void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, const float *sx, float *const *part)
 {
-    int rows = 0, K = 0;
-    matrix_shape(c->cfg, tensor, &rows, &K);
     BGemm a{};
-    a.m = qmat(c, tensor, (uint64_t)layer * rows * K);
-    a.rows = rows; a.K = K; a.x = x; a.sx = sx; a.part = part; a.gps = kBatchGps;
-    hipLaunchKernelGGL(k_bgemm, dim3((rows + kBgRowsPerWG - 1) / kBgRowsPerWG, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
+    int blocks = 0, K = 0;
+    for (int tensor : tensors) {
+        int rows = 0;
+        matrix_shape(c->cfg, tensor, &rows, &K);
+        a.m[a.nmat] = qmat(c, tensor, (uint64_t)layer * rows * K);
+        a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
+        blocks += bg_row_blocks(rows);
+        a.nmat++;
+    }
+    a.K = K; a.x = x; a.sx = sx; a.gps = kBatchGps;
+    BT(*tensors.begin() == L2J_WQ ? "gemm qkv" : *tensors.begin() == L2J_WO ? "gemm wo" : *tensors.begin() == L2J_W2 ? "gemm w2" : "gemm w1,w3");
+    hipLaunchKernelGGL(k_bgemm, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
 }
 
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
@@ -1643,45 +1668,45 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
     const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim;
     const int sd = batch_slices(dim), sh = batch_slices(hidden);
     hipStream_t s = c->stream;
-    hipLaunchKernelGGL(k_bembed, dim3(kBatch), dim3(256), 0, s, c->emb, b.st, b.x, dim);
+    { BT("embed"); hipLaunchKernelGGL(k_bembed, dim3(kBatch), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
+    { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw, b.xn, b.sx, dim); }
     for (int l = 0; l < L; l++) {
-        hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)l * dim, b.xn, b.sx, dim);
-        launch_bgemm(c, L2J_WQ, l, b.xn, b.sx, b.part[0]);
-        launch_bgemm(c, L2J_WK, l, b.xn, b.sx, b.part[1]);
-        launch_bgemm(c, L2J_WV, l, b.xn, b.sx, b.part[2]);
+        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.sx, b.part);
         BQkv e{};
         e.pq = b.part[0]; e.pk = b.part[1]; e.pv = b.part[2]; e.sq = sd; e.sk = sd;
         e.dim = dim; e.kv_dim = kvd; e.head_size = hs; e.rope = c->rope; e.st = b.st; e.q = b.q;
         e.kc = b.kc + (size_t)l * max_pos * kvd; e.vc = b.vc + (size_t)l * max_pos * kvd;
         e.seq_stride = (long)L * max_pos;
-        hipLaunchKernelGGL(k_bepi_qkv, dim3(((dim + 2 * kvd) / 2 + 255) / 256, kBatch), dim3(256), 0, s, e);
+        { BT("epi qkv"); hipLaunchKernelGGL(k_bepi_qkv, dim3(((dim + 2 * kvd) / 2 + 255) / 256, kBatch), dim3(256), 0, s, e); }
         BAttn t{};
         t.q = b.q; t.kc = e.kc; t.vc = e.vc; t.seq_stride = e.seq_stride; t.out = b.xb; t.st = b.st;
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
         const dim3 ag(cf.n_heads, kBatch);
-        if (hs == 64) hipLaunchKernelGGL(k_battn<16>, ag, dim3(256), 0, s, t);
-        else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
-        else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
-        hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * (dim / 256) + 3) / 4), dim3(256), 0, s, b.xb, b.sx, dim);
-        launch_bgemm(c, L2J_WO, l, b.xb, b.sx, b.part[0]);
-        hipLaunchKernelGGL(k_bepi_res, dim3((kBatch * dim + 255) / 256), dim3(256), 0, s, b.part[0], sd, b.x, dim);
-        hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, b.sx, dim);
-        launch_bgemm(c, L2J_W1, l, b.xn, b.sx, b.part[0]);
-        launch_bgemm(c, L2J_W3, l, b.xn, b.sx, b.part[1]);
-        hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, kBatch), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
-                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb, b.sx);
-        launch_bgemm(c, L2J_W2, l, b.hb, b.sx, b.part[0]);
-        hipLaunchKernelGGL(k_bepi_res, dim3((kBatch * dim + 255) / 256), dim3(256), 0, s, b.part[0], sh, b.x, dim);
+        {
+            BT("attention");
+            if (hs == 64) hipLaunchKernelGGL(k_battn<16>, ag, dim3(256), 0, s, t);
+            else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
+            else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
+        }
+        { BT("group sums"); hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * (dim / 256) + 3) / 4), dim3(256), 0, s, b.xb, b.sx, dim); }
+        launch_bgemm(c, {L2J_WO}, l, b.xb, b.sx, b.part);
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, b.sx, dim); }
+        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.sx, b.part);
+        { BT("epi swiglu"); hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, kBatch), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
+                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb, b.sx); }
+        launch_bgemm(c, {L2J_W2}, l, b.hb, b.sx, b.part);
+        // the residual, then the norm of what follows: the next layer's attention norm, or the final one (rmsw: att, ffn, final)
+        const float *wn = c->rmsw + (l + 1 < L ? (size_t)(l + 1) * dim : (size_t)2 * L * dim);
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, b.sx, dim); }
     }
-    hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw + (size_t)2 * L * dim, b.xn, b.sx, dim);
     BGemmF32 g{};
     g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
-    hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds(), s, g);
+    { BT("classifier"); hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds(), s, g); }
     BNext n{};
     n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
     n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
-    hipLaunchKernelGGL(k_bnext, dim3(kBatch), dim3(1024), 0, s, n, b.done);
+    { BT("next"); hipLaunchKernelGGL(k_bnext, dim3(kBatch), dim3(1024), 0, s, n, b.done); }
 }
 
 }  // namespace
@@ -1725,12 +1750,16 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
         alloc(&b.st, 1); alloc(&b.prompts, (size_t)kBatch * pstride); alloc(&b.out, (size_t)kBatch * steps); alloc(&b.done, 1);
         if (e == hipSuccess) e = hipEventCreate(&b.e0);
         if (e == hipSuccess) e = hipEventCreate(&b.e1);
+        const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)kBatch * pstride, out_ints = (size_t)kBatch * steps;
+        if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&b.h_pin), std::max(state_ints + prompt_ints, out_ints) * sizeof(int), hipHostMallocDefault);
         if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: ") + hipGetErrorString(e)));
         BatchState h{};
         h.pos = 0;
         for (int i = 0; i < kBatch; i++) { h.token[i] = 1; h.n_prompt[i] = n_prompt[i]; }   // BOS first (J/Run.java:612)
-        if (hipMemcpyAsync(b.st, &h, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
-            (prompt_stride > 0 && hipMemcpyAsync(b.prompts, prompts, (size_t)kBatch * prompt_stride * sizeof(int), hipMemcpyHostToDevice, c->stream) != hipSuccess) ||
+        memcpy(b.h_pin, &h, sizeof(h));
+        if (prompt_stride > 0) memcpy(b.h_pin + state_ints, prompts, prompt_ints * sizeof(int));
+        if (hipMemcpyAsync(b.st, b.h_pin, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
+            (prompt_stride > 0 && hipMemcpyAsync(b.prompts, b.h_pin + state_ints, prompt_ints * sizeof(int), hipMemcpyHostToDevice, c->stream) != hipSuccess) ||
             hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream) != hipSuccess ||
             hipFuncSetAttribute((const void *)k_bgemm, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
             hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
@@ -1751,8 +1780,27 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
         }
         if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);
-        if (e == hipSuccess) e = hipMemcpyAsync(out_tokens, b.out, (size_t)kBatch * steps * sizeof(int), hipMemcpyDeviceToHost, c->stream);
+#ifdef L2J_BATCH_TIMES
+        if (e == hipSuccess && steps > 8) {   // one more step, kernel by kernel, each between two events (position steps - 1 again)
+            (void)hipStreamSynchronize(c->stream);
+            BatchState h2{};
+            (void)hipMemcpy(&h2, b.st, sizeof(h2), hipMemcpyDeviceToHost);
+            h2.pos = steps - 1;
+            (void)hipMemcpy(b.st, &h2, sizeof(h2), hipMemcpyHostToDevice);
+            g_bt_on = true; g_bt.clear();
+            launch_batch_step(c, b, steps, pstride);
+            g_bt_on = false;
+            (void)hipStreamSynchronize(c->stream);
+            std::map<std::string, std::pair<double, int>> acc;
+            for (auto &t : g_bt) { float ms = 0; (void)hipEventElapsedTime(&ms, t.e0, t.e1); acc[t.name].first += ms * 1e3; acc[t.name].second++; (void)hipEventDestroy(t.e0); (void)hipEventDestroy(t.e1); }
+            double tot = 0; for (auto &kv : acc) tot += kv.second.first;
+            for (auto &kv : acc) fprintf(stderr, "[batch step] %-14s %4d launches %9.1f us total %7.2f us each\n", kv.first.c_str(), kv.second.second, kv.second.first, kv.second.first / kv.second.second);
+            fprintf(stderr, "[batch step] sum %.1f us\n", tot);
+        }
+#endif
+        if (e == hipSuccess) e = hipMemcpyAsync(b.h_pin, b.out, out_ints * sizeof(int), hipMemcpyDeviceToHost, c->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        if (e == hipSuccess) memcpy(out_tokens, b.h_pin, out_ints * sizeof(int));
         float ms = 0.0f;
         if (e == hipSuccess && steps > 1) e = hipEventElapsedTime(&ms, b.e0, b.e1);
         if (seconds) *seconds = (double)ms * 1e-3;
