@@ -130,6 +130,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=97, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
     ap.add_argument("--no-sampled", action="store_true", help="skip the extra decode with the device sampler")
+    ap.add_argument("--no-batched", action="store_true", help="skip the extra decode of sixteen sequences at once")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
     a = ap.parse_args()
@@ -228,6 +229,21 @@ def main():
         except l2j.L2JError as e:  # a vocabulary above the device sampler's limit
             out["sampled_decode"] = {"error": str(e)}
         g.reset()
+
+    if not a.no_batched and not long_context:
+        # Not the metric either: sixteen sequences decoded at once (every weight read once per step for all of them, the
+        # products on the fp32 matrix cores); sequence 0 has the prompt of the timed run and must repeat its tokens.
+        try:
+            bsteps = min(steps, 288)
+            prompts = [prompt] + [synth_prompt(seed + 1000 + b, n_prompt, shape[5]) for b in range(1, 16)]
+            g.decode_greedy_batch(prompts, min(bsteps, 8))          # warm
+            btoks, bsec = g.decode_greedy_batch(prompts, bsteps)
+            n0 = min(bsteps, len(tokens))
+            out["batched_decode"] = {"sequences": 16, "steps": bsteps, "tok_s": round(16 * (bsteps - 1) / bsec, 1),
+                                     "ms_per_step": round(bsec / (bsteps - 1) * 1e3, 4),
+                                     "sequence_0_equals_the_single_decode": bool(np.array_equal(btoks[0, :n0], tokens[:n0]))}
+        except l2j.L2JError as e:  # shapes the batched path does not take (rows that are not whole groups of 256)
+            out["batched_decode"] = {"error": str(e)}
 
     if a.calibrate_copy > 0:
         g.calibration_copy(a.calibrate_copy << 20, 3)
