@@ -1765,18 +1765,27 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
             hipStreamSynchronize(c->stream) != hipSuccess)
             return done(fail(L2J_E_HIP, "batched decode: set-up failed"));
-        // one position as a graph: every kernel reads the position and the tokens from device memory
-        e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
-        if (e == hipSuccess) {
-            launch_batch_step(c, b, steps, pstride);
-            const hipError_t le = hipGetLastError();
-            e = hipStreamEndCapture(c->stream, &b.graph);
-            if (e == hipSuccess) e = le;
+        // one position as a graph: every kernel reads the position and the tokens from device memory ("graph" = 0: the
+        // kernels are launched one by one, for profilers)
+        const bool use_graph = c->opt[OPT_GRAPH] != 0;
+        if (use_graph) {
+            e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+            if (e == hipSuccess) {
+                launch_batch_step(c, b, steps, pstride);
+                const hipError_t le = hipGetLastError();
+                e = hipStreamEndCapture(c->stream, &b.graph);
+                if (e == hipSuccess) e = le;
+            }
+            if (e == hipSuccess) e = hipGraphInstantiate(&b.exec, b.graph, nullptr, nullptr, 0);
+            if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: graph capture: ") + hipGetErrorString(e)));
         }
-        if (e == hipSuccess) e = hipGraphInstantiate(&b.exec, b.graph, nullptr, nullptr, 0);
-        if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: graph capture: ") + hipGetErrorString(e)));
         for (int pos = 0; pos < steps && e == hipSuccess; pos++) {
-            e = hipGraphLaunch(b.exec, c->stream);
+            if (use_graph) {
+                e = hipGraphLaunch(b.exec, c->stream);
+            } else {
+                launch_batch_step(c, b, steps, pstride);
+                e = hipGetLastError();
+            }
             if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
         }
         if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);
