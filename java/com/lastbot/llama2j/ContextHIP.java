@@ -40,7 +40,7 @@ public final class ContextHIP implements AutoCloseable {
     // buffers of the token loop's thread, allocated once (no allocation per token)
     private final MemorySegment logitsSeg, intSeg, tokensSeg, promptSeg, countSeg, secondsSeg;
     private final MethodHandle lastError, ctxLastError, destroy, setOption, uploadQuant, uploadF32, finalizeH, reset, forward,
-            forwardArgmax, decodeGreedy, decodeSample, samplerSeed, sample;
+            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSample, samplerSeed, sample;
 
     private MethodHandle handle(String name, FunctionDescriptor fd) {
         return LINKER.downcallHandle(lib.find(name).orElseThrow(), fd);
@@ -60,6 +60,8 @@ public final class ContextHIP implements AutoCloseable {
         forwardArgmax = handle("l2j_forward_argmax", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS));
         decodeGreedy = handle("l2j_decode_greedy",
                 FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS));
+        decodeGreedyBatch = handle("l2j_decode_greedy_batch",
+                FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
         decodeSample = handle("l2j_decode_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
                 JAVA_FLOAT, JAVA_FLOAT, JAVA_LONG, ADDRESS, ADDRESS, ADDRESS));
         samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
@@ -226,6 +228,31 @@ public final class ContextHIP implements AutoCloseable {
     public Generation decodeGreedy(int[] prompt, int steps) {
         check(call(decodeGreedy, ctx, stagePrompt(prompt), prompt.length, steps, tokensSeg, countSeg, secondsSeg));
         return generation();
+    }
+
+    /**
+     * Sixteen greedy token loops at once (l2j_decode_greedy_batch): every weight is read once per step for all of them.
+     * prompts: at most sixteen id arrays (missing ones run without a prompt); result[b] holds `steps` tokens of
+     * sequence b, which runs on after token 1: cut it there.  No counterpart in the reference.
+     */
+    public int[][] decodeGreedyBatch(int[][] prompts, int steps) {
+        final int batch = 16;
+        if (prompts.length > batch) throw new IllegalArgumentException("at most 16 sequences");
+        int stride = 1;
+        for (int[] p : prompts) stride = Math.max(stride, p.length);
+        try (Arena a = Arena.ofConfined()) {
+            MemorySegment ids = a.allocate((long) batch * stride * Integer.BYTES, 16);
+            MemorySegment counts = a.allocate((long) batch * Integer.BYTES, 16);
+            MemorySegment out = a.allocate((long) batch * steps * Integer.BYTES, 16);
+            for (int b = 0; b < prompts.length; b++) {
+                MemorySegment.copy(prompts[b], 0, ids, JAVA_INT, (long) b * stride * Integer.BYTES, prompts[b].length);
+                counts.setAtIndex(JAVA_INT, b, prompts[b].length);
+            }
+            check(call(decodeGreedyBatch, ctx, ids, counts, stride, steps, out, secondsSeg));
+            int[][] tokens = new int[batch][steps];
+            for (int b = 0; b < batch; b++) MemorySegment.copy(out, JAVA_INT, (long) b * steps * Integer.BYTES, tokens[b], 0, steps);
+            return tokens;
+        }
     }
 
     /** The token loop of Run.main with Sampler(rngSeed) on the device (temperature, top-p as in CommandLine). */
