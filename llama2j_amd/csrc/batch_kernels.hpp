@@ -31,7 +31,7 @@ struct BGemm {
     int gps;                  // groups of 256 codes per slice
 };
 
-__host__ __device__ inline int bg_row_blocks(int rows) { return (rows + kBgRowsPerWG - 1) / kBgRowsPerWG; }
+__host__ __device__ inline int bg_row_blocks(int rows, int tiles) { const int per = 16 * tiles * (kBgThreads / 64); return (rows + per - 1) / per; }
 
 __device__ __forceinline__ float code_f(const uint4 &w, int j)
 {
@@ -40,9 +40,10 @@ __device__ __forceinline__ float code_f(const uint4 &w, int j)
 }
 
 // Workgroup (x: 128 rows, y: one slice of K): the slice of the sixteen activation vectors is staged in LDS; every
-// wave takes 32 rows.  A lane (r = lane % 16, s = lane / 16) holds the codes of row r at k = 64 T + 16 s + j (T < 4,
+// wave takes 32 rows (TILES = 2; or 16, TILES = 1, for a matrix too small to fill the GPU otherwise).  A lane (r = lane % 16, s = lane / 16) holds the codes of row r at k = 64 T + 16 s + j (T < 4,
 // j < 16: four 16-byte loads per group and tile); step (T, j) of the MFMA multiplies the 16 rows by the 16 sequences
 // over the four k of the four s.  After the 64 steps of a group the 16 x 16 sums get the group's scale and offset.
+template <int TILES>
 __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
 {
     extern __shared__ float xs[];
@@ -50,14 +51,15 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     const int ngroups = a.K >> 8;
     const int g0 = blockIdx.y * a.gps, g1 = min(ngroups, g0 + a.gps), nk = (g1 - g0) << 8;
     int mi = 0, rb = blockIdx.x;   // which matrix, which of its row blocks
-    while (mi + 1 < a.nmat && rb >= bg_row_blocks(a.rows[mi])) { rb -= bg_row_blocks(a.rows[mi]); mi++; }
+    while (mi + 1 < a.nmat && rb >= bg_row_blocks(a.rows[mi], TILES)) { rb -= bg_row_blocks(a.rows[mi], TILES); mi++; }
     const QMat mat = a.m[mi];
     const int rows = a.rows[mi];
     float *const part = a.part[mi];
-    const int row0 = min(rb * kBgRowsPerWG + wave * kBgRowsPerWave, rows - 16);   // (a wave past the end repeats the last tile)
-    const bool live = rb * kBgRowsPerWG + wave * kBgRowsPerWave < rows;
+    constexpr int kRowsWave = 16 * TILES, kRowsWG = kRowsWave * (kBgThreads / 64);
+    const int row0 = min(rb * kRowsWG + wave * kRowsWave, rows - 16);   // (a wave past the end repeats the last tile)
+    const bool live = rb * kRowsWG + wave * kRowsWave < rows;
     const int r = lane & 15, s = lane >> 4;
-    const bool two = row0 + 16 < rows;
+    const bool two = TILES == 2 && row0 + 16 < rows;
     const uint4 *c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
     const uint4 *c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
     const float2 *gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
@@ -66,7 +68,7 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
     uint4 w0[4], w1[4];   // the first codes are requested before the activations are staged
 #pragma unroll
-    for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); w1[T] = load_stream(c1 + 4 * T); }
+    for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
     const int pitch = nk + kXPad;   // LDS: sequence-major, xs[b * pitch + k]
     {
         const int nk4 = nk >> 2;   // 16-byte words per sequence in the slice
@@ -85,11 +87,11 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         if (g + 1 < g1) {   // the next group's codes are requested before this one is multiplied
             c0 += 16; c1 += 16;
 #pragma unroll
-            for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); w1[T] = load_stream(c1 + 4 * T); }
+            for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
         }
         float2 sc0[4], sc1[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; sc1[i] = gs1[(long)i * ngroups]; }
+        for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; if (TILES == 2) sc1[i] = gs1[(long)i * ngroups]; }
         const float sxv = *sxp;
         v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
         const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + ((g - g0) << 8) + 16 * s);   // sequence r, k = 64 T + 16 s + j
@@ -113,10 +115,10 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
                     const int j = 4 * q + e;
                     if (e & 1) {   // two sums per tile: four independent chains of MFMAs
                         acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc2, 0, 0, 0);
-                        acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc3, 0, 0, 0);
+                        if (TILES == 2) acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc3, 0, 0, 0);
                     } else {
                         acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc1, 0, 0, 0);
+                        if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc1, 0, 0, 0);
                     }
                 }
             }
@@ -124,7 +126,7 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
-            y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
+            if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
         }
         gs0++; gs1++; sxp++;
     }

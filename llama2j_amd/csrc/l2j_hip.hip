@@ -1570,18 +1570,18 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
         if (e == hipSuccess) e = hipEventCreate(&e0);
         if (e == hipSuccess) e = hipEventCreate(&e1);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             BGemm a{};
             a.m[0] = qmat(c, tensor, (uint64_t)layer * rows * K);
             a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.sx = dsx; a.gps = gps;
             hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * ngroups + 3) / 4), dim3(256), 0, c->stream, dx, dsx, K);
-            const dim3 grid((rows + kBgRowsPerWG - 1) / kBgRowsPerWG, slices);
+            const dim3 grid(bg_row_blocks(rows, 2), slices);
             const int n = std::max(1, (int)rounds);
-            hipLaunchKernelGGL(k_bgemm, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
+            hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
             (void)hipEventRecord(e0, c->stream);
-            for (int i = 0; i < n; i++) hipLaunchKernelGGL(k_bgemm, grid, dim3(kBgThreads), lds, c->stream, a);
+            for (int i = 0; i < n; i++) hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);
             (void)hipEventRecord(e1, c->stream);
             hipLaunchKernelGGL(k_breduce, dim3(256), dim3(256), 0, c->stream, dpart, dy, rows, slices);
             e = hipGetLastError();
@@ -1647,18 +1647,22 @@ size_t batch_lds() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(
 void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, const float *sx, float *const *part)
 {
     BGemm a{};
-    int blocks = 0, K = 0;
+    int K = 0;
     for (int tensor : tensors) {
         int rows = 0;
         matrix_shape(c->cfg, tensor, &rows, &K);
         a.m[a.nmat] = qmat(c, tensor, (uint64_t)layer * rows * K);
         a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
-        blocks += bg_row_blocks(rows);
         a.nmat++;
     }
     a.K = K; a.x = x; a.sx = sx; a.gps = kBatchGps;
+    // 32 rows per wave, or 16 when that leaves more than half of the GPU's workgroup slots (4 per compute unit) empty
+    auto blocks_of = [&](int tiles) { int n = 0; for (int i = 0; i < a.nmat; i++) n += bg_row_blocks(a.rows[i], tiles); return n; };
+    const int tiles = blocks_of(2) * batch_slices(K) * 2 <= 4 * c->n_cu ? 1 : 2;
+    const int blocks = blocks_of(tiles);
     BT(*tensors.begin() == L2J_WQ ? "gemm qkv" : *tensors.begin() == L2J_WO ? "gemm wo" : *tensors.begin() == L2J_W2 ? "gemm w2" : "gemm w1,w3");
-    hipLaunchKernelGGL(k_bgemm, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
+    if (tiles == 1) hipLaunchKernelGGL(k_bgemm<1>, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
+    else hipLaunchKernelGGL(k_bgemm<2>, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
 }
 
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
@@ -1761,7 +1765,8 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
         if (hipMemcpyAsync(b.st, b.h_pin, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
             (prompt_stride > 0 && hipMemcpyAsync(b.prompts, b.h_pin + state_ints, prompt_ints * sizeof(int), hipMemcpyHostToDevice, c->stream) != hipSuccess) ||
             hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream) != hipSuccess ||
-            hipFuncSetAttribute((const void *)k_bgemm, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
             hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
             hipStreamSynchronize(c->stream) != hipSuccess)
             return done(fail(L2J_E_HIP, "batched decode: set-up failed"));
