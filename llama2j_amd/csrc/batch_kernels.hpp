@@ -20,6 +20,7 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 // y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].  Up to three matrices that
 // share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
 constexpr int kBgMaxMat = 3;
+constexpr int kBgMaxGps = 16;       // most groups per slice
 struct BGemm {
     QMat m[kBgMaxMat];        // m.off: the layer's matrix (a multiple of 256), rows of K codes
     int rows[kBgMaxMat];      // rows % 16 == 0
@@ -27,7 +28,6 @@ struct BGemm {
     int nmat;
     int K;                    // K % 256 == 0
     const float *x;           // (kBatch, K)
-    const float *sx;          // (kBatch, K / 256): sum of x over each group
     int gps;                  // groups of 256 codes per slice
 };
 
@@ -64,7 +64,6 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     const uint4 *c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
     const float2 *gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
     const float2 *gs1 = gs0 + (two ? 16L * ngroups : 0L);
-    const float *sxp = a.sx + (long)r * ngroups + g0;   // this lane's column is sequence r
     v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
     uint4 w0[4], w1[4];   // the first codes are requested before the activations are staged
 #pragma unroll
@@ -76,6 +75,22 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         for (int f = tid; f < kBatch * nk4; f += kBgThreads) {
             const int b = f / nk4, k4 = f - b * nk4;
             *reinterpret_cast<float4 *>(xs + b * pitch + 4 * k4) = *reinterpret_cast<const float4 *>(a.x + (long)b * a.K + (g0 << 8) + 4 * k4);
+        }
+    }
+    __syncthreads();
+    // sum of every sequence's activations over each group of the slice (for the groups' offsets): 16 threads per sequence,
+    // while the first codes are on their way
+    __shared__ float sxs[kBatch][kBgMaxGps];
+    {
+        const int b = tid >> 4, part = tid & 15;
+        for (int gi = 0; gi < g1 - g0; gi++) {
+            const float4 *xp = reinterpret_cast<const float4 *>(xs + b * pitch + (gi << 8) + 16 * part);
+            const float4 v0 = xp[0], v1 = xp[1], v2 = xp[2], v3 = xp[3];
+            float t = ((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w)) + ((v2.x + v2.y) + (v2.z + v2.w)) +
+                      ((v3.x + v3.y) + (v3.z + v3.w));
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
+            if (part == 0) sxs[b][gi] = t;
         }
     }
     __syncthreads();
@@ -92,7 +107,7 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         float2 sc0[4], sc1[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; if (TILES == 2) sc1[i] = gs1[(long)i * ngroups]; }
-        const float sxv = *sxp;
+        const float sxv = sxs[r][g - g0];   // this lane's column is sequence r
         v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
         const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + ((g - g0) << 8) + 16 * s);   // sequence r, k = 64 T + 16 s + j
         float4 xn[4];
@@ -128,24 +143,12 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
             y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
             if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
         }
-        gs0++; gs1++; sxp++;
+        gs0++; gs1++;
     }
     // lane holds rows row0 + 4 s + (0..3) of sequence r
     float *p = part + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;
     *reinterpret_cast<v4f32 *>(p) = y0;
     if (two) *reinterpret_cast<v4f32 *>(p + 16) = y1;
-}
-
-// sx[b][g] = sum of x[b][256 g .. 256 g + 255]: one wave per (b, g)
-__global__ void __launch_bounds__(256) k_bgroup_sums(const float *__restrict__ x, float *__restrict__ sx, int K)
-{
-    const int ngroups = K >> 8, lane = threadIdx.x & 63;
-    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= kBatch * ngroups) return;
-    const int b = item / ngroups, g = item % ngroups;
-    const float4 v = *reinterpret_cast<const float4 *>(x + (long)b * K + (g << 8) + 4 * lane);
-    const float t = wave_sum((v.x + v.y) + (v.z + v.w));
-    if (lane == 0) sx[(long)b * ngroups + g] = t;
 }
 
 // ---- the classifier: fp32 weights (K/MatMul.java:37-60), the same tiling -------------------------------------------
@@ -236,10 +239,9 @@ __global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, c
     for (int i = threadIdx.x; i < (dim >> 2); i += blockDim.x) dst[i] = src[i];
 }
 
-// xn[b] = w * (ss * x[b]), ss = 1 / sqrt(sum(x^2) / n + 1e-5) (K/RootMeanSquare.java:25-35, K/WeightNormalizeAndScale.java:73),
-// and the sum of xn over every group of 256.  One workgroup of 1024 threads per sequence; n a multiple of 256.
-__global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ xn,
-                                               float *__restrict__ sx, int n)
+// xn[b] = w * (ss * x[b]), ss = 1 / sqrt(sum(x^2) / n + 1e-5) (K/RootMeanSquare.java:25-35, K/WeightNormalizeAndScale.java:73).
+// One workgroup of 1024 threads per sequence.
+__global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ xn, int n)
 {
     __shared__ float red[16];
     const int b = blockIdx.x, tid = threadIdx.x, n4 = n >> 2;
@@ -253,28 +255,21 @@ __global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, cons
     const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
     const float4 *wp = reinterpret_cast<const float4 *>(w);
     float4 *op = reinterpret_cast<float4 *>(xn + (long)b * n);
-    for (int i0 = 0; i0 < n4; i0 += 1024) {   // a wave's 64 words are one group
-        const int i = i0 + tid;
-        float t = 0.0f;
-        if (i < n4) {
-            float4 v = xp[i];
-            const float4 wv = wp[i];
-            v.x = __fmul_rn(wv.x, __fmul_rn(ss, v.x));
-            v.y = __fmul_rn(wv.y, __fmul_rn(ss, v.y));
-            v.z = __fmul_rn(wv.z, __fmul_rn(ss, v.z));
-            v.w = __fmul_rn(wv.w, __fmul_rn(ss, v.w));
-            op[i] = v;
-            t = (v.x + v.y) + (v.z + v.w);
-        }
-        t = wave_sum(t);
-        if ((tid & 63) == 0 && i < n4) sx[(long)b * (n >> 8) + (i >> 6)] = t;
+    for (int i = tid; i < n4; i += 1024) {
+        float4 v = xp[i];
+        const float4 wv = wp[i];
+        v.x = __fmul_rn(wv.x, __fmul_rn(ss, v.x));
+        v.y = __fmul_rn(wv.y, __fmul_rn(ss, v.y));
+        v.z = __fmul_rn(wv.z, __fmul_rn(ss, v.z));
+        v.w = __fmul_rn(wv.w, __fmul_rn(ss, v.w));
+        op[i] = v;
     }
 }
 
-// x[b] += the slices of a product summed in order (K/Accum.java:26-30), then xn[b] and its group sums as k_brms does: the
+// x[b] += the slices of a product summed in order (K/Accum.java:26-30), then xn[b] as k_brms does: the
 // hand-over from Wo to W1/W3 and from W2 to the next layer's Wq/Wk/Wv (or to the classifier) in one kernel.
 __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ part, int slices, float *__restrict__ x, const float *__restrict__ w,
-                                                   float *__restrict__ xn, float *__restrict__ sx, int n)
+                                                   float *__restrict__ xn, int n)
 {
     __shared__ float red[16];
     const int b = blockIdx.x, tid = threadIdx.x, n4 = n >> 2;
@@ -298,21 +293,14 @@ __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ par
     const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
     const float4 *wp = reinterpret_cast<const float4 *>(w);
     float4 *op = reinterpret_cast<float4 *>(xn + (long)b * n);
-    for (int i0 = 0; i0 < n4; i0 += 1024) {
-        const int i = i0 + tid;
-        float t = 0.0f;
-        if (i < n4) {
-            float4 v = xp[i];   // (written by this same thread)
-            const float4 wv = wp[i];
-            v.x = __fmul_rn(wv.x, __fmul_rn(ss, v.x));
-            v.y = __fmul_rn(wv.y, __fmul_rn(ss, v.y));
-            v.z = __fmul_rn(wv.z, __fmul_rn(ss, v.z));
-            v.w = __fmul_rn(wv.w, __fmul_rn(ss, v.w));
-            op[i] = v;
-            t = (v.x + v.y) + (v.z + v.w);
-        }
-        t = wave_sum(t);
-        if ((tid & 63) == 0 && i < n4) sx[(long)b * (n >> 8) + (i >> 6)] = t;
+    for (int i = tid; i < n4; i += 1024) {
+        float4 v = xp[i];   // (written by this same thread)
+        const float4 wv = wp[i];
+        v.x = __fmul_rn(wv.x, __fmul_rn(ss, v.x));
+        v.y = __fmul_rn(wv.y, __fmul_rn(ss, v.y));
+        v.z = __fmul_rn(wv.z, __fmul_rn(ss, v.z));
+        v.w = __fmul_rn(wv.w, __fmul_rn(ss, v.w));
+        op[i] = v;
     }
 }
 
@@ -354,21 +342,18 @@ __global__ void __launch_bounds__(256) k_bepi_qkv(const BQkv a)
     *reinterpret_cast<float2 *>(dst) = make_float2(v0, v1);
 }
 
-// hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74) and the group sums of hb.
-// grid (hidden / 256, kBatch), 256 threads: a workgroup is one group.
+// hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74), h1 and h3 the slices summed in order.
+// grid (hidden / 256, kBatch), 256 threads.
 __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p1, const float *__restrict__ p3, int slices, int hidden,
-                                                     const float *__restrict__ silu, int exact, float *__restrict__ hb, float *__restrict__ sx)
+                                                     const float *__restrict__ silu, int exact, float *__restrict__ hb)
 {
-    __shared__ float red[4];
     const int b = blockIdx.y, rix = blockIdx.x * 256 + threadIdx.x;
     const long n = (long)kBatch * hidden, i = (long)b * hidden + rix;
     float h1 = 0.0f, h3 = 0.0f;
+#pragma unroll 8
     for (int s = 0; s < slices; s++) { h1 += p1[(long)s * n + i]; h3 += p3[(long)s * n + i]; }
     const float sg = silu_sigma(silu, h1, exact);
-    const float v = __fmul_rn(h1, __fmul_rn(sg, h3));
-    hb[i] = v;
-    const float t = block_sum(v, red, 4);
-    if (threadIdx.x == 0) sx[(long)b * (hidden >> 8) + blockIdx.x] = t;
+    hb[i] = __fmul_rn(h1, __fmul_rn(sg, h3));
 }
 
 struct BAttn {

@@ -1552,20 +1552,19 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (K % 256 || rows % 16) return fail(L2J_E_SIZE, "the batched matrix product needs rows of whole groups (K % 256 == 0) and rows % 16 == 0");
         const QTensor &t = c->qt[tensor];
         if (t.groups_loaded != t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
-        const int ngroups = K / 256, gps = std::max(1, std::min(ngroups, (int)groups_per_slice));
+        const int ngroups = K / 256, gps = std::max(1, std::min(std::min(ngroups, kBgMaxGps), (int)groups_per_slice));
         const int slices = (ngroups + gps - 1) / gps;
         const size_t lds = (size_t)kBatch * (gps * 256 + kXPad) * sizeof(float);
         if (lds > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
         HIPCHK(hipSetDevice(c->cfg.device));
-        float *dx = nullptr, *dsx = nullptr, *dpart = nullptr, *dy = nullptr;
+        float *dx = nullptr, *dpart = nullptr, *dy = nullptr;
         hipEvent_t e0 = nullptr, e1 = nullptr;
         auto release = [&]() {
-            (void)hipFree(dx); (void)hipFree(dsx); (void)hipFree(dpart); (void)hipFree(dy);
+            (void)hipFree(dx); (void)hipFree(dpart); (void)hipFree(dy);
             if (e0) (void)hipEventDestroy(e0);
             if (e1) (void)hipEventDestroy(e1);
         };
         hipError_t e = hipMalloc(reinterpret_cast<void **>(&dx), (size_t)kBatch * K * sizeof(float));
-        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dsx), (size_t)kBatch * ngroups * sizeof(float));
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dpart), (size_t)slices * kBatch * rows * sizeof(float));
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
         if (e == hipSuccess) e = hipEventCreate(&e0);
@@ -1575,8 +1574,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) {
             BGemm a{};
             a.m[0] = qmat(c, tensor, (uint64_t)layer * rows * K);
-            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.sx = dsx; a.gps = gps;
-            hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * ngroups + 3) / 4), dim3(256), 0, c->stream, dx, dsx, K);
+            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
             const dim3 grid(bg_row_blocks(rows, 2), slices);
             const int n = std::max(1, (int)rounds);
             hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
@@ -1602,7 +1600,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
 namespace {
 
 struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
-    float *x = nullptr, *xn = nullptr, *sx = nullptr, *q = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
+    float *x = nullptr, *xn = nullptr, *q = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
     float *part[3] = {nullptr, nullptr, nullptr};
     float *kc = nullptr, *vc = nullptr;
     BatchState *st = nullptr;
@@ -1618,7 +1616,7 @@ struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
         if (graph) (void)hipGraphDestroy(graph);
         if (e0) (void)hipEventDestroy(e0);
         if (e1) (void)hipEventDestroy(e1);
-        void *ps[] = {x, xn, sx, q, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
+        void *ps[] = {x, xn, q, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
         for (void *p : ps) (void)hipFree(p);
         if (h_pin) (void)hipHostFree(h_pin);
     }
@@ -1644,7 +1642,7 @@ int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
 size_t batch_lds() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }
 
 // The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
-void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, const float *sx, float *const *part)
+void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part)
 {
     BGemm a{};
     int K = 0;
@@ -1655,7 +1653,7 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
         a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
         a.nmat++;
     }
-    a.K = K; a.x = x; a.sx = sx; a.gps = kBatchGps;
+    a.K = K; a.x = x; a.gps = kBatchGps;
     // 32 rows per wave, or 16 when that leaves more than half of the GPU's workgroup slots (4 per compute unit) empty
     auto blocks_of = [&](int tiles) { int n = 0; for (int i = 0; i < a.nmat; i++) n += bg_row_blocks(a.rows[i], tiles); return n; };
     const int tiles = blocks_of(2) * batch_slices(K) * 2 <= 4 * c->n_cu ? 1 : 2;
@@ -1673,9 +1671,9 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
     const int sd = batch_slices(dim), sh = batch_slices(hidden);
     hipStream_t s = c->stream;
     { BT("embed"); hipLaunchKernelGGL(k_bembed, dim3(kBatch), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
-    { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw, b.xn, b.sx, dim); }
+    { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
     for (int l = 0; l < L; l++) {
-        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.sx, b.part);
+        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part);
         BQkv e{};
         e.pq = b.part[0]; e.pk = b.part[1]; e.pv = b.part[2]; e.sq = sd; e.sk = sd;
         e.dim = dim; e.kv_dim = kvd; e.head_size = hs; e.rope = c->rope; e.st = b.st; e.q = b.q;
@@ -1693,16 +1691,15 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
             else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
             else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
         }
-        { BT("group sums"); hipLaunchKernelGGL(k_bgroup_sums, dim3((kBatch * (dim / 256) + 3) / 4), dim3(256), 0, s, b.xb, b.sx, dim); }
-        launch_bgemm(c, {L2J_WO}, l, b.xb, b.sx, b.part);
-        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, b.sx, dim); }
-        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.sx, b.part);
+        launch_bgemm(c, {L2J_WO}, l, b.xb, b.part);
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim); }
+        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.part);
         { BT("epi swiglu"); hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, kBatch), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
-                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb, b.sx); }
-        launch_bgemm(c, {L2J_W2}, l, b.hb, b.sx, b.part);
+                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb); }
+        launch_bgemm(c, {L2J_W2}, l, b.hb, b.part);
         // the residual, then the norm of what follows: the next layer's attention norm, or the final one (rmsw: att, ffn, final)
         const float *wn = c->rmsw + (l + 1 < L ? (size_t)(l + 1) * dim : (size_t)2 * L * dim);
-        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, b.sx, dim); }
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, dim); }
     }
     BGemmF32 g{};
     g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
@@ -1747,7 +1744,7 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
         };
         alloc(&b.x, (size_t)kBatch * dim); alloc(&b.xn, (size_t)kBatch * std::max(dim, hidden));
-        alloc(&b.sx, (size_t)kBatch * (std::max(dim, hidden) / 256)); alloc(&b.q, (size_t)kBatch * dim);
+        alloc(&b.q, (size_t)kBatch * dim);
         alloc(&b.xb, (size_t)kBatch * dim); alloc(&b.hb, (size_t)kBatch * hidden); alloc(&b.logits, (size_t)kBatch * vocab);
         for (int i = 0; i < 3; i++) alloc(&b.part[i], part_floats);
         alloc(&b.kc, cache_floats); alloc(&b.vc, cache_floats);
