@@ -304,44 +304,6 @@ __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ par
     }
 }
 
-struct BQkv {
-    const float *pq, *pk, *pv;   // partial products (slices, kBatch, dim | kv_dim)
-    int sq, sk;                  // slices of q, of k and v
-    int dim, kv_dim, head_size, n_layers_stride;
-    const float2 *rope;          // (seq_len, head_size / 2) cos, sin
-    const BatchState *st;
-    float *q;                    // (kBatch, dim)
-    float *kc, *vc;              // this layer's rows of the batch cache: + (b * seq_stride + pos) * kv_dim
-    long seq_stride;             // floats between the caches of two sequences
-};
-
-// q, k, v of the step: the slices summed in order, RoPE on the pairs of q and k (K/ApplyRope.java:74-90), k and v into
-// the cache row of this position (J/Run.java:95-99).  One thread per pair; grid (pairs / 256, kBatch).
-__global__ void __launch_bounds__(256) k_bepi_qkv(const BQkv a)
-{
-    const int b = blockIdx.y, pos = a.st->pos;
-    const int p = blockIdx.x * 256 + threadIdx.x, npairs = (a.dim + 2 * a.kv_dim) >> 1;
-    if (p >= npairs) return;
-    int rr = 2 * p, which = 0, rows = a.dim, sl = a.sq;
-    const float *part = a.pq;
-    if (rr >= a.dim + a.kv_dim) { which = 2; rr -= a.dim + a.kv_dim; rows = a.kv_dim; sl = a.sk; part = a.pv; }
-    else if (rr >= a.dim) { which = 1; rr -= a.dim; rows = a.kv_dim; sl = a.sk; part = a.pk; }
-    float v0 = 0.0f, v1 = 0.0f;
-    for (int s = 0; s < sl; s++) {
-        const float2 t = *reinterpret_cast<const float2 *>(part + ((long)s * kBatch + b) * rows + rr);
-        v0 += t.x; v1 += t.y;
-    }
-    if (which < 2) {
-        const float2 cs = a.rope[(long)pos * (a.head_size >> 1) + ((rr % a.head_size) >> 1)];
-        const float r0 = __fsub_rn(__fmul_rn(v0, cs.x), __fmul_rn(v1, cs.y));
-        const float r1 = __fadd_rn(__fmul_rn(v0, cs.y), __fmul_rn(v1, cs.x));
-        v0 = r0; v1 = r1;
-    }
-    float *dst = which == 0 ? a.q + (long)b * a.dim + rr
-                            : (which == 1 ? a.kc : a.vc) + ((long)b * a.seq_stride + pos) * a.kv_dim + rr;
-    *reinterpret_cast<float2 *>(dst) = make_float2(v0, v1);
-}
-
 // hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74), h1 and h3 the slices summed in order.
 // grid (hidden / 256, kBatch), 256 threads.
 __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p1, const float *__restrict__ p3, int slices, int hidden,
@@ -357,40 +319,75 @@ __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p
 }
 
 struct BAttn {
-    const float *q;          // (kBatch, dim)
-    const float *kc, *vc;    // this layer's rows of the batch cache
-    long seq_stride;
-    float *out;              // (kBatch, dim)
+    const float *pq, *pk, *pv;   // partial products of Wq, Wk, Wv: (slices, kBatch, dim | kv_dim)
+    int slices;
+    const float2 *rope;          // (seq_len, head_size / 2) cos, sin
+    float *kc, *vc;              // this layer's rows of the batch cache: + (b * seq_stride + pos) * kv_dim
+    long seq_stride;             // cache rows between two sequences
+    float *out;                  // (kBatch, dim)
     const BatchState *st;
     int n_heads, kv_mul, head_size, kv_dim, dim;
     float sqrt_hs;
 };
 
 // Attention of one head of one sequence over positions 0..pos (K/AttentionLoop.java:29-54, K/ExpSumNormalize.java:25-38,
-// K/AccumWeightedValue.java): LPR lanes per cache row (four floats of the head each), the row slots of the workgroup
-// take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, kBatch).
+// K/AccumWeightedValue.java).  First q of the head and k, v of its kv head at this position: the slices of the products
+// summed in order, RoPE on the pairs of q and k (K/ApplyRope.java:74-90), k and v into the cache row (J/Run.java:95-99; by
+// the first head of the kv group).  Then LPR lanes per cache row (four floats of the head each): the row slots of the
+// workgroup take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, kBatch).
 template <int LPR>
 __global__ void __launch_bounds__(256) k_battn(const BAttn a)
 {
     constexpr int RPW = 64 / LPR, NSLOT = 4 * RPW;
     __shared__ float sm_m[NSLOT], sm_l[NSLOT];
     __shared__ float4 sm_acc[NSLOT * LPR];
+    __shared__ __align__(16) float sm_qkv[3][4 * LPR];
     const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     const int j = lane % LPR, slot = (tid >> 6) * RPW + lane / LPR;
-    const int len = a.st->pos + 1, hs = a.head_size;
+    const int pos = a.st->pos, len = pos + 1, hs = a.head_size, kvh = h / a.kv_mul;
+    const int half = hs >> 1;
+    for (int p = tid; p < 3 * half; p += 256) {   // one thread per pair of q, k, v
+        const int which = p / half, idx = p - which * half;
+        {
+            const int rows = which == 0 ? a.dim : a.kv_dim, row = (which == 0 ? h : kvh) * hs + 2 * idx;
+            const float *part = which == 0 ? a.pq : which == 1 ? a.pk : a.pv;
+            float v0 = 0.0f, v1 = 0.0f;
+            for (int s = 0; s < a.slices; s++) {
+                const float2 t = *reinterpret_cast<const float2 *>(part + ((long)s * kBatch + b) * rows + row);
+                v0 += t.x; v1 += t.y;
+            }
+            if (which < 2) {
+                const float2 cs = a.rope[(long)pos * half + idx];
+                const float r0 = __fsub_rn(__fmul_rn(v0, cs.x), __fmul_rn(v1, cs.y));
+                const float r1 = __fadd_rn(__fmul_rn(v0, cs.y), __fmul_rn(v1, cs.x));
+                v0 = r0; v1 = r1;
+            }
+            sm_qkv[which][2 * idx] = v0;
+            sm_qkv[which][2 * idx + 1] = v1;
+            if (which > 0 && h % a.kv_mul == 0)
+                *reinterpret_cast<float2 *>((which == 1 ? a.kc : a.vc) + ((long)b * a.seq_stride + pos) * a.kv_dim + kvh * hs + 2 * idx) =
+                    make_float2(v0, v1);
+        }
+    }
+    __syncthreads();
     const bool on = 4 * j < hs;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float4 q4 = on ? *reinterpret_cast<const float4 *>(a.q + (long)b * a.dim + h * hs + 4 * j) : zero;
-    const long base = (long)b * a.seq_stride * a.kv_dim + (h / a.kv_mul) * hs + 4 * j;
+    const float4 q4 = on ? *reinterpret_cast<const float4 *>(&sm_qkv[0][4 * j]) : zero;
+    const float4 kp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[1][4 * j]) : zero;   // the row of this position
+    const float4 vp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[2][4 * j]) : zero;
+    const long base = (long)b * a.seq_stride * a.kv_dim + kvh * hs + 4 * j;
     float m = -3.0e38f, l = 0.0f;
     float4 acc = zero;
     for (int t0 = slot; t0 < len; t0 += 2 * NSLOT) {   // two rows in flight per slot
         const int t1 = t0 + NSLOT;
         const bool ok1 = t1 < len;
-        const float4 k0 = on ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t0 * a.kv_dim) : zero;
-        const float4 v0 = on ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t0 * a.kv_dim) : zero;
-        const float4 k1 = on && ok1 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t1 * a.kv_dim) : zero;
-        const float4 v1 = on && ok1 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t1 * a.kv_dim) : zero;
+        const bool c0 = on && t0 < pos, c1 = on && t1 < pos;   // rows of earlier positions come from the cache
+        float4 k0 = c0 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t0 * a.kv_dim) : zero;
+        float4 v0 = c0 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t0 * a.kv_dim) : zero;
+        float4 k1 = c1 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t1 * a.kv_dim) : zero;
+        float4 v1 = c1 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t1 * a.kv_dim) : zero;
+        if (t0 == pos) { k0 = kp; v0 = vp; }
+        if (t1 == pos) { k1 = kp; v1 = vp; }
         float s0 = (q4.x * k0.x + q4.y * k0.y) + (q4.z * k0.z + q4.w * k0.w);
         float s1 = (q4.x * k1.x + q4.y * k1.y) + (q4.z * k1.z + q4.w * k1.w);
 #pragma unroll

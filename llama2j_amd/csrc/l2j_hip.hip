@@ -1600,7 +1600,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
 namespace {
 
 struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
-    float *x = nullptr, *xn = nullptr, *q = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
+    float *x = nullptr, *xn = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
     float *part[3] = {nullptr, nullptr, nullptr};
     float *kc = nullptr, *vc = nullptr;
     BatchState *st = nullptr;
@@ -1616,7 +1616,7 @@ struct BatchBufs {   // device memory of one l2j_decode_greedy_batch call
         if (graph) (void)hipGraphDestroy(graph);
         if (e0) (void)hipEventDestroy(e0);
         if (e1) (void)hipEventDestroy(e1);
-        void *ps[] = {x, xn, q, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
+        void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
         for (void *p : ps) (void)hipFree(p);
         if (h_pin) (void)hipHostFree(h_pin);
     }
@@ -1674,14 +1674,10 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
     { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
     for (int l = 0; l < L; l++) {
         launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part);
-        BQkv e{};
-        e.pq = b.part[0]; e.pk = b.part[1]; e.pv = b.part[2]; e.sq = sd; e.sk = sd;
-        e.dim = dim; e.kv_dim = kvd; e.head_size = hs; e.rope = c->rope; e.st = b.st; e.q = b.q;
-        e.kc = b.kc + (size_t)l * max_pos * kvd; e.vc = b.vc + (size_t)l * max_pos * kvd;
-        e.seq_stride = (long)L * max_pos;
-        { BT("epi qkv"); hipLaunchKernelGGL(k_bepi_qkv, dim3(((dim + 2 * kvd) / 2 + 255) / 256, kBatch), dim3(256), 0, s, e); }
         BAttn t{};
-        t.q = b.q; t.kc = e.kc; t.vc = e.vc; t.seq_stride = e.seq_stride; t.out = b.xb; t.st = b.st;
+        t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
+        t.kc = b.kc + (size_t)l * max_pos * kvd; t.vc = b.vc + (size_t)l * max_pos * kvd;
+        t.seq_stride = (long)L * max_pos; t.out = b.xb; t.st = b.st;
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
         const dim3 ag(cf.n_heads, kBatch);
@@ -1744,7 +1740,6 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
         };
         alloc(&b.x, (size_t)kBatch * dim); alloc(&b.xn, (size_t)kBatch * std::max(dim, hidden));
-        alloc(&b.q, (size_t)kBatch * dim);
         alloc(&b.xb, (size_t)kBatch * dim); alloc(&b.hb, (size_t)kBatch * hidden); alloc(&b.logits, (size_t)kBatch * vocab);
         for (int i = 0; i < 3; i++) alloc(&b.part[i], part_floats);
         alloc(&b.kc, cache_floats); alloc(&b.vc, cache_floats);
