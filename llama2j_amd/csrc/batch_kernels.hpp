@@ -31,7 +31,6 @@ struct BGemm {
     int gps;                  // groups of 256 codes per slice
 };
 
-__host__ __device__ inline int bg_row_blocks(int rows, int tiles) { const int per = 16 * tiles * (kBgThreads / 64); return (rows + per - 1) / per; }
 
 __device__ __forceinline__ float code_f(const uint4 &w, int j)
 {
@@ -39,35 +38,50 @@ __device__ __forceinline__ float code_f(const uint4 &w, int j)
     return ubyte_f(d, j & 3);
 }
 
-// Workgroup (x: 128 rows, y: one slice of K): the slice of the sixteen activation vectors is staged in LDS; every
-// wave takes 32 rows (TILES = 2; or 16, TILES = 1, for a matrix too small to fill the GPU otherwise).  A lane (r = lane % 16, s = lane / 16) holds the codes of row r at k = 64 T + 16 s + j (T < 4,
-// j < 16: four 16-byte loads per group and tile); step (T, j) of the MFMA multiplies the 16 rows by the 16 sequences
-// over the four k of the four s.  After the 64 steps of a group the 16 x 16 sums get the group's scale and offset.
+__host__ __device__ inline int bg_units(int rows, int tiles) { return (rows + 16 * tiles - 1) / (16 * tiles); }
+
+// Workgroup (y: one slice of K; x: a share of the rows): the slice of the sixteen activation vectors is staged in LDS once,
+// then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in turn: unit
+// blockIdx.x * 4 + wave, then every gridDim.x * 4-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of row r at
+// k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile); step (T, j) of the MFMA multiplies the 16
+// rows by the 16 sequences over the four k of the four s.  After the 64 steps of a group the 16 x 16 sums get the
+// group's scale and offset.  TILES = 2: two tiles share the activations fetched from LDS.
 template <int TILES>
 __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
 {
     extern __shared__ float xs[];
+    __shared__ float sxs[kBatch][kBgMaxGps];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngroups = a.K >> 8;
     const int g0 = blockIdx.y * a.gps, g1 = min(ngroups, g0 + a.gps), nk = (g1 - g0) << 8;
-    int mi = 0, rb = blockIdx.x;   // which matrix, which of its row blocks
-    while (mi + 1 < a.nmat && rb >= bg_row_blocks(a.rows[mi], TILES)) { rb -= bg_row_blocks(a.rows[mi], TILES); mi++; }
-    const QMat mat = a.m[mi];
-    const int rows = a.rows[mi];
-    float *const part = a.part[mi];
-    constexpr int kRowsWave = 16 * TILES, kRowsWG = kRowsWave * (kBgThreads / 64);
-    const int row0 = min(rb * kRowsWG + wave * kRowsWave, rows - 16);   // (a wave past the end repeats the last tile)
-    const bool live = rb * kRowsWG + wave * kRowsWave < rows;
     const int r = lane & 15, s = lane >> 4;
-    const bool two = TILES == 2 && row0 + 16 < rows;
-    const uint4 *c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
-    const uint4 *c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
-    const float2 *gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
-    const float2 *gs1 = gs0 + (two ? 16L * ngroups : 0L);
-    v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
-    uint4 w0[4], w1[4];   // the first codes are requested before the activations are staged
+    int total = 0;
+    for (int i = 0; i < a.nmat; i++) total += bg_units(a.rows[i], TILES);
+    const int stride = gridDim.x * (kBgThreads / 64);
+    int u = blockIdx.x * (kBgThreads / 64) + wave;
+
+    QMat mat;
+    int rows = 0, row0 = 0;
+    float *part = nullptr;
+    bool two = false;
+    const uint4 *c0 = nullptr, *c1 = nullptr;
+    const float2 *gs0 = nullptr, *gs1 = nullptr;
+    uint4 w0[4], w1[4];
+    auto begin_unit = [&](int unit) {   // where the unit's rows are, and its first group of codes requested
+        int mi = 0;
+        while (mi + 1 < a.nmat && unit >= bg_units(a.rows[mi], TILES)) { unit -= bg_units(a.rows[mi], TILES); mi++; }
+        mat = a.m[mi]; rows = a.rows[mi]; part = a.part[mi];
+        row0 = unit * 16 * TILES;
+        two = TILES == 2 && row0 + 16 < rows;
+        c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
+        c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
+        gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
+        gs1 = gs0 + (two ? 16L * ngroups : 0L);
 #pragma unroll
-    for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
+        for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
+    };
+    if (u < total) begin_unit(u);   // the first codes are requested before the activations are staged
+
     const int pitch = nk + kXPad;   // LDS: sequence-major, xs[b * pitch + k]
     {
         const int nk4 = nk >> 2;   // 16-byte words per sequence in the slice
@@ -80,75 +94,79 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     __syncthreads();
     // sum of every sequence's activations over each group of the slice (for the groups' offsets): 16 threads per sequence,
     // while the first codes are on their way
-    __shared__ float sxs[kBatch][kBgMaxGps];
     {
-        const int b = tid >> 4, part = tid & 15;
+        const int b = tid >> 4, pt = tid & 15;
         for (int gi = 0; gi < g1 - g0; gi++) {
-            const float4 *xp = reinterpret_cast<const float4 *>(xs + b * pitch + (gi << 8) + 16 * part);
+            const float4 *xp = reinterpret_cast<const float4 *>(xs + b * pitch + (gi << 8) + 16 * pt);
             const float4 v0 = xp[0], v1 = xp[1], v2 = xp[2], v3 = xp[3];
             float t = ((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w)) + ((v2.x + v2.y) + (v2.z + v2.w)) +
                       ((v3.x + v3.y) + (v3.z + v3.w));
 #pragma unroll
             for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
-            if (part == 0) sxs[b][gi] = t;
+            if (pt == 0) sxs[b][gi] = t;
         }
     }
     __syncthreads();
-    if (!live) return;
-    for (int g = g0; g < g1; g++) {
-        uint4 u0[4], u1[4];
+    bool first = true;
+    for (; u < total; u += stride) {
+        if (!first) begin_unit(u);
+        first = false;
+        v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
+        for (int g = g0; g < g1; g++) {
+            uint4 u0[4], u1[4];
 #pragma unroll
-        for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
-        if (g + 1 < g1) {   // the next group's codes are requested before this one is multiplied
-            c0 += 16; c1 += 16;
+            for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
+            if (g + 1 < g1) {   // the next group's codes are requested before this one is multiplied
+                c0 += 16; c1 += 16;
 #pragma unroll
-            for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
-        }
-        float2 sc0[4], sc1[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; if (TILES == 2) sc1[i] = gs1[(long)i * ngroups]; }
-        const float sxv = sxs[r][g - g0];   // this lane's column is sequence r
-        v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
-        const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + ((g - g0) << 8) + 16 * s);   // sequence r, k = 64 T + 16 s + j
-        float4 xn[4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) xn[q] = xk[q];
-#pragma unroll
-        for (int T = 0; T < 4; T++) {
-            float4 xc[4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) xc[q] = xn[q];
-            if (T < 3) {   // the activations of the next 16 steps are fetched while these are multiplied
-#pragma unroll
-                for (int q = 0; q < 4; q++) xn[q] = xk[16 * (T + 1) + q];
+                for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
             }
+            float2 sc0[4], sc1[4];
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const float bx[4] = {xc[q].x, xc[q].y, xc[q].z, xc[q].w};
+            for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; if (TILES == 2) sc1[i] = gs1[(long)i * ngroups]; }
+            const float sxv = sxs[r][g - g0];   // this lane's column is sequence r
+            v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
+            const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + ((g - g0) << 8) + 16 * s);   // sequence r, k = 64 T + 16 s + j
+            float4 xn[4];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int j = 4 * q + e;
-                    if (e & 1) {   // two sums per tile: four independent chains of MFMAs
-                        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc2, 0, 0, 0);
-                        if (TILES == 2) acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc3, 0, 0, 0);
-                    } else {
-                        acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc0, 0, 0, 0);
-                        if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc1, 0, 0, 0);
+            for (int q = 0; q < 4; q++) xn[q] = xk[q];
+#pragma unroll
+            for (int T = 0; T < 4; T++) {
+                float4 xc[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) xc[q] = xn[q];
+                if (T < 3) {   // the activations of the next 16 steps are fetched while these are multiplied
+#pragma unroll
+                    for (int q = 0; q < 4; q++) xn[q] = xk[16 * (T + 1) + q];
+                }
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float bx[4] = {xc[q].x, xc[q].y, xc[q].z, xc[q].w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int j = 4 * q + e;
+                        if (e & 1) {   // two sums per tile: independent chains of MFMAs
+                            acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc2, 0, 0, 0);
+                            if (TILES == 2) acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc3, 0, 0, 0);
+                        } else {
+                            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc0, 0, 0, 0);
+                            if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc1, 0, 0, 0);
+                        }
                     }
                 }
             }
-        }
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
-            if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
+            for (int i = 0; i < 4; i++) {
+                y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
+                if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
+            }
+            gs0++; gs1++;
         }
-        gs0++; gs1++;
+        // lane holds rows row0 + 4 s + (0..3) of sequence r
+        float *p = part + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;
+        *reinterpret_cast<v4f32 *>(p) = y0;
+        if (two) *reinterpret_cast<v4f32 *>(p + 16) = y1;
     }
-    // lane holds rows row0 + 4 s + (0..3) of sequence r
-    float *p = part + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;
-    *reinterpret_cast<v4f32 *>(p) = y0;
-    if (two) *reinterpret_cast<v4f32 *>(p + 16) = y1;
 }
 
 // ---- the classifier: fp32 weights (K/MatMul.java:37-60), the same tiling -------------------------------------------

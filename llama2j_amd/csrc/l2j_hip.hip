@@ -1575,7 +1575,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
             BGemm a{};
             a.m[0] = qmat(c, tensor, (uint64_t)layer * rows * K);
             a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
-            const dim3 grid(bg_row_blocks(rows, 2), slices);
+            const dim3 grid((bg_units(rows, 2) + 3) / 4, slices);
             const int n = std::max(1, (int)rounds);
             hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
             (void)hipEventRecord(e0, c->stream);
@@ -1654,13 +1654,23 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
         a.nmat++;
     }
     a.K = K; a.x = x; a.gps = kBatchGps;
-    // 32 rows per wave, or 16 when that leaves more than half of the GPU's workgroup slots (4 per compute unit) empty
-    auto blocks_of = [&](int tiles) { int n = 0; for (int i = 0; i < a.nmat; i++) n += bg_row_blocks(a.rows[i], tiles); return n; };
-    const int tiles = blocks_of(2) * batch_slices(K) * 2 <= 4 * c->n_cu ? 1 : 2;
-    const int blocks = blocks_of(tiles);
+    // All workgroups of the launch are resident at once (4 per compute unit); a wave takes one unit of 16 or 32 rows
+    // after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
+    // activations they fetch from LDS).
+    const int S = batch_slices(K), gmax = std::max(1, 4 * c->n_cu / S);
+    int tiles = 2, gx = 1, best = 1 << 30;
+    for (int t = 2; t >= 1; t--) {
+        int units = 0;
+        for (int i = 0; i < a.nmat; i++) units += bg_units(a.rows[i], t);
+        const int g = std::min(gmax, (units + 3) / 4), iters = (units + 4 * g - 1) / (4 * g);
+        if (iters * t < best) {
+            best = iters * t; tiles = t;
+            gx = (units + 4 * iters - 1) / (4 * iters);   // no more workgroups than that many rounds need
+        }
+    }
     BT(*tensors.begin() == L2J_WQ ? "gemm qkv" : *tensors.begin() == L2J_WO ? "gemm wo" : *tensors.begin() == L2J_W2 ? "gemm w2" : "gemm w1,w3");
-    if (tiles == 1) hipLaunchKernelGGL(k_bgemm<1>, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
-    else hipLaunchKernelGGL(k_bgemm<2>, dim3(blocks, batch_slices(K)), dim3(kBgThreads), batch_lds(), c->stream, a);
+    if (tiles == 1) hipLaunchKernelGGL(k_bgemm<1>, dim3(gx, S), dim3(kBgThreads), batch_lds(), c->stream, a);
+    else hipLaunchKernelGGL(k_bgemm<2>, dim3(gx, S), dim3(kBgThreads), batch_lds(), c->stream, a);
 }
 
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
