@@ -620,7 +620,7 @@ def test_checkpoint_loader_and_quant_caches(orc, tmp_path):
     assert e.value.code == -6
 
 
-# ------------------------------------------------------------------ whole model, BASELINE configs
+# ------------------------------------------------------------------ whole model, the five benchmark configurations
 
 def run_config(orc, name, shape, seed, n_prompt, n_steps, n_logit_steps):
     """Greedy decode on both sides: identical tokens; per-step logits for the first n_logit_steps."""
