@@ -239,8 +239,15 @@ def main():
             g.decode_greedy_batch(prompts, min(bsteps, 8))          # warm
             btoks, bsec = g.decode_greedy_batch(prompts, bsteps)
             n0 = min(bsteps, len(tokens))
+            dim, hidden, L, H, kvH, vocab = shape[:6]
+            kvd = dim // H * kvH
+            macs = 16 * (L * (2 * dim * dim + 2 * dim * kvd + 3 * dim * hidden) + vocab * dim)   # per step: every weight x 16 sequences
             out["batched_decode"] = {"sequences": 16, "steps": bsteps, "tok_s": round(16 * (bsteps - 1) / bsec, 1),
                                      "ms_per_step": round(bsec / (bsteps - 1) * 1e3, 4),
+                                     "roofline": {"bound": "mfma", "achieved": round(2 * macs / (bsec / (bsteps - 1)) / 1e12, 1),
+                                                  "peak": 157.3, "unit": "TFLOP/s",
+                                                  "frac": round(2 * macs / (bsec / (bsteps - 1)) / 1e12 / 157.3, 4),
+                                                  "note": "fp32 matrix cores; whole step, element-wise kernels and attention included in the time"},
                                      "sequence_0_equals_the_single_decode": bool(np.array_equal(btoks[0, :n0], tokens[:n0]))}
         except l2j.L2JError as e:  # shapes the batched path does not take (rows that are not whole groups of 256)
             out["batched_decode"] = {"error": str(e)}
