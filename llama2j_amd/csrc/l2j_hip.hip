@@ -200,8 +200,10 @@ struct l2j_ctx {
     float *pi_prob[2] = {nullptr, nullptr};     // the ProbIndex array, before and after the sort of a call
     int *pi_idx[2] = {nullptr, nullptr};
     int pi_cur = 0;                             // which of the two holds the array between calls
-    void *sort_temp = nullptr;
+    void *sort_temp = nullptr;     // rocPRIM's work space (vocabularies beyond the LDS)
     size_t sort_temp_bytes = 0;
+    float *sort_k[2] = {nullptr, nullptr};   // intermediate runs of the hand-written sort (padded to whole runs of 4096)
+    int *sort_v[2] = {nullptr, nullptr};
     float *sample_exp = nullptr;   // exp(logit / temperature - max) of one sampling step (k_sample_exp)
 };
 
@@ -622,6 +624,10 @@ void free_sampler(l2j_ctx *c)
     }
     (void)hipFree(c->sort_temp);
     c->sort_temp = nullptr;
+    for (int i = 0; i < 2; i++) {
+        (void)hipFree(c->sort_k[i]); (void)hipFree(c->sort_v[i]);
+        c->sort_k[i] = nullptr; c->sort_v[i] = nullptr;
+    }
     (void)hipFree(c->sample_exp);
     c->sample_exp = nullptr;
     if (c->h_ss) (void)hipHostFree(c->h_ss);
@@ -649,6 +655,12 @@ int alloc_sampler(l2j_ctx *c)
     if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n + 4))) return rc;
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
     if (n <= kSampleMaxVocab) {
+        const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+        for (int i = 0; i < 2; i++) {
+            if ((rc = dev_alloc(&c->sort_k[i], (uint64_t)npad))) return rc;
+            if ((rc = dev_alloc(&c->sort_v[i], (uint64_t)npad))) return rc;
+        }
+        HIPCHK(hipFuncSetAttribute((const void *)k_merge_runs, hipFuncAttributeMaxDynamicSharedMemorySize, npad * (int)sizeof(float)));
         const int lds = (int)sampler_lds_bytes(n);
         HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         HIPCHK(hipFuncSetAttribute((const void *)k_topp_pick<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -712,10 +724,20 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     else hipLaunchKernelGGL(k_sample_probs<false>, dim3(1), dim3(1024), 0, c->stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.plain) return e;
-    size_t bytes = c->sort_temp_bytes;
-    int in_second = 0;
-    e = sort_prob_index_desc(c->sort_temp, &bytes, c->pi_prob[cur], c->pi_prob[other], c->pi_idx[cur], c->pi_idx[other],
-                             (unsigned)n, c->stream, &in_second);
+    int in_second = 1;
+    if (in_lds) {   // J/Sampler.java:97 by three counting kernels: tiles, runs of tiles, all runs
+        const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+        hipLaunchKernelGGL(k_sort_tiles, dim3(npad / kSortTile), dim3(kSortTile), 0, c->stream, c->pi_prob[cur], c->pi_idx[cur], n,
+                           c->sort_k[0], c->sort_v[0]);
+        hipLaunchKernelGGL(k_merge_tiles, dim3(npad / kSortRun, 16), dim3(256), 0, c->stream, c->sort_k[0], c->sort_v[0], c->sort_k[1], c->sort_v[1]);
+        hipLaunchKernelGGL(k_merge_runs, dim3(npad / 256), dim3(256), (size_t)npad * sizeof(float), c->stream, c->sort_k[1], c->sort_v[1], n,
+                           npad, c->pi_prob[other], c->pi_idx[other]);
+        e = hipGetLastError();
+    } else {
+        size_t bytes = c->sort_temp_bytes;
+        e = sort_prob_index_desc(c->sort_temp, &bytes, c->pi_prob[cur], c->pi_prob[other], c->pi_idx[cur], c->pi_idx[other],
+                                 (unsigned)n, c->stream, &in_second);
+    }
     if (e != hipSuccess) return e;
     const int sorted = in_second ? other : cur;   // the array stays there until the next call
     a.sorted_prob = c->pi_prob[sorted]; a.sorted_idx = c->pi_idx[sorted];

@@ -13,8 +13,8 @@
 //
 // sample_topp sorts its whole ProbIndex array, not just the candidates of the call: entries of earlier calls
 // stay behind them and take part (J/Sampler.java:92-97).  The array therefore lives in device memory between
-// calls (SampleArgs::cand_*, sorted_*) and is sorted whole by rocPRIM's stable descending sort of (key, value) pairs,
-// which the host launches between the two kernels below.
+// calls (SampleArgs::cand_*, sorted_*) and is sorted whole between the two kernels below: by k_sort_tiles, k_merge_tiles
+// and k_merge_runs when it fits in LDS, else by rocPRIM's stable descending sort of (key, value) pairs.
 #pragma once
 
 #include "kernels.hpp"
@@ -689,6 +689,119 @@ __global__ void __launch_bounds__(1024) k_running_sums(float *x, int n, int scan
             acc = __fadd_rn(acc, sp[i]);
             x[i] = acc;
         }
+    }
+}
+
+// ---- Arrays.sort(probIndex) (J/Sampler.java:97): stable, by descending probability -------------------------------------
+// Three launches, each of which places every pair at its final position within a larger sorted run by counting:
+// the rank of a pair is the number of pairs that come before it, i.e. those with a greater probability plus those with
+// an equal one that stood earlier (compareTo, J/Sampler.java:64-73, only says greater / less / equal; the sort is stable).
+//   k_sort_tiles:   tiles of 256 pairs, every pair compared with the 255 others of its tile;
+//   k_merge_tiles:  runs of 16 sorted tiles (4096 pairs): the rank inside the run = the rank inside the tile + what a
+//                   binary search counts in each of the 15 other tiles (>= for tiles that stood earlier, > for later ones);
+//   k_merge_runs:   the same over the (at most nine) runs, every workgroup holding all keys in LDS.
+// Pairs past n (the array is padded to whole runs) carry the key -1 and sort behind everything.
+constexpr int kSortTile = 256, kSortRun = 4096, kSortTilesPerRun = kSortRun / kSortTile;
+
+// grid: padded n / 256 workgroups of 256 threads
+__global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
+                                                          float *__restrict__ kout, int *__restrict__ vout)
+{
+    __shared__ __align__(16) float keys[kSortTile];
+    const int tid = threadIdx.x, i = blockIdx.x * kSortTile + tid;
+    const float k = i < n ? kin[i] : -1.0f;
+    const int v = i < n ? vin[i] : 0;
+    keys[tid] = k;
+    __syncthreads();
+    int rank = 0;
+#pragma unroll 8
+    for (int j4 = 0; j4 < kSortTile / 4; j4++) {
+        const float4 o = *reinterpret_cast<const float4 *>(&keys[4 * j4]);
+        const int j = 4 * j4;
+        rank += (o.x > k || (o.x == k && j < tid)) + (o.y > k || (o.y == k && j + 1 < tid)) + (o.z > k || (o.z == k && j + 2 < tid)) +
+                (o.w > k || (o.w == k && j + 3 < tid));
+    }
+    kout[blockIdx.x * kSortTile + rank] = k;
+    vout[blockIdx.x * kSortTile + rank] = v;
+}
+
+// grid: (padded n / 4096, 16) workgroups of 256 threads: a workgroup holds the keys of its run in LDS and places a
+// sixteenth of them, one per thread.  The fifteen binary searches of a pair advance together, step by step (their LDS reads are
+// independent: one after the other they cost fifteen times the latency).
+__global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
+                                                     int *__restrict__ vout)
+{
+    __shared__ __align__(16) float keys[kSortRun];
+    const int tid = threadIdx.x, base = blockIdx.x * kSortRun;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        *reinterpret_cast<float4 *>(&keys[4 * (tid + 256 * q)]) = *reinterpret_cast<const float4 *>(kin + base + 4 * (tid + 256 * q));
+    __syncthreads();
+    const int i = blockIdx.y * 256 + tid;
+    const float k = keys[i];
+    const int v = vin[base + i];
+    const int ti = i / kSortTile;
+    int pos[kSortTilesPerRun];
+#pragma unroll
+    for (int tj = 0; tj < kSortTilesPerRun; tj++) pos[tj] = 0;
+#pragma unroll
+    for (int st = kSortTile / 2; st > 0; st >>= 1) {
+#pragma unroll
+        for (int tj = 0; tj < kSortTilesPerRun; tj++) {
+            const float o = keys[tj * kSortTile + pos[tj] + st - 1];
+            pos[tj] += (tj < ti ? o >= k : o > k) ? st : 0;   // tiles that stood earlier win ties
+        }
+    }
+    int rank = i - ti * kSortTile;
+#pragma unroll
+    for (int tj = 0; tj < kSortTilesPerRun; tj++) {
+        const float o = keys[tj * kSortTile + pos[tj]];
+        const int cnt = pos[tj] + ((tj < ti ? o >= k : o > k) ? 1 : 0);
+        rank += tj == ti ? 0 : cnt;
+    }
+    kout[base + rank] = k;
+    vout[base + rank] = v;
+}
+
+constexpr int kSortMaxRuns = (kSampleMaxVocab + kSortRun - 1) / kSortRun;
+
+// grid: padded n / 256 workgroups of 256 threads; dynamic LDS: padded n floats.  Only the first n pairs are written.
+__global__ void __launch_bounds__(256) k_merge_runs(const float *__restrict__ kin, const int *__restrict__ vin, int n, int npad,
+                                                     float *__restrict__ kout, int *__restrict__ vout)
+{
+    extern __shared__ __align__(16) float keys[];
+    const int tid = threadIdx.x;
+#pragma unroll 8
+    for (int i = 4 * tid; i < npad; i += 1024) *reinterpret_cast<float4 *>(keys + i) = *reinterpret_cast<const float4 *>(kin + i);
+    __syncthreads();
+    const int i = blockIdx.x * 256 + tid;
+    const float k = keys[i];
+    const int v = vin[i];
+    const int ri = i / kSortRun, nruns = npad / kSortRun;
+    int pos[kSortMaxRuns];
+#pragma unroll
+    for (int rj = 0; rj < kSortMaxRuns; rj++) pos[rj] = 0;
+#pragma unroll
+    for (int st = kSortRun / 2; st > 0; st >>= 1) {
+#pragma unroll
+        for (int rj = 0; rj < kSortMaxRuns; rj++) {
+            if (rj < nruns) {
+                const float o = keys[rj * kSortRun + pos[rj] + st - 1];
+                pos[rj] += (rj < ri ? o >= k : o > k) ? st : 0;
+            }
+        }
+    }
+    int rank = i - ri * kSortRun;
+#pragma unroll
+    for (int rj = 0; rj < kSortMaxRuns; rj++) {
+        if (rj < nruns && rj != ri) {
+            const float o = keys[rj * kSortRun + pos[rj]];
+            rank += pos[rj] + ((rj < ri ? o >= k : o > k) ? 1 : 0);
+        }
+    }
+    if (rank < n) {
+        kout[rank] = k;
+        vout[rank] = v;
     }
 }
 
