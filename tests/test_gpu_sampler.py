@@ -66,6 +66,23 @@ def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, vo
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
+@pytest.mark.parametrize("vocab", [4097, 32000])
+def test_topp_with_many_equal_probabilities_keeps_the_stable_order(orc, vocab):
+    # logits on a coarse grid: thousands of equal probabilities, inside tiles, across tiles and across runs of the sort,
+    # and among the entries that earlier calls left behind; Arrays.sort is stable, so their order is the array's
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(vocab + 7)
+    g.sampler_seed(3)
+    o = orc.Sampler(3, vocab)
+    for call in range(12):
+        step = float(rng.choice([0.25, 0.5, 1.0]))
+        lg = (np.round(rng.standard_normal(vocab) * 2.0 / step) * step).astype(np.float32)
+        topp = float(rng.choice([0.3, 0.8, 0.95, 0.99]))
+        want, probs = o.step(lg, 1.0, topp)
+        assert g.sample(1.0, topp, logits=lg) == want, (call, step, topp)
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
+
+
 def test_topp_worked_example_with_entries_of_an_earlier_call(orc):
     # the hand-worked case of the oracle's tests, on the device: eight tokens, padded with impossible ones
     vocab = 16
