@@ -6,5 +6,5 @@ out="$here/../libllama2j_hip.so"
 hipcc -O3 -std=c++17 --offload-arch=gfx950 -fPIC -shared \
     -Xclang -target-feature -Xclang -packed-fp32-ops \
     -Wall -Wno-unused-function \
-    -o "$out" "$here/l2j_hip.hip" "$here/sampler_sort.hip" "$here/host_io.cpp" "$here/host_tokenizer.cpp" -lpthread
+    -o "$out" "$here/l2j_hip.hip" "$here/host_io.cpp" "$here/host_tokenizer.cpp" -lpthread
 echo "built $out"

@@ -23,12 +23,6 @@
 
 using namespace l2j;
 
-namespace l2j {
-// stable descending sort of (prob, index) pairs; temp == nullptr: only report the scratch size (sampler_sort.hip)
-hipError_t sort_prob_index_desc(void *temp, size_t *temp_bytes, float *k0, float *k1, int *v0, int *v1, unsigned n, hipStream_t s,
-                                int *in_second);
-}  // namespace l2j
-
 // Device memory of l2j_running_sums_noalloc: the terms and their sums of one call.  Every GPU the library runs on holds
 // its own copy of the array until the process ends; in host code the name is only a handle for hipGetSymbolAddress.
 static __device__ __align__(256) float scratch[kSampleMaxVocab];
@@ -200,9 +194,7 @@ struct l2j_ctx {
     float *pi_prob[2] = {nullptr, nullptr};     // the ProbIndex array, before and after the sort of a call
     int *pi_idx[2] = {nullptr, nullptr};
     int pi_cur = 0;                             // which of the two holds the array between calls
-    void *sort_temp = nullptr;     // rocPRIM's work space (vocabularies beyond the LDS)
-    size_t sort_temp_bytes = 0;
-    float *sort_k[2] = {nullptr, nullptr};   // intermediate runs of the hand-written sort (padded to whole runs of 4096)
+    float *sort_k[2] = {nullptr, nullptr};   // intermediate runs of the sort (padded to whole runs of 4096)
     int *sort_v[2] = {nullptr, nullptr};
     float *sample_exp = nullptr;   // exp(logit / temperature - max) of one sampling step (k_sample_exp)
 };
@@ -622,8 +614,6 @@ void free_sampler(l2j_ctx *c)
         c->pi_prob[i] = nullptr;
         c->pi_idx[i] = nullptr;
     }
-    (void)hipFree(c->sort_temp);
-    c->sort_temp = nullptr;
     for (int i = 0; i < 2; i++) {
         (void)hipFree(c->sort_k[i]); (void)hipFree(c->sort_v[i]);
         c->sort_k[i] = nullptr; c->sort_v[i] = nullptr;
@@ -648,18 +638,14 @@ int alloc_sampler(l2j_ctx *c)
         if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n + 4))) return rc;   // (read in 16-byte words: stage_terms)
         if ((rc = dev_alloc(&c->pi_idx[i], (uint64_t)n))) return rc;
     }
-    size_t bytes = 0;
-    HIPCHK(sort_prob_index_desc(nullptr, &bytes, c->pi_prob[0], c->pi_prob[1], c->pi_idx[0], c->pi_idx[1], (unsigned)n, c->stream, nullptr));
-    c->sort_temp_bytes = bytes;
-    HIPCHK(hipMalloc(&c->sort_temp, std::max<size_t>(bytes, 256)));
     if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n + 4))) return rc;
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
+    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+    for (int i = 0; i < 2; i++) {
+        if ((rc = dev_alloc(&c->sort_k[i], (uint64_t)npad))) return rc;
+        if ((rc = dev_alloc(&c->sort_v[i], (uint64_t)npad))) return rc;
+    }
     if (n <= kSampleMaxVocab) {
-        const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
-        for (int i = 0; i < 2; i++) {
-            if ((rc = dev_alloc(&c->sort_k[i], (uint64_t)npad))) return rc;
-            if ((rc = dev_alloc(&c->sort_v[i], (uint64_t)npad))) return rc;
-        }
         HIPCHK(hipFuncSetAttribute((const void *)k_merge_runs, hipFuncAttributeMaxDynamicSharedMemorySize, npad * (int)sizeof(float)));
         const int lds = (int)sampler_lds_bytes(n);
         HIPCHK(hipFuncSetAttribute((const void *)k_sample_probs<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -724,24 +710,28 @@ hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin,
     else hipLaunchKernelGGL(k_sample_probs<false>, dim3(1), dim3(1024), 0, c->stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.plain) return e;
-    int in_second = 1;
-    if (in_lds) {   // J/Sampler.java:97 by three counting kernels: tiles, runs of tiles, all runs
-        const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
-        hipLaunchKernelGGL(k_sort_tiles, dim3(npad / kSortTile), dim3(kSortTile), 0, c->stream, c->pi_prob[cur], c->pi_idx[cur], n,
-                           c->sort_k[0], c->sort_v[0]);
-        hipLaunchKernelGGL(k_merge_tiles, dim3(npad / kSortRun, 16), dim3(256), 0, c->stream, c->sort_k[0], c->sort_v[0], c->sort_k[1], c->sort_v[1]);
+    // J/Sampler.java:97 by counting kernels: tiles, runs of tiles, then all runs at once (in LDS) or sixteen at a time
+    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+    hipLaunchKernelGGL(k_sort_tiles, dim3(npad / kSortTile), dim3(kSortTile), 0, c->stream, c->pi_prob[cur], c->pi_idx[cur], n,
+                       c->sort_k[0], c->sort_v[0]);
+    hipLaunchKernelGGL(k_merge_tiles, dim3(npad / kSortRun, 16), dim3(256), 0, c->stream, c->sort_k[0], c->sort_v[0], c->sort_k[1], c->sort_v[1]);
+    if (in_lds) {
         hipLaunchKernelGGL(k_merge_runs, dim3(npad / 256), dim3(256), (size_t)npad * sizeof(float), c->stream, c->sort_k[1], c->sort_v[1], n,
                            npad, c->pi_prob[other], c->pi_idx[other]);
-        e = hipGetLastError();
     } else {
-        size_t bytes = c->sort_temp_bytes;
-        e = sort_prob_index_desc(c->sort_temp, &bytes, c->pi_prob[cur], c->pi_prob[other], c->pi_idx[cur], c->pi_idx[other],
-                                 (unsigned)n, c->stream, &in_second);
+        int from = 1;
+        for (long run_len = kSortRun; run_len < npad; run_len *= kSortFanIn, from ^= 1) {
+            const long group_len = run_len * kSortFanIn;
+            const bool last = group_len >= npad;
+            hipLaunchKernelGGL(k_merge_far, dim3(npad / 256), dim3(256), 0, c->stream, c->sort_k[from], c->sort_v[from], npad,
+                               last ? n : npad, (int)run_len, (int)group_len, last ? c->pi_prob[other] : c->sort_k[from ^ 1],
+                               last ? c->pi_idx[other] : c->sort_v[from ^ 1]);
+        }
     }
+    e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int sorted = in_second ? other : cur;   // the array stays there until the next call
-    a.sorted_prob = c->pi_prob[sorted]; a.sorted_idx = c->pi_idx[sorted];
-    c->pi_cur = sorted;
+    a.sorted_prob = c->pi_prob[other]; a.sorted_idx = c->pi_idx[other];   // the array stays there until the next call
+    c->pi_cur = other;
     if (in_lds) hipLaunchKernelGGL(k_topp_pick<true>, dim3(1), dim3(1024), lds, c->stream, a);
     else hipLaunchKernelGGL(k_topp_pick<false>, dim3(1), dim3(1024), 0, c->stream, a);
     return hipGetLastError();

@@ -14,7 +14,7 @@
 // sample_topp sorts its whole ProbIndex array, not just the candidates of the call: entries of earlier calls
 // stay behind them and take part (J/Sampler.java:92-97).  The array therefore lives in device memory between
 // calls (SampleArgs::cand_*, sorted_*) and is sorted whole between the two kernels below: by k_sort_tiles, k_merge_tiles
-// and k_merge_runs when it fits in LDS, else by rocPRIM's stable descending sort of (key, value) pairs.
+// and k_merge_runs when it fits in LDS, else by k_sort_tiles, k_merge_tiles and as many levels of k_merge_far as it takes.
 #pragma once
 
 #include "kernels.hpp"
@@ -699,7 +699,8 @@ __global__ void __launch_bounds__(1024) k_running_sums(float *x, int n, int scan
 //   k_sort_tiles:   tiles of 256 pairs, every pair compared with the 255 others of its tile;
 //   k_merge_tiles:  runs of 16 sorted tiles (4096 pairs): the rank inside the run = the rank inside the tile + what a
 //                   binary search counts in each of the 15 other tiles (>= for tiles that stood earlier, > for later ones);
-//   k_merge_runs:   the same over the (at most nine) runs, every workgroup holding all keys in LDS.
+//   k_merge_runs:   the same over the (at most nine) runs, every workgroup holding all keys in LDS;
+//   k_merge_far:    larger arrays: sixteen runs at a time become one, level by level, the keys read from device memory.
 // Pairs past n (the array is padded to whole runs) carry the key -1 and sort behind everything.
 constexpr int kSortTile = 256, kSortRun = 4096, kSortTilesPerRun = kSortRun / kSortTile;
 
@@ -800,6 +801,50 @@ __global__ void __launch_bounds__(256) k_merge_runs(const float *__restrict__ ki
         }
     }
     if (rank < n) {
+        kout[rank] = k;
+        vout[rank] = v;
+    }
+}
+
+// The same step for arrays that do not fit in LDS: the keys stay in device memory (the caches hold them).  The array
+// consists of sorted runs of run_len pairs; a launch merges every group of group_len / run_len neighbouring runs (at
+// most kSortFanIn) into one run of group_len pairs.  The last run of the array may be shorter.  Pairs whose rank is nout
+// or more are dropped (the padding, at the last level).  The sixteen searches of a pair advance together.
+// grid: padded n / 256 workgroups of 256 threads; run_len and group_len are powers of two, npad a multiple of 256.
+constexpr int kSortFanIn = 16;
+
+__global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
+                                                    int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const float k = kin[i];
+    const int v = vin[i];
+    const int g0 = i & ~(group_len - 1);
+    const int off = i - g0, ri = off / run_len;
+    const int gend = min(npad, g0 + group_len);
+    int rank = g0 + off - ri * run_len;
+    int pos[kSortFanIn], len[kSortFanIn];
+#pragma unroll
+    for (int u = 0; u < kSortFanIn; u++) {
+        len[u] = max(0, min(run_len, gend - g0 - u * run_len));   // 0: no such run in this group
+        pos[u] = 0;
+    }
+    const float *run = kin + g0;
+    for (int st = run_len >> 1; st > 0; st >>= 1) {
+#pragma unroll
+        for (int u = 0; u < kSortFanIn; u++) {
+            const int at = pos[u] + st - 1;
+            const float o = run[min(u * run_len + at, gend - g0 - 1)];
+            pos[u] += (at < len[u] && (u < ri ? o >= k : o > k)) ? st : 0;   // runs that stood earlier win ties
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kSortFanIn; u++) {
+        const float o = run[min(u * run_len + pos[u], gend - g0 - 1)];
+        const int cnt = pos[u] + ((pos[u] < len[u] && (u < ri ? o >= k : o > k)) ? 1 : 0);
+        rank += u != ri ? cnt : 0;
+    }
+    if (rank < nout) {
         kout[rank] = k;
         vout[rank] = v;
     }

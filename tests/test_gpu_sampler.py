@@ -66,7 +66,7 @@ def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, vo
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
-@pytest.mark.parametrize("vocab", [4097, 32000])
+@pytest.mark.parametrize("vocab", [4097, 32000, 70001])
 def test_topp_with_many_equal_probabilities_keeps_the_stable_order(orc, vocab):
     # logits on a coarse grid: thousands of equal probabilities, inside tiles, across tiles and across runs of the sort,
     # and among the entries that earlier calls left behind; Arrays.sort is stable, so their order is the array's
@@ -195,9 +195,10 @@ def test_largest_vocabulary_the_sampler_takes(orc):
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
-@pytest.mark.parametrize("vocab", [36865, 50257, 131072])
+@pytest.mark.parametrize("vocab", [36865, 50257, 70001, 131072])
 def test_vocabularies_beyond_the_lds(orc, vocab):
-    """Above 36864 entries the probabilities stay in device memory; the tokens are still the reference's."""
+    """Above 36864 entries the probabilities stay in device memory and the sort merges sixteen runs at a time (70001: a
+    short last run at the second level; 131072: two full levels); the tokens are still the reference's."""
     g = small_transformer(vocab)
     rng = np.random.default_rng(vocab)
     g.sampler_seed(11)
