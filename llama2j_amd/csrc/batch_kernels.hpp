@@ -1,8 +1,11 @@
 // Several sequences per pass over the weights ("parallel processing of multiple queries", the reference's README
 // wish-list): with sixteen activation vectors per weight matrix the multiply-adds are a 16-wide GEMM and run on the
-// matrix cores.  v_mfma_f32_16x16x4_f32 multiplies and accumulates in fp32, so the arithmetic of the single-sequence
-// path is kept (byte code -> float, fp32 activations, fp32 sums, rm * sum(code * x) + min * sum(x) per group of 256;
-// K/MatMul.java:117-151 is the loop it restates); the vector units only convert the codes.
+// matrix cores.  The arithmetic of the single-sequence path is kept (byte code -> float, fp32 activations, fp32 sums,
+// rm * sum(code * x) + min * sum(x) per group of 256; K/MatMul.java:117-151 is the loop it restates) although the
+// products run on the bf16 cores, sixteen times as fast as the fp32 ones: a code (0..255) is a bf16 exactly, and an
+// fp32 activation is the sum of three bf16 (its 24 significant bits cut into 8 + 8 + 8), so code * x is the sum of
+// three products that v_mfma_f32_16x16x32_bf16 forms exactly and accumulates in fp32.  The vector units only convert
+// the codes.  The fp32 classifier keeps the fp32 cores (v_mfma_f32_16x16x4_f32).
 #pragma once
 
 #include "kernels.hpp"
@@ -10,19 +13,21 @@
 namespace l2j {
 
 constexpr int kBatch = 16;          // sequences per step: the 16 columns of one MFMA
-constexpr int kBgThreads = 256;     // four waves share the staged activations (measured at the 7B shape, ms per step: 64: 7.2, 128: 6.0, 256: 4.8, 512: 5.3, 1024: 6.0)
+constexpr int kBgThreads = 256;     // four waves share the staged activations
 constexpr int kBgRowsPerWave = 32;  // two 16-row tiles share the activations fetched from LDS
 constexpr int kBgRowsPerWG = kBgRowsPerWave * (kBgThreads / 64);
 constexpr int kXPad = 4;            // floats between the slices of two sequences in LDS: a quarter wave's 16-byte reads then cover every bank once
+constexpr int kXPadH = 8;           // the same for the bf16 planes of k_bgemm (16 bytes)
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
 
 // y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].  Up to three matrices that
 // share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
 constexpr int kBgMaxMat = 3;
 constexpr int kBgMaxGps = 16;       // most groups per slice
 struct BGemm {
-    QMat m[kBgMaxMat];        // m.off: the layer's matrix (a multiple of 256), rows of K codes
+    QMat m[kBgMaxMat];        // the tensor's copy in tile order (k_btile), m.off: the layer's matrix (a multiple of 4096)
     int rows[kBgMaxMat];      // rows % 16 == 0
     float *part[kBgMaxMat];   // (slices, kBatch, rows)
     int nmat;
@@ -32,24 +37,64 @@ struct BGemm {
 };
 
 
-__device__ __forceinline__ float code_f(const uint4 &w, int j)
-{
-    const uint32_t d = (j >> 2) == 0 ? w.x : (j >> 2) == 1 ? w.y : (j >> 2) == 2 ? w.z : w.w;
-    return ubyte_f(d, j & 3);
-}
-
 __host__ __device__ inline int bg_units(int rows, int tiles) { return (rows + 16 * tiles - 1) / (16 * tiles); }
 
+// The batched path keeps its own copy of the quantized matrices, in the order its waves read them: the 16 rows x 256
+// codes of a (tile of 16 rows, group) block are 4 KB in a row, [T][lane][16 codes] with lane = r + 16 s holding row r of
+// the tile at k = 64 T + 16 s + j, so that each of a wave's four load instructions per block reads 1 KB in one piece
+// (row by row a wave's instruction touches 16 rows, 64 bytes each: a third slower, measured); the blocks of a tile
+// follow each other group by group, then come those of the next tile.  The scales likewise: 16 (rm, min) per block.
+// One thread per 16 codes of the whole tensor (layers x rows x K); rows % 16 == 0, K % 256 == 0.
+__global__ void __launch_bounds__(256) k_btile(const uint8_t *__restrict__ codes, const float2 *__restrict__ gs, long n16, int rows, int K,
+                                               uint8_t *__restrict__ tcodes, float2 *__restrict__ tgs)
+{
+    const long o = (long)blockIdx.x * 256 + threadIdx.x;   // index of the 16 codes in the tiled copy
+    if (o >= n16) return;
+    const int ngroups = K >> 8;
+    const long per = (long)rows * K >> 4, layer = o / per;
+    const long w = o - layer * per;                         // within the layer's matrix
+    const int block = (int)(w >> 8), in = (int)(w & 255), T = in >> 6, lane = in & 63, r = lane & 15, sq = lane >> 4;
+    const int tile = block / ngroups, g = block - tile * ngroups;
+    const long src = layer * (long)rows * K + (long)(16 * tile + r) * K + (g << 8) + 64 * T + 16 * sq;
+    reinterpret_cast<uint4 *>(tcodes)[o] = *reinterpret_cast<const uint4 *>(codes + src);
+    if (in < 16)   // the block's 16 scales: rows 16 tile + in
+        tgs[(layer * (long)rows * K >> 8) + (long)block * 16 + in] = gs[((layer * (long)rows * K + (long)(16 * tile + in) * K) >> 8) + g];
+}
+
+// LDS of k_bgemm for slices of gps groups: three bf16 planes of (kBatch, gps * 256 + kXPadH)
+__host__ __device__ inline size_t bg_lds_bytes(int gps) { return (size_t)3 * kBatch * (gps * 256 + kXPadH) * sizeof(unsigned short); }
+
+// eight codes (two words of a row) as eight bf16: the upper halves of the codes' floats, two to a register
+__device__ __forceinline__ v8bf16 codes_bf16(uint32_t d0, uint32_t d1)
+{
+    uint4 o;
+    o.x = __builtin_amdgcn_perm(__float_as_uint(ubyte_f(d0, 1)), __float_as_uint(ubyte_f(d0, 0)), 0x07060302u);
+    o.y = __builtin_amdgcn_perm(__float_as_uint(ubyte_f(d0, 3)), __float_as_uint(ubyte_f(d0, 2)), 0x07060302u);
+    o.z = __builtin_amdgcn_perm(__float_as_uint(ubyte_f(d1, 1)), __float_as_uint(ubyte_f(d1, 0)), 0x07060302u);
+    o.w = __builtin_amdgcn_perm(__float_as_uint(ubyte_f(d1, 3)), __float_as_uint(ubyte_f(d1, 2)), 0x07060302u);
+    return __builtin_bit_cast(v8bf16, o);
+}
+
+// x = h[0] + h[1] + h[2] exactly, each the upper half of a float (a bf16): 8 of x's 24 significant bits at a time
+__device__ __forceinline__ void split_bf16(float x, uint32_t h[3])
+{
+    const uint32_t b0 = __float_as_uint(x) & 0xffff0000u;
+    const float r1 = x - __uint_as_float(b0);
+    const uint32_t b1 = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(b1);
+    h[0] = b0 >> 16; h[1] = b1 >> 16; h[2] = __float_as_uint(r2) >> 16;
+}
+
 // Workgroup (y: one slice of K; x: a share of the rows): the slice of the sixteen activation vectors is staged in LDS once,
-// then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in turn: unit
-// blockIdx.x * 4 + wave, then every gridDim.x * 4-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of row r at
-// k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile); step (T, j) of the MFMA multiplies the 16
-// rows by the 16 sequences over the four k of the four s.  After the 64 steps of a group the 16 x 16 sums get the
-// group's scale and offset.  TILES = 2: two tiles share the activations fetched from LDS.
+// as three bf16 planes, then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in turn:
+// unit blockIdx.x * 4 + wave, then every gridDim.x * 4-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of row r
+// at k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile, from the copy in tile order); one MFMA multiplies the 16 rows by the 16
+// sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane.  After the 24 MFMAs of a group
+// the 16 x 16 sums get the group's scale and offset.  TILES = 2: two tiles share the activations fetched from LDS.
 template <int TILES>
 __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
 {
-    extern __shared__ float xs[];
+    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * kBatch + b) * pitch + k]
     __shared__ float sxs[kBatch][kBgMaxGps];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngroups = a.K >> 8;
@@ -60,98 +105,117 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     const int stride = gridDim.x * (kBgThreads / 64);
     int u = blockIdx.x * (kBgThreads / 64) + wave;
 
-    QMat mat;
-    int rows = 0, row0 = 0;
-    float *part = nullptr;
-    bool two = false;
-    const uint4 *c0 = nullptr, *c1 = nullptr;
-    const float2 *gs0 = nullptr, *gs1 = nullptr;
-    uint4 w0[4], w1[4];
-    auto begin_unit = [&](int unit) {   // where the unit's rows are, and its first group of codes requested
+    struct Unit {   // 16 * TILES rows of one matrix: where this lane's codes, scales and results are
+        const uint4 *c0, *c1;
+        const float2 *gs0, *gs1;
+        float *out;
+        bool two;
+    };
+    auto locate = [&](int unit) {
         int mi = 0;
         while (mi + 1 < a.nmat && unit >= bg_units(a.rows[mi], TILES)) { unit -= bg_units(a.rows[mi], TILES); mi++; }
-        mat = a.m[mi]; rows = a.rows[mi]; part = a.part[mi];
-        row0 = unit * 16 * TILES;
-        two = TILES == 2 && row0 + 16 < rows;
-        c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
-        c1 = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(c0) + (two ? 16L * a.K : 0L));
-        gs0 = mat.gs + ((mat.off + (long)(row0 + 4 * s) * a.K) >> 8) + g0;
-        gs1 = gs0 + (two ? 16L * ngroups : 0L);
-#pragma unroll
-        for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
+        const QMat mat = a.m[mi];
+        const int rows = a.rows[mi], row0 = unit * 16 * TILES;
+        Unit n;
+        n.two = TILES == 2 && row0 + 16 < rows;
+        const long block = (long)(row0 >> 4) * ngroups + g0;   // the tile's first block of this slice
+        n.c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (block << 12)) + lane;
+        n.c1 = n.c0 + (n.two ? (long)ngroups << 8 : 0L);   // the next tile: ngroups blocks of 256 16-byte words on
+        n.gs0 = mat.gs + (mat.off >> 8) + (block << 4) + 4 * s;
+        n.gs1 = n.gs0 + (n.two ? (long)ngroups << 4 : 0L);
+        n.out = a.part[mi] + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r
+        return n;
     };
-    if (u < total) begin_unit(u);   // the first codes are requested before the activations are staged
-
-    const int pitch = nk + kXPad;   // LDS: sequence-major, xs[b * pitch + k]
-    {
-        const int nk4 = nk >> 2;   // 16-byte words per sequence in the slice
-#pragma unroll 8
-        for (int f = tid; f < kBatch * nk4; f += kBgThreads) {
-            const int b = f / nk4, k4 = f - b * nk4;
-            *reinterpret_cast<float4 *>(xs + b * pitch + 4 * k4) = *reinterpret_cast<const float4 *>(a.x + (long)b * a.K + (g0 << 8) + 4 * k4);
-        }
-    }
-    __syncthreads();
-    // sum of every sequence's activations over each group of the slice (for the groups' offsets): 16 threads per sequence,
-    // while the first codes are on their way
-    {
-        const int b = tid >> 4, pt = tid & 15;
-        for (int gi = 0; gi < g1 - g0; gi++) {
-            const float4 *xp = reinterpret_cast<const float4 *>(xs + b * pitch + (gi << 8) + 16 * pt);
-            const float4 v0 = xp[0], v1 = xp[1], v2 = xp[2], v3 = xp[3];
-            float t = ((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w)) + ((v2.x + v2.y) + (v2.z + v2.w)) +
-                      ((v3.x + v3.y) + (v3.z + v3.w));
+    uint4 w0[4], w1[4];
+    auto request = [&](const Unit &n) {   // one group of the unit's codes
 #pragma unroll
-            for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
-            if (pt == 0) sxs[b][gi] = t;
+        for (int T = 0; T < 4; T++) { w0[T] = load_stream(n.c0 + 64 * T); if (TILES == 2) w1[T] = load_stream(n.c1 + 64 * T); }
+    };
+    // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
+    // offsets) and their three bf16 parts.  The activations of the first two groups are requested before the wave's
+    // first codes (a wave's loads return in order: behind 8 KB of codes they would arrive with them).
+    const int pitch = nk + kXPadH, plane = kBatch * pitch;
+    const int sb = tid >> 4, pt = tid & 15;
+    const float4 *xsrc = reinterpret_cast<const float4 *>(a.x + (long)sb * a.K + (g0 << 8) + 16 * pt);
+    float4 xa[2][4];
+#pragma unroll
+    for (int gi = 0; gi < 2; gi++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) xa[gi][q] = gi < g1 - g0 ? xsrc[64 * gi + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+    Unit cur{};
+    if (u < total) { cur = locate(u); request(cur); }
+    auto stage = [&](int gi, const float4 (&v)[4]) {
+        float t = ((v[0].x + v[0].y) + (v[0].z + v[0].w)) + ((v[1].x + v[1].y) + (v[1].z + v[1].w)) + ((v[2].x + v[2].y) + (v[2].z + v[2].w)) +
+                  ((v[3].x + v[3].y) + (v[3].z + v[3].w));
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
+        if (pt == 0) sxs[sb][gi] = t;
+        const float xv[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w, v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
+        uint32_t pk[3][8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            uint32_t lo[3], hi[3];
+            split_bf16(xv[2 * e], lo);
+            split_bf16(xv[2 * e + 1], hi);
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) pk[pl][e] = lo[pl] | (hi[pl] << 16);
         }
+        unsigned short *dst = xh + sb * pitch + (gi << 8) + 16 * pt;
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) {
+            reinterpret_cast<uint4 *>(dst + pl * plane)[0] = make_uint4(pk[pl][0], pk[pl][1], pk[pl][2], pk[pl][3]);
+            reinterpret_cast<uint4 *>(dst + pl * plane)[1] = make_uint4(pk[pl][4], pk[pl][5], pk[pl][6], pk[pl][7]);
+        }
+    };
+    stage(0, xa[0]);
+    if (g1 - g0 > 1) stage(1, xa[1]);
+    for (int gi = 2; gi < g1 - g0; gi++) {
+        const float4 v[4] = {xsrc[64 * gi], xsrc[64 * gi + 1], xsrc[64 * gi + 2], xsrc[64 * gi + 3]};
+        stage(gi, v);
     }
     __syncthreads();
-    bool first = true;
     for (; u < total; u += stride) {
-        if (!first) begin_unit(u);
-        first = false;
+        const bool more = u + stride < total;
+        Unit nxt{};
+        if (more) nxt = locate(u + stride);
         v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
         for (int g = g0; g < g1; g++) {
             uint4 u0[4], u1[4];
 #pragma unroll
             for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
-            if (g + 1 < g1) {   // the next group's codes are requested before this one is multiplied
-                c0 += 16; c1 += 16;
-#pragma unroll
-                for (int T = 0; T < 4; T++) { w0[T] = load_stream(c0 + 4 * T); if (TILES == 2) w1[T] = load_stream(c1 + 4 * T); }
+            // the next group's codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
+            if (g + 1 < g1) {
+                cur.c0 += 256; cur.c1 += 256;
+                request(cur);
+            } else if (more) {
+                request(nxt);
             }
-            float2 sc0[4], sc1[4];
+            float2 sc0[4], sc1[4];   // (rm, min) of rows 4 s + (0..3) of the tile
 #pragma unroll
-            for (int i = 0; i < 4; i++) { sc0[i] = gs0[(long)i * ngroups]; if (TILES == 2) sc1[i] = gs1[(long)i * ngroups]; }
+            for (int i = 0; i < 4; i++) { sc0[i] = cur.gs0[i]; if (TILES == 2) sc1[i] = cur.gs1[i]; }
             const float sxv = sxs[r][g - g0];   // this lane's column is sequence r
             v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
-            const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + ((g - g0) << 8) + 16 * s);   // sequence r, k = 64 T + 16 s + j
-            float4 xn[4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) xn[q] = xk[q];
+            const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r, k = 64 T + 16 s + j
 #pragma unroll
             for (int T = 0; T < 4; T++) {
-                float4 xc[4];
+                v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
 #pragma unroll
-                for (int q = 0; q < 4; q++) xc[q] = xn[q];
-                if (T < 3) {   // the activations of the next 16 steps are fetched while these are multiplied
-#pragma unroll
-                    for (int q = 0; q < 4; q++) xn[q] = xk[16 * (T + 1) + q];
+                for (int pl = 0; pl < 3; pl++) {
+                    bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + 64 * T);
+                    bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + 64 * T + 8);
                 }
+                const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const float bx[4] = {xc[q].x, xc[q].y, xc[q].z, xc[q].w};
+                for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
+                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0, 0, 0, 0);
+                    acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2, 0, 0, 0);
+                }
+                if (TILES == 2) {
+                    const v8bf16 a10 = codes_bf16(u1[T].x, u1[T].y), a11 = codes_bf16(u1[T].z, u1[T].w);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int j = 4 * q + e;
-                        if (e & 1) {   // two sums per tile: independent chains of MFMAs
-                            acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc2, 0, 0, 0);
-                            if (TILES == 2) acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc3, 0, 0, 0);
-                        } else {
-                            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u0[T], j), bx[e], acc0, 0, 0, 0);
-                            if (TILES == 2) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(code_f(u1[T], j), bx[e], acc1, 0, 0, 0);
-                        }
+                    for (int pl = 2; pl >= 0; pl--) {
+                        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1, 0, 0, 0);
+                        acc3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3, 0, 0, 0);
                     }
                 }
             }
@@ -160,12 +224,11 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
                 y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
                 if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
             }
-            gs0++; gs1++;
+            cur.gs0 += 16; cur.gs1 += 16;
         }
-        // lane holds rows row0 + 4 s + (0..3) of sequence r
-        float *p = part + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;
-        *reinterpret_cast<v4f32 *>(p) = y0;
-        if (two) *reinterpret_cast<v4f32 *>(p + 16) = y1;
+        *reinterpret_cast<v4f32 *>(cur.out) = y0;
+        if (cur.two) *reinterpret_cast<v4f32 *>(cur.out + 16) = y1;
+        cur = nxt;
     }
 }
 

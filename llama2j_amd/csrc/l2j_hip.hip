@@ -133,6 +133,9 @@ struct l2j_ctx {
     bool finalized = false;
 
     QTensor qt[L2J_TENSOR_COUNT];
+    uint8_t *bt_codes[L2J_TENSOR_COUNT] = {};   // the batched path's copy of the matrices in tile order (k_btile), made by its first call
+    float2 *bt_gs[L2J_TENSOR_COUNT] = {};
+    bool bt_ready = false;
     float *emb = nullptr, *wcls = nullptr;
     bool emb_loaded = false, wcls_loaded = false;
 
@@ -1024,6 +1027,8 @@ void l2j_destroy(l2j_ctx *c)
         (void)hipFree(c->qt[t].codes);
         (void)hipFree(c->qt[t].gs);
         (void)hipFree(c->qt[t].mm);
+        (void)hipFree(c->bt_codes[t]);
+        (void)hipFree(c->bt_gs[t]);
     }
     if (c->wcls != c->emb) (void)hipFree(c->wcls);
     (void)hipFree(c->emb);
@@ -1552,6 +1557,34 @@ static bool matrix_shape(const l2j_config &cf, int tensor, int *rows, int *K)
     }
 }
 
+// The tile-ordered copy of `tensor` for the batched path (rows % 16 == 0 and K % 256 == 0 checked by the caller).
+static int ensure_batch_tiles(l2j_ctx *c, int tensor)
+{
+    if (c->bt_codes[tensor] && c->bt_gs[tensor]) return L2J_OK;
+    int rows = 0, K = 0;
+    if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
+    const QTensor &t = c->qt[tensor];
+    if (t.groups_loaded != t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
+    const uint64_t n = (uint64_t)c->cfg.n_layers * rows * K;
+    int rc;
+    if (!c->bt_codes[tensor] && (rc = dev_alloc(&c->bt_codes[tensor], n))) return rc;
+    if (!c->bt_gs[tensor] && (rc = dev_alloc(&c->bt_gs[tensor], n / 256))) return rc;
+    const long n16 = (long)(n / 16);
+    hipLaunchKernelGGL(k_btile, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, c->stream, t.codes, t.gs, n16, rows, K, c->bt_codes[tensor],
+                       c->bt_gs[tensor]);
+    HIPCHK(hipGetLastError());
+    return L2J_OK;
+}
+
+static QMat bqmat(const l2j_ctx *c, int t, uint64_t off)
+{
+    QMat m;
+    m.codes = c->bt_codes[t];
+    m.gs = c->bt_gs[t];
+    m.off = (long)off;
+    return m;
+}
+
 int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y, int32_t groups_per_slice, int32_t rounds,
                      double *mean_us)
 {
@@ -1566,9 +1599,11 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (t.groups_loaded != t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
         const int ngroups = K / 256, gps = std::max(1, std::min(std::min(ngroups, kBgMaxGps), (int)groups_per_slice));
         const int slices = (ngroups + gps - 1) / gps;
-        const size_t lds = (size_t)kBatch * (gps * 256 + kXPad) * sizeof(float);
-        if (lds > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
+        const size_t lds = bg_lds_bytes(gps);
+        if (lds + sizeof(float) * kBatch * kBgMaxGps > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
         HIPCHK(hipSetDevice(c->cfg.device));
+        int trc = ensure_batch_tiles(c, tensor);
+        if (trc) return trc;
         float *dx = nullptr, *dpart = nullptr, *dy = nullptr;
         hipEvent_t e0 = nullptr, e1 = nullptr;
         auto release = [&]() {
@@ -1585,7 +1620,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             BGemm a{};
-            a.m[0] = qmat(c, tensor, (uint64_t)layer * rows * K);
+            a.m[0] = bqmat(c, tensor, (uint64_t)layer * rows * K);
             a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
             const dim3 grid((bg_units(rows, 2) + 3) / 4, slices);
             const int n = std::max(1, (int)rounds);
@@ -1651,7 +1686,10 @@ struct BtScope {
 constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
 
 int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
-size_t batch_lds() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }
+size_t batch_lds() { return bg_lds_bytes(kBatchGps); }   // k_bgemm: bf16 planes
+size_t batch_lds_f32() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
+// workgroups of k_bgemm a compute unit holds at once: its 160 KB of LDS, and at most three by their registers
+int batch_resident() { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds() + sizeof(float) * kBatch * kBgMaxGps)))); }
 
 // The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
 void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part)
@@ -1661,15 +1699,15 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
     for (int tensor : tensors) {
         int rows = 0;
         matrix_shape(c->cfg, tensor, &rows, &K);
-        a.m[a.nmat] = qmat(c, tensor, (uint64_t)layer * rows * K);
+        a.m[a.nmat] = bqmat(c, tensor, (uint64_t)layer * rows * K);
         a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
         a.nmat++;
     }
     a.K = K; a.x = x; a.gps = kBatchGps;
-    // All workgroups of the launch are resident at once (4 per compute unit); a wave takes one unit of 16 or 32 rows
+    // All workgroups of the launch are resident at once (batch_resident() per compute unit); a wave takes one unit of 16 or 32 rows
     // after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
     // activations they fetch from LDS).
-    const int S = batch_slices(K), gmax = std::max(1, 4 * c->n_cu / S);
+    const int S = batch_slices(K), gmax = std::max(1, batch_resident() * c->n_cu / S);
     int tiles = 2, gx = 1, best = 1 << 30;
     for (int t = 2; t >= 1; t--) {
         int units = 0;
@@ -1721,7 +1759,7 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
     }
     BGemmF32 g{};
     g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
-    { BT("classifier"); hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds(), s, g); }
+    { BT("classifier"); hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds_f32(), s, g); }
     BNext n{};
     n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
     n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
@@ -1750,6 +1788,13 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
                     return fail(L2J_E_ARG, "prompt id out of range");
         }
         HIPCHK(hipSetDevice(cf.device));
+        if (!c->bt_ready) {   // the matrices once more, in the order the batched products read them
+            for (int t : {L2J_WQ, L2J_WK, L2J_WV, L2J_WO, L2J_W1, L2J_W2, L2J_W3}) {
+                const int trc = ensure_batch_tiles(c, t);
+                if (trc) return trc;
+            }
+            c->bt_ready = true;
+        }
         const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, kvd = c->kv_dim, vocab = cf.vocab_size;
         const int sd = batch_slices(dim), sh = batch_slices(hidden);
         const size_t part_floats = (size_t)kBatch * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
@@ -1781,7 +1826,7 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream) != hipSuccess ||
             hipFuncSetAttribute((const void *)k_bgemm<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
             hipFuncSetAttribute((const void *)k_bgemm<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
-            hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32()) != hipSuccess ||
             hipStreamSynchronize(c->stream) != hipSuccess)
             return done(fail(L2J_E_HIP, "batched decode: set-up failed"));
         // one position as a graph: every kernel reads the position and the tokens from device memory ("graph" = 0: the

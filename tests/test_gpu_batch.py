@@ -39,7 +39,7 @@ def test_matrix_core_product_matches_float64():
     for tensor, rows, K in ((TENSOR.WQ, 1024, 1024), (TENSOR.WK, kvd, 1024), (TENSOR.W1, 2816, 1024), (TENSOR.W2, 1024, 2816)):
         x = (rng.standard_normal((16, K)) * np.exp(rng.uniform(-3, 3, (16, 1)))).astype(np.float32)
         want = x.astype(np.float64) @ dequantized(g, tensor, 1, rows, K).T
-        for gps in (1, 2, 3, 8):
+        for gps in (1, 2, 3, 6):
             got, _ = g.batch_matmul(tensor, 1, x, rows, groups_per_slice=gps)
             err = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)      # per sequence
             assert err.max() < 5e-6, (int(tensor), gps, float(err.max()))
