@@ -135,18 +135,21 @@ int l2j_forward_taps(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_
 int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps,
                       int32_t *out_tokens, int32_t *n_out, double *seconds);
 
-/* Sixteen sequences at once, every weight read once per step for all of them (the reference has no counterpart:
- * "parallel processing of multiple queries" is on its wish-list, README.md:347).  Every sequence runs the token loop
- * of l2j_decode_greedy (BOS first, its own prompt ids forced, first-maximum argmax afterwards) for exactly `steps`
- * positions; a sequence that emits token 1 keeps running and the caller cuts it there.  prompts: 16 rows of
- * prompt_stride ids, n_prompt[b] of them used; out_tokens: 16 rows of `steps` ids.  The matrix products run on the
- * matrix cores in fp32 (fp32 activations and sums as in K/MatMul.java:117-151; sums are formed in another order
- * than in the single-sequence path, so logits agree to rounding, not bit for bit).  The call allocates its own
- * activation buffers and a KV cache of 16 x steps rows per layer and frees them when it returns; the context's
- * cache is not touched.  Needs dim and hidden_dim in whole groups of 256 and head_size 64, 128 or 256.
+/* Sixteen or thirty-two sequences at once (n_seq), every weight read once per step for all of them (the reference has
+ * no counterpart: "parallel processing of multiple queries" is on its wish-list, README.md:347).  Every sequence runs
+ * the token loop of l2j_decode_greedy (BOS first, its own prompt ids forced, first-maximum argmax afterwards) for
+ * exactly `steps` positions; a sequence that emits token 1 keeps running and the caller cuts it there.  prompts: n_seq
+ * rows of prompt_stride ids, n_prompt[b] of them used; out_tokens: n_seq rows of `steps` ids.  The products of the
+ * quantized matrices run on the bf16 matrix cores with the arithmetic of K/MatMul.java:117-151 kept: a code is a bf16
+ * exactly, an fp32 activation is cut exactly into three bf16, the products are exact and the sums fp32 (the fp32
+ * classifier runs on the fp32 matrix cores); sums are formed in another order than in the single-sequence path, so
+ * logits agree to rounding, not bit for bit.  The first call makes a second copy of the quantized matrices on the
+ * device, in the order this path reads them (freed by l2j_destroy); every call allocates its own activation buffers
+ * and a KV cache of n_seq x steps rows per layer and frees them when it returns; the context's cache is not touched.
+ * Needs dim and hidden_dim in whole groups of 256 and head_size 64, 128 or 256.
  * *seconds (may be NULL): GPU time from the end of the first step to the end of the last. */
-int l2j_decode_greedy_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t prompt_stride,
-                            int32_t steps, int32_t *out_tokens, double *seconds);
+int l2j_decode_greedy_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,
+                            int32_t prompt_stride, int32_t steps, int32_t *out_tokens, double *seconds);
 
 /* ---- sampling on the device: J/Sampler.java and the sampling branch of J/Run.java:643-665 ----
  * The context holds one sampler = the reference's Sampler object: a java.util.Random and the ProbIndex

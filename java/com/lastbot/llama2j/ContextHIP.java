@@ -61,7 +61,7 @@ public final class ContextHIP implements AutoCloseable {
         decodeGreedy = handle("l2j_decode_greedy",
                 FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS));
         decodeGreedyBatch = handle("l2j_decode_greedy_batch",
-                FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
+                FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
         decodeSample = handle("l2j_decode_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
                 JAVA_FLOAT, JAVA_FLOAT, JAVA_LONG, ADDRESS, ADDRESS, ADDRESS));
         samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
@@ -231,13 +231,14 @@ public final class ContextHIP implements AutoCloseable {
     }
 
     /**
-     * Sixteen greedy token loops at once (l2j_decode_greedy_batch): every weight is read once per step for all of them.
-     * prompts: at most sixteen id arrays (missing ones run without a prompt); result[b] holds `steps` tokens of
-     * sequence b, which runs on after token 1: cut it there.  No counterpart in the reference.
+     * Sixteen or thirty-two greedy token loops at once (l2j_decode_greedy_batch): every weight is read once per step for
+     * all of them.  prompts: at most 32 id arrays (16 sequences run for up to sixteen prompts, else 32; missing ones run
+     * without a prompt); result[b] holds `steps` tokens of sequence b, which runs on after token 1: cut it there.  No
+     * counterpart in the reference.
      */
     public int[][] decodeGreedyBatch(int[][] prompts, int steps) {
-        final int batch = 16;
-        if (prompts.length > batch) throw new IllegalArgumentException("at most 16 sequences");
+        if (prompts.length > 32) throw new IllegalArgumentException("at most 32 sequences");
+        final int batch = prompts.length <= 16 ? 16 : 32;
         int stride = 1;
         for (int[] p : prompts) stride = Math.max(stride, p.length);
         try (Arena a = Arena.ofConfined()) {
@@ -248,7 +249,7 @@ public final class ContextHIP implements AutoCloseable {
                 MemorySegment.copy(prompts[b], 0, ids, JAVA_INT, (long) b * stride * Integer.BYTES, prompts[b].length);
                 counts.setAtIndex(JAVA_INT, b, prompts[b].length);
             }
-            check(call(decodeGreedyBatch, ctx, ids, counts, stride, steps, out, secondsSeg));
+            check(call(decodeGreedyBatch, ctx, ids, counts, batch, stride, steps, out, secondsSeg));
             int[][] tokens = new int[batch][steps];
             for (int b = 0; b < batch; b++) MemorySegment.copy(out, JAVA_INT, (long) b * steps * Integer.BYTES, tokens[b], 0, steps);
             return tokens;

@@ -114,7 +114,7 @@ def _signatures():
         "l2j_sync": (C.c_int, [vp]),
         "l2j_time_kernel": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
-        "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
+        "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
         "l2j_batch_matmul": (C.c_int, [vp, C.c_int, C.c_int, fp, fp, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
         "l2j_bytes_per_token": (C.c_uint64, [cfgp, C.c_int32]),
         "l2j_quant_nbytes": (C.c_uint64, [C.c_uint64]),
@@ -420,19 +420,22 @@ class Transformer:
         self._check(lib().l2j_running_sums_noalloc(self._h, _fp(terms), terms.size, _fp(out)))
         return out
 
-    def decode_greedy_batch(self, prompts, steps):
-        """Sixteen greedy token loops at once (l2j_decode_greedy_batch).  prompts: up to sixteen id sequences (missing
-        ones run without a prompt); returns (tokens of shape (16, steps), seconds after the first step)."""
-        assert len(prompts) <= 16
+    def decode_greedy_batch(self, prompts, steps, n_seq=None):
+        """Sixteen or thirty-two greedy token loops at once (l2j_decode_greedy_batch).  prompts: up to n_seq id sequences
+        (missing ones run without a prompt; n_seq defaults to 16, or 32 for more than sixteen prompts); returns (tokens of
+        shape (n_seq, steps), seconds after the first step)."""
+        if n_seq is None:
+            n_seq = 16 if len(prompts) <= 16 else 32
+        assert len(prompts) <= n_seq
         stride = max([len(p) for p in prompts] + [1])
-        ids = np.zeros((16, stride), dtype=np.int32)
-        n = np.zeros(16, dtype=np.int32)
+        ids = np.zeros((n_seq, stride), dtype=np.int32)
+        n = np.zeros(n_seq, dtype=np.int32)
         for b, p in enumerate(prompts):
             ids[b, :len(p)] = p
             n[b] = len(p)
-        out = np.zeros((16, steps), dtype=np.int32)
+        out = np.zeros((n_seq, steps), dtype=np.int32)
         sec = C.c_double(0.0)
-        self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), stride, steps, _i32(out), C.byref(sec)))
+        self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), C.byref(sec)))
         return out, sec.value
 
     def batch_matmul(self, tensor, layer, x, rows, groups_per_slice=2, rounds=1):

@@ -12,8 +12,9 @@
 
 namespace l2j {
 
-constexpr int kBatch = 16;          // sequences per step: the 16 columns of one MFMA
-constexpr int kBgThreads = 256;     // four waves share the staged activations
+constexpr int kBatch = 16;          // sequences per column block: the 16 columns of one MFMA
+constexpr int kMaxBatch = 32;       // sequences per step: one or two column blocks
+constexpr int kBgThreads = 256;     // threads per column block: four waves per 16 sequences share the staged activations
 constexpr int kBgRowsPerWave = 32;  // two 16-row tiles share the activations fetched from LDS
 constexpr int kBgRowsPerWG = kBgRowsPerWave * (kBgThreads / 64);
 constexpr int kXPad = 4;            // floats between the slices of two sequences in LDS: a quarter wave's 16-byte reads then cover every bank once
@@ -29,10 +30,10 @@ constexpr int kBgMaxGps = 16;       // most groups per slice
 struct BGemm {
     QMat m[kBgMaxMat];        // the tensor's copy in tile order (k_btile), m.off: the layer's matrix (a multiple of 4096)
     int rows[kBgMaxMat];      // rows % 16 == 0
-    float *part[kBgMaxMat];   // (slices, kBatch, rows)
+    float *part[kBgMaxMat];   // (slices, nseq, rows)
     int nmat;
     int K;                    // K % 256 == 0
-    const float *x;           // (kBatch, K)
+    const float *x;           // (nseq, K)
     int gps;                  // groups of 256 codes per slice
 };
 
@@ -61,8 +62,8 @@ __global__ void __launch_bounds__(256) k_btile(const uint8_t *__restrict__ codes
         tgs[(layer * (long)rows * K >> 8) + (long)block * 16 + in] = gs[((layer * (long)rows * K + (long)(16 * tile + in) * K) >> 8) + g];
 }
 
-// LDS of k_bgemm for slices of gps groups: three bf16 planes of (kBatch, gps * 256 + kXPadH)
-__host__ __device__ inline size_t bg_lds_bytes(int gps) { return (size_t)3 * kBatch * (gps * 256 + kXPadH) * sizeof(unsigned short); }
+// LDS of k_bgemm for slices of gps groups: three bf16 planes of (nseq, gps * 256 + kXPadH)
+__host__ __device__ inline size_t bg_lds_bytes(int gps, int nseq) { return (size_t)3 * nseq * (gps * 256 + kXPadH) * sizeof(unsigned short); }
 
 // eight codes (two words of a row) as eight bf16: the upper halves of the codes' floats, two to a register
 __device__ __forceinline__ v8bf16 codes_bf16(uint32_t d0, uint32_t d1)
@@ -85,30 +86,33 @@ __device__ __forceinline__ void split_bf16(float x, uint32_t h[3])
     h[0] = b0 >> 16; h[1] = b1 >> 16; h[2] = __float_as_uint(r2) >> 16;
 }
 
-// Workgroup (y: one slice of K; x: a share of the rows): the slice of the sixteen activation vectors is staged in LDS once,
+// Workgroup (y: one slice of K; x: a share of the rows): the slice of the 16 NB activation vectors is staged in LDS once,
 // as three bf16 planes, then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in turn:
-// unit blockIdx.x * 4 + wave, then every gridDim.x * 4-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of row r
-// at k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile, from the copy in tile order); one MFMA multiplies the 16 rows by the 16
-// sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane.  After the 24 MFMAs of a group
-// the 16 x 16 sums get the group's scale and offset.  TILES = 2: two tiles share the activations fetched from LDS.
-template <int TILES>
-__global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
+// unit blockIdx.x * 4 NB + wave, then every gridDim.x * 4 NB-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of
+// row r at k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile, from the copy in tile order); one MFMA
+// multiplies the 16 rows by 16 sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane and
+// column block.  After the 24 NB MFMAs of a group the 16 x 16 sums get the group's scale and offset.  TILES = 2: two
+// tiles share the activations fetched from LDS; NB = 2: two column blocks share the converted codes.  256 NB threads.
+template <int TILES, int NB>
+__global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
 {
-    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * kBatch + b) * pitch + k]
-    __shared__ float sxs[kBatch][kBgMaxGps];
+    constexpr int NSEQ = kBatch * NB, WAVES = 4 * NB;
+    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * NSEQ + b) * pitch + k]
+    __shared__ float sxs[NSEQ][kBgMaxGps];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngroups = a.K >> 8;
     const int g0 = blockIdx.y * a.gps, g1 = min(ngroups, g0 + a.gps), nk = (g1 - g0) << 8;
     const int r = lane & 15, s = lane >> 4;
     int total = 0;
     for (int i = 0; i < a.nmat; i++) total += bg_units(a.rows[i], TILES);
-    const int stride = gridDim.x * (kBgThreads / 64);
-    int u = blockIdx.x * (kBgThreads / 64) + wave;
+    const int stride = gridDim.x * WAVES;
+    int u = blockIdx.x * WAVES + wave;
 
     struct Unit {   // 16 * TILES rows of one matrix: where this lane's codes, scales and results are
         const uint4 *c0, *c1;
         const float2 *gs0, *gs1;
         float *out;
+        int rows;
         bool two;
     };
     auto locate = [&](int unit) {
@@ -117,13 +121,14 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         const QMat mat = a.m[mi];
         const int rows = a.rows[mi], row0 = unit * 16 * TILES;
         Unit n;
+        n.rows = rows;
         n.two = TILES == 2 && row0 + 16 < rows;
         const long block = (long)(row0 >> 4) * ngroups + g0;   // the tile's first block of this slice
         n.c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (block << 12)) + lane;
         n.c1 = n.c0 + (n.two ? (long)ngroups << 8 : 0L);   // the next tile: ngroups blocks of 256 16-byte words on
         n.gs0 = mat.gs + (mat.off >> 8) + (block << 4) + 4 * s;
         n.gs1 = n.gs0 + (n.two ? (long)ngroups << 4 : 0L);
-        n.out = a.part[mi] + ((long)blockIdx.y * kBatch + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r
+        n.out = a.part[mi] + ((long)blockIdx.y * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
         return n;
     };
     uint4 w0[4], w1[4];
@@ -134,7 +139,7 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
     // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
     // offsets) and their three bf16 parts.  The activations of the first two groups are requested before the wave's
     // first codes (a wave's loads return in order: behind 8 KB of codes they would arrive with them).
-    const int pitch = nk + kXPadH, plane = kBatch * pitch;
+    const int pitch = nk + kXPadH, plane = NSEQ * pitch;
     const int sb = tid >> 4, pt = tid & 15;
     const float4 *xsrc = reinterpret_cast<const float4 *>(a.x + (long)sb * a.K + (g0 << 8) + 16 * pt);
     float4 xa[2][4];
@@ -178,7 +183,9 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
         const bool more = u + stride < total;
         Unit nxt{};
         if (more) nxt = locate(u + stride);
-        v4f32 y0 = {0.f, 0.f, 0.f, 0.f}, y1 = {0.f, 0.f, 0.f, 0.f};
+        v4f32 y0[NB], y1[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) y0[nb] = y1[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
         for (int g = g0; g < g1; g++) {
             uint4 u0[4], u1[4];
 #pragma unroll
@@ -193,41 +200,51 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
             float2 sc0[4], sc1[4];   // (rm, min) of rows 4 s + (0..3) of the tile
 #pragma unroll
             for (int i = 0; i < 4; i++) { sc0[i] = cur.gs0[i]; if (TILES == 2) sc1[i] = cur.gs1[i]; }
-            const float sxv = sxs[r][g - g0];   // this lane's column is sequence r
-            v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
-            const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r, k = 64 T + 16 s + j
+            v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
+            const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
 #pragma unroll
             for (int T = 0; T < 4; T++) {
-                v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
-#pragma unroll
-                for (int pl = 0; pl < 3; pl++) {
-                    bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + 64 * T);
-                    bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + 64 * T + 8);
-                }
                 const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
+                v8bf16 a10 = a00, a11 = a01;
+                if (TILES == 2) { a10 = codes_bf16(u1[T].x, u1[T].y); a11 = codes_bf16(u1[T].z, u1[T].w); }
 #pragma unroll
-                for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0, 0, 0, 0);
-                    acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2, 0, 0, 0);
-                }
-                if (TILES == 2) {
-                    const v8bf16 a10 = codes_bf16(u1[T].x, u1[T].y), a11 = codes_bf16(u1[T].z, u1[T].w);
+                for (int nb = 0; nb < NB; nb++) {
+                    v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
 #pragma unroll
-                    for (int pl = 2; pl >= 0; pl--) {
-                        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1, 0, 0, 0);
-                        acc3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3, 0, 0, 0);
+                    for (int pl = 0; pl < 3; pl++) {
+                        bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
+                        bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
+                    }
+#pragma unroll
+                    for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
+                        acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0[nb], 0, 0, 0);
+                        acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2[nb], 0, 0, 0);
+                        if (TILES == 2) {
+                            acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1[nb], 0, 0, 0);
+                            acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3[nb], 0, 0, 0);
+                        }
                     }
                 }
             }
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                y0[i] += fmaf(sc0[i].x, acc0[i] + acc2[i], sc0[i].y * sxv);
-                if (TILES == 2) y1[i] += fmaf(sc1[i].x, acc1[i] + acc3[i], sc1[i].y * sxv);
+            for (int nb = 0; nb < NB; nb++) {
+                const float sxv = sxs[16 * nb + r][g - g0];   // this lane's column is sequence 16 nb + r
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    y0[nb][i] += fmaf(sc0[i].x, acc0[nb][i] + acc2[nb][i], sc0[i].y * sxv);
+                    if (TILES == 2) y1[nb][i] += fmaf(sc1[i].x, acc1[nb][i] + acc3[nb][i], sc1[i].y * sxv);
+                }
             }
             cur.gs0 += 16; cur.gs1 += 16;
         }
-        *reinterpret_cast<v4f32 *>(cur.out) = y0;
-        if (cur.two) *reinterpret_cast<v4f32 *>(cur.out + 16) = y1;
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+            float *o = cur.out + (long)nb * 16 * cur.rows;
+            *reinterpret_cast<v4f32 *>(o) = y0[nb];
+            if (cur.two) *reinterpret_cast<v4f32 *>(o + 16) = y1[nb];
+        }
         cur = nxt;
     }
 }
@@ -237,14 +254,19 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm(const BGemm a)
 struct BGemmF32 {
     const float *w;    // (rows, K) fp32
     int rows, K;       // rows % 16 == 0, K % 256 == 0
-    const float *x;    // (kBatch, K)
-    float *part;       // (slices, kBatch, rows)
+    const float *x;    // (nseq, K)
+    float *part;       // (slices, nseq, rows)
     int gps;
 };
 
-// As k_bgemm with float weights: a lane (r, s) holds row r at k = 64 T + 16 s + j as four 16-byte loads per block of 64 k.
+// As k_bgemm with float weights on the fp32 matrix cores (v_mfma_f32_16x16x4_f32), rows as they lie in memory: a lane
+// (r, s) holds row r at k = 64 T + 16 q + 4 s + e as four 16-byte loads (q) per block of 64 k, so that the four lanes of a
+// row read 64 bytes in one piece per load; step (q, e) multiplies the 16 rows by 16 sequences over the four k of the four s.
+// NB = 2: two column blocks of 16 sequences share the weights.  256 threads, 32 rows per wave.
+template <int NB>
 __global__ void __launch_bounds__(kBgThreads) k_bgemm_f32(const BGemmF32 a)
 {
+    constexpr int NSEQ = kBatch * NB;
     extern __shared__ float xs[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int ngroups = a.K >> 8;
@@ -253,53 +275,64 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm_f32(const BGemmF32 a)
     const bool live = blockIdx.x * kBgRowsPerWG + wave * kBgRowsPerWave < a.rows;
     const int r = lane & 15, s = lane >> 4;
     const bool two = row0 + 16 < a.rows;
-    const float4 *c0 = reinterpret_cast<const float4 *>(a.w + (long)(row0 + r) * a.K + (g0 << 8) + 16 * s);
+    const float4 *c0 = reinterpret_cast<const float4 *>(a.w + (long)(row0 + r) * a.K + (g0 << 8) + 4 * s);
     const float4 *c1 = c0 + (two ? 4L * a.K : 0L);   // 16 rows on, in 16-byte words
     float4 w0[4], w1[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) { w0[q] = load_stream(c0 + q); w1[q] = load_stream(c1 + q); }
+    for (int q = 0; q < 4; q++) { w0[q] = load_stream(c0 + 4 * q); w1[q] = load_stream(c1 + 4 * q); }
     const int pitch = nk + kXPad;
     {
         const int nk4 = nk >> 2;
 #pragma unroll 8
-        for (int f = tid; f < kBatch * nk4; f += kBgThreads) {
+        for (int f = tid; f < NSEQ * nk4; f += kBgThreads) {
             const int b = f / nk4, k4 = f - b * nk4;
             *reinterpret_cast<float4 *>(xs + b * pitch + 4 * k4) = *reinterpret_cast<const float4 *>(a.x + (long)b * a.K + (g0 << 8) + 4 * k4);
         }
     }
     __syncthreads();
     if (!live) return;
-    v4f32 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
-    const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + 16 * s);
+    v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
+    const float4 *xk = reinterpret_cast<const float4 *>(xs + r * pitch + 4 * s);
     const int nblocks = nk >> 6;   // blocks of 64 k
     for (int T = 0; T < nblocks; T++) {
-        float4 u0[4], u1[4], xc[4];
+        float4 u0[4], u1[4];
 #pragma unroll
-        for (int q = 0; q < 4; q++) { u0[q] = w0[q]; u1[q] = w1[q]; xc[q] = xk[16 * T + q]; }
+        for (int q = 0; q < 4; q++) { u0[q] = w0[q]; u1[q] = w1[q]; }
         if (T + 1 < nblocks) {
             c0 += 16; c1 += 16;   // 64 floats on
 #pragma unroll
-            for (int q = 0; q < 4; q++) { w0[q] = load_stream(c0 + q); w1[q] = load_stream(c1 + q); }
+            for (int q = 0; q < 4; q++) { w0[q] = load_stream(c0 + 4 * q); w1[q] = load_stream(c1 + 4 * q); }
         }
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const float bx[4] = {xc[q].x, xc[q].y, xc[q].z, xc[q].w};
-            const float a0[4] = {u0[q].x, u0[q].y, u0[q].z, u0[q].w}, a1[4] = {u1[q].x, u1[q].y, u1[q].z, u1[q].w};
+        for (int nb = 0; nb < NB; nb++) {
+            float4 xc[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                if (e & 1) {
-                    acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[e], bx[e], acc2, 0, 0, 0);
-                    acc3 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[e], bx[e], acc3, 0, 0, 0);
-                } else {
-                    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[e], bx[e], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[e], bx[e], acc1, 0, 0, 0);
+            for (int q = 0; q < 4; q++) xc[q] = xk[nb * 4 * pitch + 16 * T + 4 * q];   // (16 sequences on: 16 pitch floats)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float bx[4] = {xc[q].x, xc[q].y, xc[q].z, xc[q].w};
+                const float a0[4] = {u0[q].x, u0[q].y, u0[q].z, u0[q].w}, a1[4] = {u1[q].x, u1[q].y, u1[q].z, u1[q].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (e & 1) {
+                        acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[e], bx[e], acc2[nb], 0, 0, 0);
+                        acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[e], bx[e], acc3[nb], 0, 0, 0);
+                    } else {
+                        acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[e], bx[e], acc0[nb], 0, 0, 0);
+                        acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1[e], bx[e], acc1[nb], 0, 0, 0);
+                    }
                 }
             }
         }
     }
-    float *p = a.part + ((long)blockIdx.y * kBatch + r) * a.rows + row0 + 4 * s;
-    *reinterpret_cast<v4f32 *>(p) = acc0 + acc2;
-    if (two) *reinterpret_cast<v4f32 *>(p + 16) = acc1 + acc3;
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        float *p = a.part + ((long)blockIdx.y * NSEQ + 16 * nb + r) * a.rows + row0 + 4 * s;
+        *reinterpret_cast<v4f32 *>(p) = acc0[nb] + acc2[nb];
+        if (two) *reinterpret_cast<v4f32 *>(p + 16) = acc1[nb] + acc3[nb];
+    }
 }
 
 // ---- the element-wise kernels between the products --------------------------------------------------------------
@@ -307,8 +340,8 @@ __global__ void __launch_bounds__(kBgThreads) k_bgemm_f32(const BGemmF32 a)
 // Loop state of a batched decode, on the device.
 struct BatchState {
     int pos;              // position of the step being computed
-    int token[kBatch];    // input token of every sequence at this position
-    int n_prompt[kBatch];
+    int token[kMaxBatch];    // input token of every sequence at this position
+    int n_prompt[kMaxBatch];
 };
 
 // x[b] = row token[b] of the embedding table (J/Run.java:72)
@@ -354,7 +387,7 @@ __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ par
 {
     __shared__ float red[16];
     const int b = blockIdx.x, tid = threadIdx.x, n4 = n >> 2;
-    const long stride4 = (long)kBatch * n4;   // 16-byte words between two slices
+    const long stride4 = (long)gridDim.x * n4;   // 16-byte words between two slices (one workgroup per sequence)
     const float4 *pp = reinterpret_cast<const float4 *>(part) + (long)b * n4;
     float4 *xp = reinterpret_cast<float4 *>(x + (long)b * n);
     float ssq = 0.0f;
@@ -386,12 +419,12 @@ __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ par
 }
 
 // hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74), h1 and h3 the slices summed in order.
-// grid (hidden / 256, kBatch), 256 threads.
+// grid (hidden / 256, sequences), 256 threads.
 __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p1, const float *__restrict__ p3, int slices, int hidden,
                                                      const float *__restrict__ silu, int exact, float *__restrict__ hb)
 {
     const int b = blockIdx.y, rix = blockIdx.x * 256 + threadIdx.x;
-    const long n = (long)kBatch * hidden, i = (long)b * hidden + rix;
+    const long n = (long)gridDim.y * hidden, i = (long)b * hidden + rix;
     float h1 = 0.0f, h3 = 0.0f;
 #pragma unroll 8
     for (int s = 0; s < slices; s++) { h1 += p1[(long)s * n + i]; h3 += p3[(long)s * n + i]; }
@@ -400,12 +433,12 @@ __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p
 }
 
 struct BAttn {
-    const float *pq, *pk, *pv;   // partial products of Wq, Wk, Wv: (slices, kBatch, dim | kv_dim)
+    const float *pq, *pk, *pv;   // partial products of Wq, Wk, Wv: (slices, sequences, dim | kv_dim)
     int slices;
     const float2 *rope;          // (seq_len, head_size / 2) cos, sin
     float *kc, *vc;              // this layer's rows of the batch cache: + (b * seq_stride + pos) * kv_dim
     long seq_stride;             // cache rows between two sequences
-    float *out;                  // (kBatch, dim)
+    float *out;                  // (sequences, dim)
     const BatchState *st;
     int n_heads, kv_mul, head_size, kv_dim, dim;
     float sqrt_hs;
@@ -415,7 +448,7 @@ struct BAttn {
 // K/AccumWeightedValue.java).  First q of the head and k, v of its kv head at this position: the slices of the products
 // summed in order, RoPE on the pairs of q and k (K/ApplyRope.java:74-90), k and v into the cache row (J/Run.java:95-99; by
 // the first head of the kv group).  Then LPR lanes per cache row (four floats of the head each): the row slots of the
-// workgroup take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, kBatch).
+// workgroup take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, sequences).
 template <int LPR>
 __global__ void __launch_bounds__(256) k_battn(const BAttn a)
 {
@@ -434,7 +467,7 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
             const float *part = which == 0 ? a.pq : which == 1 ? a.pk : a.pv;
             float v0 = 0.0f, v1 = 0.0f;
             for (int s = 0; s < a.slices; s++) {
-                const float2 t = *reinterpret_cast<const float2 *>(part + ((long)s * kBatch + b) * rows + row);
+                const float2 t = *reinterpret_cast<const float2 *>(part + ((long)s * gridDim.y + b) * rows + row);
                 v0 += t.x; v1 += t.y;
             }
             if (which < 2) {
@@ -506,13 +539,13 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
 }
 
 struct BNext {
-    const float *part;    // (slices, kBatch, vocab) partial logits
+    const float *part;    // (slices, sequences, vocab) partial logits
     int slices, vocab;
-    float *logits;        // (kBatch, vocab)
+    float *logits;        // (sequences, vocab)
     BatchState *st;
-    const int *prompts;   // (kBatch, prompt_stride)
+    const int *prompts;   // (sequences, prompt_stride)
     int prompt_stride;
-    int *out_tokens;      // (kBatch, out_stride): `next` of every step
+    int *out_tokens;      // (sequences, out_stride): `next` of every step
     int out_stride;
 };
 
@@ -524,7 +557,7 @@ __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *done)
     __shared__ float bval[16];
     __shared__ int bidx[16];
     const int b = blockIdx.x, tid = threadIdx.x;
-    const long n = (long)kBatch * a.vocab;
+    const long n = (long)gridDim.x * a.vocab;
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
     for (int i = tid; i < a.vocab; i += 1024) {
@@ -551,7 +584,7 @@ __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *done)
         a.out_tokens[(long)b * a.out_stride + pos] = next;
         a.st->token[b] = next;
         __threadfence();
-        if (atomicAdd(done, 1u) == kBatch - 1) {   // every sequence has its token: the step is over
+        if (atomicAdd(done, 1u) == gridDim.x - 1) {   // every sequence has its token: the step is over
             *done = 0u;
             a.st->pos = pos + 1;
         }

@@ -1599,7 +1599,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (t.groups_loaded != t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
         const int ngroups = K / 256, gps = std::max(1, std::min(std::min(ngroups, kBgMaxGps), (int)groups_per_slice));
         const int slices = (ngroups + gps - 1) / gps;
-        const size_t lds = bg_lds_bytes(gps);
+        const size_t lds = bg_lds_bytes(gps, kBatch);
         if (lds + sizeof(float) * kBatch * kBgMaxGps > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
         HIPCHK(hipSetDevice(c->cfg.device));
         int trc = ensure_batch_tiles(c, tensor);
@@ -1616,7 +1616,7 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
         if (e == hipSuccess) e = hipEventCreate(&e0);
         if (e == hipSuccess) e = hipEventCreate(&e1);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             BGemm a{};
@@ -1624,9 +1624,9 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
             a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
             const dim3 grid((bg_units(rows, 2) + 3) / 4, slices);
             const int n = std::max(1, (int)rounds);
-            hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);   // warm
+            hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);   // warm
             (void)hipEventRecord(e0, c->stream);
-            for (int i = 0; i < n; i++) hipLaunchKernelGGL(k_bgemm<2>, grid, dim3(kBgThreads), lds, c->stream, a);
+            for (int i = 0; i < n; i++) hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);
             (void)hipEventRecord(e1, c->stream);
             hipLaunchKernelGGL(k_breduce, dim3(256), dim3(256), 0, c->stream, dpart, dy, rows, slices);
             e = hipGetLastError();
@@ -1686,13 +1686,13 @@ struct BtScope {
 constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
 
 int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
-size_t batch_lds() { return bg_lds_bytes(kBatchGps); }   // k_bgemm: bf16 planes
-size_t batch_lds_f32() { return (size_t)kBatch * (kBatchGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
+size_t batch_lds(int nseq) { return bg_lds_bytes(kBatchGps, nseq); }   // k_bgemm: bf16 planes
+size_t batch_lds_f32(int nseq) { return (size_t)nseq * (kBatchGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
 // workgroups of k_bgemm a compute unit holds at once: its 160 KB of LDS, and at most three by their registers
-int batch_resident() { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds() + sizeof(float) * kBatch * kBgMaxGps)))); }
+int batch_resident(int nseq) { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds(nseq) + sizeof(float) * nseq * kBgMaxGps)))); }
 
 // The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
-void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part)
+void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part, int nseq)
 {
     BGemm a{};
     int K = 0;
@@ -1707,81 +1707,96 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
     // All workgroups of the launch are resident at once (batch_resident() per compute unit); a wave takes one unit of 16 or 32 rows
     // after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
     // activations they fetch from LDS).
-    const int S = batch_slices(K), gmax = std::max(1, batch_resident() * c->n_cu / S);
+    const int nb = nseq / kBatch, waves = 4 * nb;
+    const int S = batch_slices(K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
     int tiles = 2, gx = 1, best = 1 << 30;
     for (int t = 2; t >= 1; t--) {
         int units = 0;
         for (int i = 0; i < a.nmat; i++) units += bg_units(a.rows[i], t);
-        const int g = std::min(gmax, (units + 3) / 4), iters = (units + 4 * g - 1) / (4 * g);
+        const int g = std::min(gmax, (units + waves - 1) / waves), iters = (units + waves * g - 1) / (waves * g);
         if (iters * t < best) {
             best = iters * t; tiles = t;
-            gx = (units + 4 * iters - 1) / (4 * iters);   // no more workgroups than that many rounds need
+            gx = (units + waves * iters - 1) / (waves * iters);   // no more workgroups than that many rounds need
         }
     }
     BT(*tensors.begin() == L2J_WQ ? "gemm qkv" : *tensors.begin() == L2J_WO ? "gemm wo" : *tensors.begin() == L2J_W2 ? "gemm w2" : "gemm w1,w3");
-    if (tiles == 1) hipLaunchKernelGGL(k_bgemm<1>, dim3(gx, S), dim3(kBgThreads), batch_lds(), c->stream, a);
-    else hipLaunchKernelGGL(k_bgemm<2>, dim3(gx, S), dim3(kBgThreads), batch_lds(), c->stream, a);
+    const dim3 grid(gx, S), block(kBgThreads * nb);
+    const size_t lds = batch_lds(nseq);
+    if (nb == 1) {
+        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 1>), grid, block, lds, c->stream, a);
+        else hipLaunchKernelGGL((k_bgemm<2, 1>), grid, block, lds, c->stream, a);
+    } else {
+        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 2>), grid, block, lds, c->stream, a);
+        else hipLaunchKernelGGL((k_bgemm<2, 2>), grid, block, lds, c->stream, a);
+    }
 }
 
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
-void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride)
+void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride, int nseq)
 {
     const l2j_config &cf = c->cfg;
     const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim;
     const int sd = batch_slices(dim), sh = batch_slices(hidden);
     hipStream_t s = c->stream;
-    { BT("embed"); hipLaunchKernelGGL(k_bembed, dim3(kBatch), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
-    { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(kBatch), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
+    { BT("embed"); hipLaunchKernelGGL(k_bembed, dim3(nseq), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
+    { BT("rms"); hipLaunchKernelGGL(k_brms, dim3(nseq), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
     for (int l = 0; l < L; l++) {
-        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part);
+        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part, nseq);
         BAttn t{};
         t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
         t.kc = b.kc + (size_t)l * max_pos * kvd; t.vc = b.vc + (size_t)l * max_pos * kvd;
         t.seq_stride = (long)L * max_pos; t.out = b.xb; t.st = b.st;
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
-        const dim3 ag(cf.n_heads, kBatch);
+        const dim3 ag(cf.n_heads, nseq);
         {
             BT("attention");
             if (hs == 64) hipLaunchKernelGGL(k_battn<16>, ag, dim3(256), 0, s, t);
             else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
             else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
         }
-        launch_bgemm(c, {L2J_WO}, l, b.xb, b.part);
-        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim); }
-        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.part);
-        { BT("epi swiglu"); hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, kBatch), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
+        launch_bgemm(c, {L2J_WO}, l, b.xb, b.part, nseq);
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim); }
+        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.part, nseq);
+        { BT("epi swiglu"); hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, nseq), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
                            (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb); }
-        launch_bgemm(c, {L2J_W2}, l, b.hb, b.part);
+        launch_bgemm(c, {L2J_W2}, l, b.hb, b.part, nseq);
         // the residual, then the norm of what follows: the next layer's attention norm, or the final one (rmsw: att, ffn, final)
         const float *wn = c->rmsw + (l + 1 < L ? (size_t)(l + 1) * dim : (size_t)2 * L * dim);
-        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(kBatch), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, dim); }
+        { BT("res + rms"); hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, dim); }
     }
-    BGemmF32 g{};
-    g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
-    { BT("classifier"); hipLaunchKernelGGL(k_bgemm_f32, dim3((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd), dim3(kBgThreads), batch_lds_f32(), s, g); }
+    {
+        BGemmF32 g{};
+        g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
+        BT("classifier");
+        const dim3 cg((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd);
+        if (nseq == kBatch) hipLaunchKernelGGL(k_bgemm_f32<1>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
+        else hipLaunchKernelGGL(k_bgemm_f32<2>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
+    }
     BNext n{};
     n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
     n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
-    { BT("next"); hipLaunchKernelGGL(k_bnext, dim3(kBatch), dim3(1024), 0, s, n, b.done); }
+    { BT("next"); hipLaunchKernelGGL(k_bnext, dim3(nseq), dim3(1024), 0, s, n, b.done); }
 }
 
 }  // namespace
 
-int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t prompt_stride, int32_t steps,
-                            int32_t *out_tokens, double *seconds)
+int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride,
+                            int32_t steps, int32_t *out_tokens, double *seconds)
 {
     return ctx_rc(c, [&]() -> int {
         std::lock_guard<std::mutex> forward_lock(g_forward_mu);
         if (!c || !n_prompt || !out_tokens || (prompt_stride > 0 && !prompts) || prompt_stride < 0) return fail(L2J_E_ARG, "bad argument");
         if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
+        if (n_seq != kBatch && n_seq != kMaxBatch) return fail(L2J_E_ARG, "n_seq must be 16 or 32");
+        const int nseq = n_seq;
         const l2j_config &cf = c->cfg;
         const int hs = c->head_size;
         if (cf.dim % 256 || cf.hidden_dim % 256 || c->kv_dim % 16 || cf.vocab_size % 16 || (hs != 64 && hs != 128 && hs != 256))
             return fail(L2J_E_SIZE, "batched decode needs dim and hidden_dim in whole groups of 256, kv_dim and vocab_size multiples of 16, "
                                     "head_size 64, 128 or 256");
         if (steps <= 0 || steps > cf.seq_len) return fail(L2J_E_ARG, "steps must be 1..seq_len");
-        for (int b = 0; b < kBatch; b++) {
+        for (int b = 0; b < nseq; b++) {
             if (n_prompt[b] < 0 || n_prompt[b] > prompt_stride) return fail(L2J_E_ARG, "n_prompt out of range");
             for (int i = 0; i < n_prompt[b]; i++)
                 if (prompts[(size_t)b * prompt_stride + i] < 0 || prompts[(size_t)b * prompt_stride + i] >= cf.vocab_size)
@@ -1797,8 +1812,8 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
         }
         const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, kvd = c->kv_dim, vocab = cf.vocab_size;
         const int sd = batch_slices(dim), sh = batch_slices(hidden);
-        const size_t part_floats = (size_t)kBatch * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
-        const size_t cache_floats = (size_t)kBatch * L * steps * kvd;
+        const size_t part_floats = (size_t)nseq * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
+        const size_t cache_floats = (size_t)nseq * L * steps * kvd;
         const int pstride = std::max(1, (int)prompt_stride);
         BatchBufs b;
         auto done = [&](int rc) { b.release(); return rc; };
@@ -1806,27 +1821,30 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
         auto alloc = [&](auto **p, size_t n) {
             if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
         };
-        alloc(&b.x, (size_t)kBatch * dim); alloc(&b.xn, (size_t)kBatch * std::max(dim, hidden));
-        alloc(&b.xb, (size_t)kBatch * dim); alloc(&b.hb, (size_t)kBatch * hidden); alloc(&b.logits, (size_t)kBatch * vocab);
+        alloc(&b.x, (size_t)nseq * dim); alloc(&b.xn, (size_t)nseq * std::max(dim, hidden));
+        alloc(&b.xb, (size_t)nseq * dim); alloc(&b.hb, (size_t)nseq * hidden); alloc(&b.logits, (size_t)nseq * vocab);
         for (int i = 0; i < 3; i++) alloc(&b.part[i], part_floats);
         alloc(&b.kc, cache_floats); alloc(&b.vc, cache_floats);
-        alloc(&b.st, 1); alloc(&b.prompts, (size_t)kBatch * pstride); alloc(&b.out, (size_t)kBatch * steps); alloc(&b.done, 1);
+        alloc(&b.st, 1); alloc(&b.prompts, (size_t)nseq * pstride); alloc(&b.out, (size_t)nseq * steps); alloc(&b.done, 1);
         if (e == hipSuccess) e = hipEventCreate(&b.e0);
         if (e == hipSuccess) e = hipEventCreate(&b.e1);
-        const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)kBatch * pstride, out_ints = (size_t)kBatch * steps;
+        const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)nseq * pstride, out_ints = (size_t)nseq * steps;
         if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&b.h_pin), std::max(state_ints + prompt_ints, out_ints) * sizeof(int), hipHostMallocDefault);
         if (e != hipSuccess) return done(fail(L2J_E_HIP, std::string("batched decode: ") + hipGetErrorString(e)));
         BatchState h{};
         h.pos = 0;
-        for (int i = 0; i < kBatch; i++) { h.token[i] = 1; h.n_prompt[i] = n_prompt[i]; }   // BOS first (J/Run.java:612)
+        for (int i = 0; i < nseq; i++) { h.token[i] = 1; h.n_prompt[i] = n_prompt[i]; }   // BOS first (J/Run.java:612)
         memcpy(b.h_pin, &h, sizeof(h));
         if (prompt_stride > 0) memcpy(b.h_pin + state_ints, prompts, prompt_ints * sizeof(int));
         if (hipMemcpyAsync(b.st, b.h_pin, sizeof(h), hipMemcpyHostToDevice, c->stream) != hipSuccess ||
             (prompt_stride > 0 && hipMemcpyAsync(b.prompts, b.h_pin + state_ints, prompt_ints * sizeof(int), hipMemcpyHostToDevice, c->stream) != hipSuccess) ||
             hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream) != hipSuccess ||
-            hipFuncSetAttribute((const void *)k_bgemm<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
-            hipFuncSetAttribute((const void *)k_bgemm<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds()) != hipSuccess ||
-            hipFuncSetAttribute((const void *)k_bgemm_f32, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32()) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<1, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kBatch)) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kBatch)) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kMaxBatch)) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kMaxBatch)) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm_f32<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kBatch)) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_bgemm_f32<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kMaxBatch)) != hipSuccess ||
             hipStreamSynchronize(c->stream) != hipSuccess)
             return done(fail(L2J_E_HIP, "batched decode: set-up failed"));
         // one position as a graph: every kernel reads the position and the tokens from device memory ("graph" = 0: the
@@ -1835,7 +1853,7 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
         if (use_graph) {
             e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
             if (e == hipSuccess) {
-                launch_batch_step(c, b, steps, pstride);
+                launch_batch_step(c, b, steps, pstride, nseq);
                 const hipError_t le = hipGetLastError();
                 e = hipStreamEndCapture(c->stream, &b.graph);
                 if (e == hipSuccess) e = le;
@@ -1847,7 +1865,7 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             if (use_graph) {
                 e = hipGraphLaunch(b.exec, c->stream);
             } else {
-                launch_batch_step(c, b, steps, pstride);
+                launch_batch_step(c, b, steps, pstride, nseq);
                 e = hipGetLastError();
             }
             if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
@@ -1861,7 +1879,7 @@ int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n
             h2.pos = steps - 1;
             (void)hipMemcpy(b.st, &h2, sizeof(h2), hipMemcpyHostToDevice);
             g_bt_on = true; g_bt.clear();
-            launch_batch_step(c, b, steps, pstride);
+            launch_batch_step(c, b, steps, pstride, nseq);
             g_bt_on = false;
             (void)hipStreamSynchronize(c->stream);
             std::map<std::string, std::pair<double, int>> acc;

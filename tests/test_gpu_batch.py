@@ -1,5 +1,5 @@
-"""Sixteen sequences at once (l2j_decode_greedy_batch, l2j_batch_matmul): the matrix-core path must give every sequence
-what it gets alone.  Checked through the C ABI against the single-sequence path (itself pinned against the CPU oracle
+"""Sixteen or thirty-two sequences at once (l2j_decode_greedy_batch, l2j_batch_matmul): the matrix-core path must give
+every sequence what it gets alone.  Checked through the C ABI against the single-sequence path (itself pinned against the CPU oracle
 in test_gpu_parity.py), against the oracle directly, and against float64 products of the dequantized weights."""
 import numpy as np
 import pytest
@@ -46,17 +46,18 @@ def test_matrix_core_product_matches_float64():
     g.close()
 
 
+@pytest.mark.parametrize("n_seq", [16, 32])
 @pytest.mark.parametrize("shape", SHAPES)
-def test_every_sequence_gets_what_it_gets_alone(orc, shape):
+def test_every_sequence_gets_what_it_gets_alone(orc, shape, n_seq):
     g = l2j.Transformer(l2j.Config(*shape))
     g.fill_synthetic(9, 0.02)
     g.finalize()
-    rng = np.random.default_rng(shape[0] + shape[4])
+    rng = np.random.default_rng(shape[0] + shape[4] + n_seq)
     steps = shape[6]
-    prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 9))).astype(np.int32) for _ in range(13)]   # three without a prompt
-    got, sec = g.decode_greedy_batch(prompts, steps)
-    assert got.shape == (16, steps) and sec > 0
-    for b in range(16):
+    prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 9))).astype(np.int32) for _ in range(n_seq - 3)]   # three without a prompt
+    got, sec = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
+    assert got.shape == (n_seq, steps) and sec > 0
+    for b in range(n_seq):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
         g.reset()
         want, _ = g.decode_greedy(p, steps)          # stops after token 1; the batch runs on
@@ -66,7 +67,7 @@ def test_every_sequence_gets_what_it_gets_alone(orc, shape):
     m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
                   vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
     m.fill_synth(9, 0.02)
-    for b in (0, 15):
+    for b in (0, n_seq - 1):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
         m.reset()
         want, _, _ = m.generate_greedy(p, steps)
@@ -88,4 +89,15 @@ def test_shapes_the_batched_path_does_not_take_are_an_error():
     with pytest.raises(L2JError):
         g.batch_matmul(TENSOR.WQ, 0, np.zeros((16, 288), dtype=np.float32), 288)
     assert len(g.decode_greedy(np.array([5, 6], dtype=np.int32), 8)[0]) > 0     # the context stays usable
+    g.close()
+
+
+def test_sequence_counts_other_than_16_and_32_are_an_error():
+    g = l2j.Transformer(l2j.Config(512, 1024, 1, 8, 8, 1008, 16, 1))
+    g.fill_synthetic(1, 0.02)
+    g.finalize()
+    for n_seq in (1, 8, 17, 48, 64):
+        with pytest.raises(L2JError) as e:
+            g.decode_greedy_batch([np.array([5], dtype=np.int32)], 4, n_seq=n_seq)
+        assert e.value.code == -1
     g.close()
