@@ -9,6 +9,7 @@
 #pragma once
 
 #include "kernels.hpp"
+#include "phase_kernels.hpp"   // grid barrier, device-coherent loads and stores
 
 namespace l2j {
 
@@ -86,28 +87,18 @@ __device__ __forceinline__ void split_bf16(float x, uint32_t h[3])
     h[0] = b0 >> 16; h[1] = b1 >> 16; h[2] = __float_as_uint(r2) >> 16;
 }
 
-// Workgroup (y: one slice of K; x: a share of the rows): the slice of the 16 NB activation vectors is staged in LDS once,
-// as three bf16 planes, then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in turn:
-// unit blockIdx.x * 4 NB + wave, then every gridDim.x * 4 NB-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of
+// Workgroup (by: one slice of K; bx of gx: a share of the rows): the slice of the 16 NB activation vectors is staged in LDS
+// once, as three bf16 planes, then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in
+// turn: unit bx * 4 NB + wave, then every gx * 4 NB-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of
 // row r at k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile, from the copy in tile order); one MFMA
 // multiplies the 16 rows by 16 sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane and
 // column block.  After the 24 NB MFMAs of a group the 16 x 16 sums get the group's scale and offset.  TILES = 2: two
 // tiles share the activations fetched from LDS; NB = 2: two column blocks share the converted codes.  256 NB threads.
+// The work of one wave, in two steps so that a kernel with several phases can request the first codes of a product
+// before the phase (and the grid barrier) that produces its activations: begin(), then run().
 template <int TILES, int NB>
-__global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
-{
-    constexpr int NSEQ = kBatch * NB, WAVES = 4 * NB;
-    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * NSEQ + b) * pitch + k]
-    __shared__ float sxs[NSEQ][kBgMaxGps];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int ngroups = a.K >> 8;
-    const int g0 = blockIdx.y * a.gps, g1 = min(ngroups, g0 + a.gps), nk = (g1 - g0) << 8;
-    const int r = lane & 15, s = lane >> 4;
-    int total = 0;
-    for (int i = 0; i < a.nmat; i++) total += bg_units(a.rows[i], TILES);
-    const int stride = gridDim.x * WAVES;
-    int u = blockIdx.x * WAVES + wave;
-
+struct BgWave {
+    static constexpr int NSEQ = kBatch * NB, WAVES = 4 * NB;
     struct Unit {   // 16 * TILES rows of one matrix: where this lane's codes, scales and results are
         const uint4 *c0, *c1;
         const float2 *gs0, *gs1;
@@ -115,7 +106,15 @@ __global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
         int rows;
         bool two;
     };
-    auto locate = [&](int unit) {
+    const BGemm &a;
+    int by, lane, r, s, ngroups, g0, g1, total, stride, u;
+    Unit cur;
+    uint4 w0[4], w1[4];
+
+    __device__ __forceinline__ BgWave(const BGemm &a_) : a(a_) {}
+
+    __device__ __forceinline__ Unit locate(int unit) const
+    {
         int mi = 0;
         while (mi + 1 < a.nmat && unit >= bg_units(a.rows[mi], TILES)) { unit -= bg_units(a.rows[mi], TILES); mi++; }
         const QMat mat = a.m[mi];
@@ -128,125 +127,180 @@ __global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
         n.c1 = n.c0 + (n.two ? (long)ngroups << 8 : 0L);   // the next tile: ngroups blocks of 256 16-byte words on
         n.gs0 = mat.gs + (mat.off >> 8) + (block << 4) + 4 * s;
         n.gs1 = n.gs0 + (n.two ? (long)ngroups << 4 : 0L);
-        n.out = a.part[mi] + ((long)blockIdx.y * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
+        n.out = a.part[mi] + ((long)by * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
         return n;
-    };
-    uint4 w0[4], w1[4];
-    auto request = [&](const Unit &n) {   // one group of the unit's codes
+    }
+
+    __device__ __forceinline__ void request(const Unit &n)   // one group of the unit's codes
+    {
 #pragma unroll
         for (int T = 0; T < 4; T++) { w0[T] = load_stream(n.c0 + 64 * T); if (TILES == 2) w1[T] = load_stream(n.c1 + 64 * T); }
-    };
-    // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
-    // offsets) and their three bf16 parts.  The activations of the first two groups are requested before the wave's
-    // first codes (a wave's loads return in order: behind 8 KB of codes they would arrive with them).
-    const int pitch = nk + kXPadH, plane = NSEQ * pitch;
-    const int sb = tid >> 4, pt = tid & 15;
-    const float4 *xsrc = reinterpret_cast<const float4 *>(a.x + (long)sb * a.K + (g0 << 8) + 16 * pt);
-    float4 xa[2][4];
-#pragma unroll
-    for (int gi = 0; gi < 2; gi++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) xa[gi][q] = gi < g1 - g0 ? xsrc[64 * gi + q] : make_float4(0.f, 0.f, 0.f, 0.f);
-    Unit cur{};
-    if (u < total) { cur = locate(u); request(cur); }
-    auto stage = [&](int gi, const float4 (&v)[4]) {
-        float t = ((v[0].x + v[0].y) + (v[0].z + v[0].w)) + ((v[1].x + v[1].y) + (v[1].z + v[1].w)) + ((v[2].x + v[2].y) + (v[2].z + v[2].w)) +
-                  ((v[3].x + v[3].y) + (v[3].z + v[3].w));
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
-        if (pt == 0) sxs[sb][gi] = t;
-        const float xv[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w, v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
-        uint32_t pk[3][8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            uint32_t lo[3], hi[3];
-            split_bf16(xv[2 * e], lo);
-            split_bf16(xv[2 * e + 1], hi);
-#pragma unroll
-            for (int pl = 0; pl < 3; pl++) pk[pl][e] = lo[pl] | (hi[pl] << 16);
-        }
-        unsigned short *dst = xh + sb * pitch + (gi << 8) + 16 * pt;
-#pragma unroll
-        for (int pl = 0; pl < 3; pl++) {
-            reinterpret_cast<uint4 *>(dst + pl * plane)[0] = make_uint4(pk[pl][0], pk[pl][1], pk[pl][2], pk[pl][3]);
-            reinterpret_cast<uint4 *>(dst + pl * plane)[1] = make_uint4(pk[pl][4], pk[pl][5], pk[pl][6], pk[pl][7]);
-        }
-    };
-    stage(0, xa[0]);
-    if (g1 - g0 > 1) stage(1, xa[1]);
-    for (int gi = 2; gi < g1 - g0; gi++) {
-        const float4 v[4] = {xsrc[64 * gi], xsrc[64 * gi + 1], xsrc[64 * gi + 2], xsrc[64 * gi + 3]};
-        stage(gi, v);
     }
-    __syncthreads();
-    for (; u < total; u += stride) {
-        const bool more = u + stride < total;
-        Unit nxt{};
-        if (more) nxt = locate(u + stride);
-        v4f32 y0[NB], y1[NB];
+
+    // This wave's share of workgroup (bx, by) of a gx-wide grid; first = false: the first codes are not requested yet
+    // (run() does it once the first activations are requested: a wave's loads return in order, and behind 8 KB of codes
+    // the activations would arrive with them).
+    __device__ __forceinline__ void begin(int bx, int by_, int gx, bool first)
+    {
+        const int tid = threadIdx.x;
+        by = by_;
+        lane = tid & 63;
+        r = lane & 15; s = lane >> 4;
+        ngroups = a.K >> 8;
+        g0 = by * a.gps; g1 = min(ngroups, g0 + a.gps);
+        total = 0;
+        for (int i = 0; i < a.nmat; i++) total += bg_units(a.rows[i], TILES);
+        stride = gx * WAVES;
+        u = bx * WAVES + (tid >> 6);
+        cur = Unit{};
+        if (u < total) {
+            cur = locate(u);
+            if (first) request(cur);
+        }
+    }
+
+    // requested = begin(.., true) was called.  COH: the activations were written by other workgroups of this launch and
+    // the partial sums are read by other workgroups of it (device-coherent loads, write-through stores).
+    template <bool COH>
+    __device__ __forceinline__ void run(unsigned short *xh, float (*sxs)[kBgMaxGps], bool requested)
+    {
+        const int tid = threadIdx.x, nk = (g1 - g0) << 8;
+        // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
+        // offsets) and their three bf16 parts.
+        const int pitch = nk + kXPadH, plane = NSEQ * pitch;
+        const int sb = tid >> 4, pt = tid & 15;
+        const float *xsrc = a.x + (long)sb * a.K + (g0 << 8) + 16 * pt;
+        float xa[2][16];
 #pragma unroll
-        for (int nb = 0; nb < NB; nb++) y0[nb] = y1[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
-        for (int g = g0; g < g1; g++) {
-            uint4 u0[4], u1[4];
+        for (int gi = 0; gi < 2; gi++) {
+            if (COH) {
 #pragma unroll
-            for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
-            // the next group's codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
-            if (g + 1 < g1) {
-                cur.c0 += 256; cur.c1 += 256;
-                request(cur);
-            } else if (more) {
-                request(nxt);
+                for (int e = 0; e < 16; e++) xa[gi][e] = gi < g1 - g0 ? ld_coh(xsrc + 256 * gi + e) : 0.0f;
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4 v = gi < g1 - g0 ? reinterpret_cast<const float4 *>(xsrc + 256 * gi)[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    xa[gi][4 * q] = v.x; xa[gi][4 * q + 1] = v.y; xa[gi][4 * q + 2] = v.z; xa[gi][4 * q + 3] = v.w;
+                }
             }
-            float2 sc0[4], sc1[4];   // (rm, min) of rows 4 s + (0..3) of the tile
+        }
+        if (!requested && u < total) request(cur);
+        auto stage = [&](int gi, const float (&v)[16]) {
+            float t = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7])) + ((v[8] + v[9]) + (v[10] + v[11])) +
+                      ((v[12] + v[13]) + (v[14] + v[15]));
 #pragma unroll
-            for (int i = 0; i < 4; i++) { sc0[i] = cur.gs0[i]; if (TILES == 2) sc1[i] = cur.gs1[i]; }
-            v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
+            for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
+            if (pt == 0) sxs[sb][gi] = t;
+            uint32_t pk[3][8];
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
-            const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
+            for (int e = 0; e < 8; e++) {
+                uint32_t lo[3], hi[3];
+                split_bf16(v[2 * e], lo);
+                split_bf16(v[2 * e + 1], hi);
 #pragma unroll
-            for (int T = 0; T < 4; T++) {
-                const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
-                v8bf16 a10 = a00, a11 = a01;
-                if (TILES == 2) { a10 = codes_bf16(u1[T].x, u1[T].y); a11 = codes_bf16(u1[T].z, u1[T].w); }
+                for (int pl = 0; pl < 3; pl++) pk[pl][e] = lo[pl] | (hi[pl] << 16);
+            }
+            unsigned short *dst = xh + sb * pitch + (gi << 8) + 16 * pt;
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) {
-                    v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
+            for (int pl = 0; pl < 3; pl++) {
+                reinterpret_cast<uint4 *>(dst + pl * plane)[0] = make_uint4(pk[pl][0], pk[pl][1], pk[pl][2], pk[pl][3]);
+                reinterpret_cast<uint4 *>(dst + pl * plane)[1] = make_uint4(pk[pl][4], pk[pl][5], pk[pl][6], pk[pl][7]);
+            }
+        };
+        stage(0, xa[0]);
+        if (g1 - g0 > 1) stage(1, xa[1]);
+        for (int gi = 2; gi < g1 - g0; gi++) {
+            float v[16];
 #pragma unroll
-                    for (int pl = 0; pl < 3; pl++) {
-                        bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
-                        bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
-                    }
+            for (int e = 0; e < 16; e++) v[e] = COH ? ld_coh(xsrc + 256 * gi + e) : xsrc[256 * gi + e];
+            stage(gi, v);
+        }
+        __syncthreads();
+        for (; u < total; u += stride) {
+            const bool more = u + stride < total;
+            Unit nxt{};
+            if (more) nxt = locate(u + stride);
+            v4f32 y0[NB], y1[NB];
 #pragma unroll
-                    for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
-                        acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0[nb], 0, 0, 0);
-                        acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2[nb], 0, 0, 0);
-                        if (TILES == 2) {
-                            acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1[nb], 0, 0, 0);
-                            acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3[nb], 0, 0, 0);
+            for (int nb = 0; nb < NB; nb++) y0[nb] = y1[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
+            for (int g = g0; g < g1; g++) {
+                uint4 u0[4], u1[4];
+#pragma unroll
+                for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
+                // the next group's codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
+                if (g + 1 < g1) {
+                    cur.c0 += 256; cur.c1 += 256;
+                    request(cur);
+                } else if (more) {
+                    request(nxt);
+                }
+                float2 sc0[4], sc1[4];   // (rm, min) of rows 4 s + (0..3) of the tile
+#pragma unroll
+                for (int i = 0; i < 4; i++) { sc0[i] = cur.gs0[i]; if (TILES == 2) sc1[i] = cur.gs1[i]; }
+                v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
+                const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
+#pragma unroll
+                for (int T = 0; T < 4; T++) {
+                    const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
+                    v8bf16 a10 = a00, a11 = a01;
+                    if (TILES == 2) { a10 = codes_bf16(u1[T].x, u1[T].y); a11 = codes_bf16(u1[T].z, u1[T].w); }
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++) {
+                        v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
+#pragma unroll
+                        for (int pl = 0; pl < 3; pl++) {
+                            bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
+                            bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
+                        }
+#pragma unroll
+                        for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
+                            acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0[nb], 0, 0, 0);
+                            acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2[nb], 0, 0, 0);
+                            if (TILES == 2) {
+                                acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1[nb], 0, 0, 0);
+                                acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3[nb], 0, 0, 0);
+                            }
                         }
                     }
                 }
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) {
+                    const float sxv = sxs[16 * nb + r][g - g0];   // this lane's column is sequence 16 nb + r
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        y0[nb][i] += fmaf(sc0[i].x, acc0[nb][i] + acc2[nb][i], sc0[i].y * sxv);
+                        if (TILES == 2) y1[nb][i] += fmaf(sc1[i].x, acc1[nb][i] + acc3[nb][i], sc1[i].y * sxv);
+                    }
+                }
+                cur.gs0 += 16; cur.gs1 += 16;
             }
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) {
-                const float sxv = sxs[16 * nb + r][g - g0];   // this lane's column is sequence 16 nb + r
+                float *o = cur.out + (long)nb * 16 * cur.rows;
+                if (COH) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    y0[nb][i] += fmaf(sc0[i].x, acc0[nb][i] + acc2[nb][i], sc0[i].y * sxv);
-                    if (TILES == 2) y1[nb][i] += fmaf(sc1[i].x, acc1[nb][i] + acc3[nb][i], sc1[i].y * sxv);
+                    for (int i = 0; i < 4; i++) { st_coh(o + i, y0[nb][i]); if (cur.two) st_coh(o + 16 + i, y1[nb][i]); }
+                } else {
+                    *reinterpret_cast<v4f32 *>(o) = y0[nb];
+                    if (cur.two) *reinterpret_cast<v4f32 *>(o + 16) = y1[nb];
                 }
             }
-            cur.gs0 += 16; cur.gs1 += 16;
+            cur = nxt;
         }
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-            float *o = cur.out + (long)nb * 16 * cur.rows;
-            *reinterpret_cast<v4f32 *>(o) = y0[nb];
-            if (cur.two) *reinterpret_cast<v4f32 *>(o + 16) = y1[nb];
-        }
-        cur = nxt;
     }
+};
+
+// grid (workgroups per slice, slices of K), 256 NB threads; dynamic LDS: bg_lds_bytes(gps, 16 NB)
+template <int TILES, int NB>
+__global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
+{
+    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * NSEQ + b) * pitch + k]
+    __shared__ float sxs[kBatch * NB][kBgMaxGps];
+    BgWave<TILES, NB> w(a);
+    w.begin(blockIdx.x, blockIdx.y, gridDim.x, false);
+    w.template run<false>(xh, sxs, false);
 }
 
 // ---- the classifier: fp32 weights (K/MatMul.java:37-60), the same tiling -------------------------------------------
@@ -466,7 +520,8 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
             const int rows = which == 0 ? a.dim : a.kv_dim, row = (which == 0 ? h : kvh) * hs + 2 * idx;
             const float *part = which == 0 ? a.pq : which == 1 ? a.pk : a.pv;
             float v0 = 0.0f, v1 = 0.0f;
-            for (int s = 0; s < a.slices; s++) {
+#pragma unroll 8
+            for (int s = 0; s < a.slices; s++) {   // (independent loads, added in slice order)
                 const float2 t = *reinterpret_cast<const float2 *>(part + ((long)s * gridDim.y + b) * rows + row);
                 v0 += t.x; v1 += t.y;
             }
