@@ -79,6 +79,28 @@ def test_every_sequence_gets_what_it_gets_alone(orc, shape, n_seq):
     m.close(); g.close()
 
 
+@pytest.mark.parametrize("shape,n_seq,steps", [
+    ((4096, 11008, 3, 32, 32, 32000, 48, 0), 32, 40),      # the widths of Llama-2-7B: rows of 16 and 43 groups
+    ((4096, 11008, 3, 32, 32, 32000, 48, 0), 16, 40),
+    ((8192, 28672, 2, 64, 8, 32000, 32, 0), 32, 24),       # the widths of Llama-2-70B: 64 heads on 8 kv heads, rows of 32 and 112 groups
+])
+def test_published_widths_match_the_single_decode(shape, n_seq, steps):
+    """At the matrix sizes of the published models (a few layers of them) every sequence of a batch gets the tokens of its
+    own single-sequence decode; the single-sequence path is pinned against the oracle at these widths in test_gpu_parity.py."""
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(21, 0.02)
+    g.finalize()
+    rng = np.random.default_rng(n_seq + shape[0])
+    prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 7))).astype(np.int32) for _ in range(n_seq - 1)]
+    got, _ = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
+    for b in range(n_seq):
+        p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
+        g.reset()
+        want, _ = g.decode_greedy(p, steps)
+        np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d" % b)
+    g.close()
+
+
 def test_shapes_the_batched_path_does_not_take_are_an_error():
     g = l2j.Transformer(l2j.Config(288, 768, 1, 6, 6, 320, 16, 1))   # rows of 288 codes: groups straddle rows
     g.fill_synthetic(1, 0.02)
