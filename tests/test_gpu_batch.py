@@ -15,6 +15,7 @@ SHAPES = [
     (512, 1024, 2, 8, 2, 1008, 64, 0),      # grouped-query attention: 8 heads on 2 kv heads
     (1024, 2816, 2, 8, 4, 2000, 96, 0),     # head 128, rows of 4 and 11 groups (an odd number of groups: a last slice of one)
     (512, 768, 2, 2, 2, 512, 40, 1),        # head 256
+    (512, 1024, 2, 8, 2, 1008, 640, 0),     # 640 positions: the row slots of the attention kernel go round forty times
 ]
 
 
