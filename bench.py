@@ -130,7 +130,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=97, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
     ap.add_argument("--no-sampled", action="store_true", help="skip the extra decode with the device sampler")
-    ap.add_argument("--no-batched", action="store_true", help="skip the extra decode of sixteen sequences at once")
+    ap.add_argument("--no-batched", action="store_true", help="skip the extra decodes of 32 and 16 sequences at once")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
     a = ap.parse_args()
