@@ -135,6 +135,7 @@ struct l2j_ctx {
     QTensor qt[L2J_TENSOR_COUNT];
     uint8_t *bt_codes[L2J_TENSOR_COUNT] = {};   // the batched path's copy of the matrices in tile order (k_btile), made by its first call
     float2 *bt_gs[L2J_TENSOR_COUNT] = {};
+    bool bt_done[L2J_TENSOR_COUNT] = {};        // the copy of this tensor has been launched
     bool bt_ready = false;
     float *emb = nullptr, *wcls = nullptr;
     bool emb_loaded = false, wcls_loaded = false;
@@ -1560,7 +1561,7 @@ static bool matrix_shape(const l2j_config &cf, int tensor, int *rows, int *K)
 // The tile-ordered copy of `tensor` for the batched path (rows % 16 == 0 and K % 256 == 0 checked by the caller).
 static int ensure_batch_tiles(l2j_ctx *c, int tensor)
 {
-    if (c->bt_codes[tensor] && c->bt_gs[tensor]) return L2J_OK;
+    if (c->bt_done[tensor]) return L2J_OK;
     int rows = 0, K = 0;
     if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
     const QTensor &t = c->qt[tensor];
@@ -1573,6 +1574,7 @@ static int ensure_batch_tiles(l2j_ctx *c, int tensor)
     hipLaunchKernelGGL(k_btile, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, c->stream, t.codes, t.gs, n16, rows, K, c->bt_codes[tensor],
                        c->bt_gs[tensor]);
     HIPCHK(hipGetLastError());
+    c->bt_done[tensor] = true;
     return L2J_OK;
 }
 
