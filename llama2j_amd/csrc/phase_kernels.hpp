@@ -228,55 +228,51 @@ struct MatvecPhase {
 // so that lane c of a wave reads consecutive 16-byte words for a fixed q (bank-conflict free);
 // sumx[c] = sum of the 16 activations of chunk c (for the group-minimum term of the dequantization).
 
-__device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
-                                             float *sumx, float *red, int T)
+// The rmsnorm scalar is not applied to the staged vector: sum_e w_e * (g_e * (ss * x_e)) = ss * sum_e w_e * (g_e * x_e), so
+// the vector is staged as g_e * x_e as its words arrive, the waves leave their sums of squares in `red`, and the one
+// workgroup barrier that publishes the vector publishes them too; the caller multiplies its row sums by the returned
+// ss = 1 / sqrt(sum x^2 / n + 1e-5) (K/RootMeanSquare.java:31-33).  The block-wide reduction and its two barriers are
+// thereby off the path between the arrival of the input and the first multiply-add (only rounding differs from
+// K/WeightNormalizeAndScale.java:73, by a few 1e-7 of a result).  Returns 1 without rmsnorm weights.
+__device__ __forceinline__ float rms_scalar(const float *red, int nw, int n)
+{
+    float ssq = 0.0f;
+    for (int w = 0; w < nw; w++) ssq += red[w];
+    // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
+    const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, ss)));  // uniform: a scalar register
+}
+
+__device__ __forceinline__ float stage_vector(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
+                                              float *sumx, float *red, int T)
 {
     const int nch = n >> 4, tid = phase_tid();
-    if (rmsw) {
-        float ssq = 0.0f;
-        for (int c = tid; c < nch; c += T) {
-            const float4 *xp = reinterpret_cast<const float4 *>(xin + 16 * c);
-            const float4 a = xp[0], b = xp[1], cc = xp[2], d = xp[3];
-            xs[c] = a;
-            xs[nch + c] = b;
-            xs[2 * nch + c] = cc;
-            xs[3 * nch + c] = d;
-            ssq += (a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w) + (b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w) +
-                   (cc.x * cc.x + cc.y * cc.y + cc.z * cc.z + cc.w * cc.w) + (d.x * d.x + d.y * d.y + d.z * d.z + d.w * d.w);
-        }
-        ssq = block_sum(ssq, red, T >> 6);
-        // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
-        const float ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
-        for (int c = tid; c < nch; c += T) {
-            const float4 *wp = reinterpret_cast<const float4 *>(rmsw + 16 * c);
-            float s = 0.0f;
+    float ssq = 0.0f;
+    for (int c = tid; c < nch; c += T) {
+        const float4 *xp = reinterpret_cast<const float4 *>(xin + 16 * c);
+        float4 v[4] = {xp[0], xp[1], xp[2], xp[3]};
+        float s = 0.0f;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                float4 xv = xs[q * nch + c];
-                const float4 wv = wp[q];
-                // out = weight * (ss * x)   (K/WeightNormalizeAndScale.java:73)
-                xv.x = __fmul_rn(wv.x, __fmul_rn(ss, xv.x));
-                xv.y = __fmul_rn(wv.y, __fmul_rn(ss, xv.y));
-                xv.z = __fmul_rn(wv.z, __fmul_rn(ss, xv.z));
-                xv.w = __fmul_rn(wv.w, __fmul_rn(ss, xv.w));
-                s += (xv.x + xv.y) + (xv.z + xv.w);
-                xs[q * nch + c] = xv;
+        for (int q = 0; q < 4; q++) {
+            ssq += (v[q].x * v[q].x + v[q].y * v[q].y) + (v[q].z * v[q].z + v[q].w * v[q].w);
+            if (rmsw) {
+                const float4 wv = reinterpret_cast<const float4 *>(rmsw + 16 * c)[q];
+                v[q].x = __fmul_rn(wv.x, v[q].x);
+                v[q].y = __fmul_rn(wv.y, v[q].y);
+                v[q].z = __fmul_rn(wv.z, v[q].z);
+                v[q].w = __fmul_rn(wv.w, v[q].w);
             }
-            sumx[c] = s;
+            s += (v[q].x + v[q].y) + (v[q].z + v[q].w);
+            xs[q * nch + c] = v[q];
         }
-    } else {
-        for (int c = tid; c < nch; c += T) {
-            const float4 *xp = reinterpret_cast<const float4 *>(xin + 16 * c);
-            const float4 a = xp[0], b = xp[1], cc = xp[2], d = xp[3];
-            xs[c] = a;
-            xs[nch + c] = b;
-            xs[2 * nch + c] = cc;
-            xs[3 * nch + c] = d;
-            sumx[c] = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w)) + ((cc.x + cc.y) + (cc.z + cc.w)) +
-                      ((d.x + d.y) + (d.z + d.w));
-        }
+        sumx[c] = s;
+    }
+    if (rmsw) {
+        ssq = wave_sum(ssq);
+        if ((tid & 63) == 0) red[tid >> 6] = ssq;
     }
     __syncthreads();
+    return rmsw ? rms_scalar(red, T >> 6, n) : 1.0f;
 }
 
 // The same with the vector read word by word as soon as its producers have written it (hand-over by value).
@@ -287,38 +283,27 @@ __device__ __forceinline__ void stage_vector(const float *__restrict__ xin, int 
 constexpr int kPollWords = 4;
 
 template <int WORDS>
-__device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
-                                                  float *sumx, float *red, int T, const Poll &pl)
+__device__ __forceinline__ float stage_vector_poll(const float *__restrict__ xin, int n, const float *__restrict__ rmsw, float4 *xs,
+                                                   float *sumx, float *red, int T, const Poll &pl)
 {
     const int nch = n >> 4, nq = n >> 2, tid = phase_tid();
     const int S = T;  // n <= 4 * WORDS * T is checked on the host
-    float4 v[WORDS], w[WORDS];
     float ssq = 0.0f;
 #pragma unroll
     for (int k = 0; k < WORDS; k++) {
-        v[k] = w[k] = make_float4(0.f, 0.f, 0.f, 0.f);
         const int i = tid + k * S;
+        float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
         if (i < nq) {
-            if (rmsw) w[k] = reinterpret_cast<const float4 *>(rmsw)[i];
-            v[k] = wait_word(xin + 4 * i, pl);
-        }
-        ssq += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
-    }
-    float ss = 1.0f;
-    if (rmsw) {
-        ssq = block_sum(ssq, red, T >> 6);
-        // ss /= size; ss += 1e-5f; ss = 1.0f / sqrt(ss)   (K/RootMeanSquare.java:31-33)
-        ss = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ssq, (float)n), 1e-5f)));
-    }
-#pragma unroll
-    for (int k = 0; k < WORDS; k++) {
-        const int i = tid + k * S;
-        float4 xv = v[k];
-        if (rmsw) {  // out = weight * (ss * x)   (K/WeightNormalizeAndScale.java:73)
-            xv.x = __fmul_rn(w[k].x, __fmul_rn(ss, xv.x));
-            xv.y = __fmul_rn(w[k].y, __fmul_rn(ss, xv.y));
-            xv.z = __fmul_rn(w[k].z, __fmul_rn(ss, xv.z));
-            xv.w = __fmul_rn(w[k].w, __fmul_rn(ss, xv.w));
+            float4 wv = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (rmsw) wv = reinterpret_cast<const float4 *>(rmsw)[i];
+            xv = wait_word(xin + 4 * i, pl);
+            ssq += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
+            if (rmsw) {
+                xv.x = __fmul_rn(wv.x, xv.x);
+                xv.y = __fmul_rn(wv.y, xv.y);
+                xv.z = __fmul_rn(wv.z, xv.z);
+                xv.w = __fmul_rn(wv.w, xv.w);
+            }
         }
         const float s0 = (xv.x + xv.y) + (xv.z + xv.w);
         const float s1 = dpp_f<0x55>(s0), s2 = dpp_f<0xAA>(s0), s3 = dpp_f<0xFF>(s0);  // quad lanes 1, 2, 3
@@ -327,7 +312,12 @@ __device__ __forceinline__ void stage_vector_poll(const float *__restrict__ xin,
             if ((i & 3) == 0) sumx[i >> 2] = ((s0 + s1) + s2) + s3;
         }
     }
+    if (rmsw) {
+        ssq = wave_sum(ssq);
+        if ((tid & 63) == 0) red[tid >> 6] = ssq;
+    }
     __syncthreads();
+    return rmsw ? rms_scalar(red, T >> 6, n) : 1.0f;
 }
 
 // The number of splits per head the attention phase uses at a position, and the rows of each.
@@ -599,11 +589,16 @@ struct MatvecRun {
     }
 
     // Reduces the sums of the resolved item over the wave, applies the phase's epilogue and stores the results.
+    // ss: the rmsnorm scalar of the input vector, which was staged without it (stage_vector); 1 for phases without a norm.
     template <bool COH>
-    __device__ __forceinline__ void finish(int it, int wh, int rr, float acc0, float acc1, float resv0, float resv1, int pos)
+    __device__ __forceinline__ void finish(int it, int wh, int rr, float acc0, float acc1, float resv0, float resv1, int pos, float ss)
     {
         acc0 = wave_sum(acc0);
         acc1 = wave_sum(acc1);
+        if (MODE == PH_QKV || MODE == PH_W13) {
+            acc0 = __fmul_rn(ss, acc0);
+            acc1 = __fmul_rn(ss, acc1);
+        }
         if (lane == 0) {
             float v0, v1 = 0.0f;
             if (MODE == PH_QKV) {
@@ -651,10 +646,11 @@ struct MatvecRun {
         float *red = sumx + nch;
         const float *emb_row = d.emb + (long)token * n;  // J/Run.java:72 (only used when n == dim)
         const float *res = d.res_emb ? emb_row : d.res_src;
+        float ss;
         if (d.poll.on && !d.from_emb) {
-            stage_vector_poll<kPollWords>(d.xin, n, d.rmsw, xs, sumx, red, d.threads, d.poll);
+            ss = stage_vector_poll<kPollWords>(d.xin, n, d.rmsw, xs, sumx, red, d.threads, d.poll);
         } else {
-            stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
+            ss = stage_vector(d.from_emb ? emb_row : d.xin, n, d.rmsw, xs, sumx, red, d.threads);
         }
 
         if (item >= nitems) return;
@@ -689,7 +685,7 @@ struct MatvecRun {
             }
             fold<true>(base, xs, sumx, acc0, acc1, nbase);
             if (last_step) {
-                finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos);
+                finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos, ss);
                 cur = nitem; cur_which = which; cur_r = r;
                 resv0 = nres0; resv1 = nres1;
                 acc0 = acc1 = 0.0f;
@@ -697,7 +693,7 @@ struct MatvecRun {
             base = nbase;
         }
         fold<false>(base, xs, sumx, acc0, acc1, 0);
-        finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos);
+        finish<COH>(cur, cur_which, cur_r, acc0, acc1, resv0, resv1, pos, ss);
         item = nitems;
     }
 };
@@ -1063,10 +1059,11 @@ struct ClsRun {
         float *red = sumx + nch;
         float *bval = red + 16;
         int *bidx = reinterpret_cast<int *>(red + 32);
+        float ss;
         if (a.poll.on) {
-            stage_vector_poll<kPollWords>(a.xin, n, a.rmsw, xs, sumx, red, a.threads, a.poll);
+            ss = stage_vector_poll<kPollWords>(a.xin, n, a.rmsw, xs, sumx, red, a.threads, a.poll);
         } else {
-            stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
+            ss = stage_vector(a.xin, n, a.rmsw, xs, sumx, red, a.threads);
         }
 
         float best_v = -__builtin_inff();
@@ -1086,7 +1083,7 @@ struct ClsRun {
                 }
             }
             first = false;
-            acc = wave_sum(acc);
+            acc = __fmul_rn(ss, wave_sum(acc));
             if (lane == 0) {
                 a.logits[row] = acc;
                 if (better(acc, row, best_v, best_i)) { best_v = acc; best_i = row; }
