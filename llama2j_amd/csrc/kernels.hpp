@@ -163,15 +163,35 @@ __device__ __forceinline__ float dot4(const float4 a, const float4 b)
     return fmaf(a.w, b.w, fmaf(a.z, b.z, fmaf(a.y, b.y, a.x * b.x)));
 }
 
+// Two consecutive floats of a read-only table at a wave-uniform address, through the scalar data path: a scalar load
+// does not queue behind the wave's outstanding vector loads (weights requested ahead), which return in order.
+__device__ __forceinline__ float2 uniform_pair(const float *p)
+{
+    const unsigned long long a = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+    const unsigned long long ua = ((unsigned long long)hi << 32) | lo;
+    unsigned long long v;
+    asm volatile("s_load_dwordx2 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ua) : "memory");
+    return make_float2(__uint_as_float((unsigned)v), __uint_as_float((unsigned)(v >> 32)));
+}
+
 // The reference's sigmoid: 8192-entry table on [-5,5) with linear interpolation and the integer
 // index multiplier 819 (K/Silu.java:41-70); exact outside the table.
+// UNIFORM: val is the same in every lane (a wave's row sum): the two table entries come through the scalar data path.
+template <bool UNIFORM = false>
 __device__ __forceinline__ float silu_sigma(const float *__restrict__ table, float val, int exact)
 {
     const float position = __fmul_rn(__fadd_rn(val, 5.0f), 819.0f);
     if (!exact && position > 0.0f && position < 8191.0f) {
         const int idx = (int)position;
-        const float lo = table[idx];
-        return __fadd_rn(lo, __fmul_rn(__fsub_rn(position, (float)idx), __fsub_rn(table[idx + 1], lo)));
+        float lo, hi;
+        if (UNIFORM) {
+            const float2 t = uniform_pair(table + idx);
+            lo = t.x; hi = t.y;
+        } else {
+            lo = table[idx]; hi = table[idx + 1];
+        }
+        return __fadd_rn(lo, __fmul_rn(__fsub_rn(position, (float)idx), __fsub_rn(hi, lo)));
     }
     // outside the table (|val| >= 5, saturated): the reference evaluates this in double and narrows;
     // fp32 differs by at most a couple of ulp
