@@ -30,6 +30,9 @@ WORKLOADS = {
     "stories110m-shape": ((768, 2048, 12, 12, 12, 32000, 1024, 1), 102, 16),
     "stories15m-shape": ((288, 768, 6, 6, 6, 32000, 256, 1), 101, 8),
 }
+# steps of a workload when --steps is not given: its prompt ids + the generated tokens BASELINE.json's configuration names
+DEFAULT_STEPS = {"llama2-7b-shape": 32 + 256, "llama2-13b-shape": 32 + 256, "llama2-70b-shape": 32 + 128,
+                 "llama2-7b-long-context": 4096, "stories110m-shape": 16 + 512, "stories15m-shape": 8 + 248}
 HBM_PEAK_GBS = 8000.0
 
 
@@ -124,7 +127,8 @@ def cpu_baseline_long_context(shape, seed, g, gpu_tokens, positions):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=288, help="tokens decoded in the timed region (32 prompt + 256 greedy)")
+    ap.add_argument("--steps", type=int, default=0,
+                    help="tokens decoded in the timed region (default: the configuration's own length, e.g. 32 prompt + 256 greedy = 288)")
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--workload", default="llama2-7b-shape", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-steps", type=int, default=97, help="forwards of the CPU baseline sample (0 = skip)")
@@ -143,7 +147,11 @@ def main():
     from llama2j_amd import KERNEL
 
     shape, seed, n_prompt = WORKLOADS[a.workload]
-    steps = min(a.steps, shape[6])
+    steps = min(a.steps if a.steps > 0 else DEFAULT_STEPS[a.workload], shape[6])
+    if not a.workload.endswith("long-context") and steps <= n_prompt:
+        # a short run (the driver's --steps 20): half of it forced prompt ids, half generated tokens, so that the timed
+        # run and the CPU leg share generated positions
+        n_prompt = steps // 2
     g = l2j.Transformer(l2j.Config(*shape))
     t0 = time.time()
     g.fill_synthetic(seed, 0.02)
@@ -224,8 +232,11 @@ def main():
             stoks, _ = g.decode_sample(prompt, steps, 0.9, 0.9, 12345)
             g.sync()
             swall = time.perf_counter() - t0
-            out["sampled_decode"] = {"temperature": 0.9, "topp": 0.9, "rng_seed": 12345, "steps": int(len(stoks)),
-                                     "tok_s": round(len(stoks) / swall, 2), "ms_per_step": round(swall / len(stoks) * 1e3, 4)}
+            n_sampled = max(0, int(len(stoks)) - n_prompt)   # forced positions run no sampler
+            if n_sampled > 0:
+                out["sampled_decode"] = {"temperature": 0.9, "topp": 0.9, "rng_seed": 12345, "steps": int(len(stoks)),
+                                         "sampled_positions": n_sampled, "forced_positions": int(len(stoks)) - n_sampled,
+                                         "tok_s": round(len(stoks) / swall, 2), "ms_per_step": round(swall / len(stoks) * 1e3, 4)}
         except l2j.L2JError as e:  # a vocabulary above the device sampler's limit
             out["sampled_decode"] = {"error": str(e)}
         g.reset()
@@ -279,13 +290,16 @@ def main():
                     (32 if dom_name == "token" else 3, pos))
         if dom_name == "token" and sec_after_first > 0 and done > 1:
             # The timed decode itself: its stream holds nothing but one k_token launch per token, back to back (32 per graph
-            # replay), and l2j_decode_greedy brackets launches 1 .. done - 1 with two HIP events on that stream.  (An event
-            # pair around every single launch, as in "kernels" above, adds about 2 % to each.)
+            # replay); the workgroup that ends a token stores the device's wall clock in its loop step, and
+            # l2j_decode_greedy returns the difference between the stamps of the first and the last token.  (An event pair
+            # around every single launch, as in "kernels" above, adds about 2 % to each.)
             us = sec_after_first / (done - 1) * 1e6
             dom = {"us": round(us, 3), "bytes": bytes_tok, "GBps": round(bytes_tok / us * 1e-3, 1),
                    "frac": round(bytes_tok / us * 1e-3 / HBM_PEAK_GBS, 4)}
-            measured = ("two HIP events on the decode's stream around the %d launches of k_token that follow the first token's "
-                        "(positions 1-%d, nothing else on the stream); bytes at the mean position %d" % (done - 1, done - 1, pos))
+            measured = ("device wall-clock stamps (s_memrealtime at %d kHz, hipDeviceAttributeWallClockRate) stored by the last "
+                        "workgroup of each k_token launch in its loop step: (stamp of position %d - stamp of position 0) / %d, the "
+                        "launch-to-launch period of the %d launches that follow the first token's (nothing else is on the "
+                        "stream); bytes at the mean position %d" % (g.get_option("wall_clock_khz"), done - 1, done - 1, done - 1, pos))
         ct = COUNTER_TRAFFIC.get(a.workload) if dom_name == "token" else None
         out["roofline"] = {"bound": "hbm",
                            "kernel": "k_token (all phases of all layers + classifier), one launch per token" if dom_name == "token"

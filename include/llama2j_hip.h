@@ -92,7 +92,8 @@ int l2j_device_count(void);
  * replay in the decode loops).  At any time: "sampler_scan", "sampler_exp_wgs", "fallback" (1: when a bounded wait of the
  * whole-token kernel runs out, because something else holds compute units of the GPU, the context switches to one launch
  * per phase for good and repeats the call; 0: the call returns L2J_E_HIP).  l2j_get_option reads the value in force
- * ("fuse" reads 0 after such a switch). */
+ * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
+ * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
 int l2j_get_option(l2j_ctx *ctx, const char *name, int32_t *value);
 
@@ -131,7 +132,10 @@ int l2j_forward_taps(l2j_ctx *ctx, int32_t token, int32_t pos, float *logits_or_
  * prompt ids forced as outputs, first-max argmax afterwards, stop after emitting token 1.
  * out_tokens (capacity min(steps, seq_len), or seq_len when steps <= 0) receives `next` of every
  * executed iteration, *n_out the final pos.  *seconds (may be NULL) = GPU time from the end of
- * the first iteration to the end of the last one (J/Run.java:682-684, 703-706). */
+ * the first iteration to the end of the last one (J/Run.java:682-684, 703-706): the last workgroup of every token
+ * stores the device's wall clock (s_memrealtime, rate = hipDeviceAttributeWallClockRate, which
+ * l2j_get_option("wall_clock_khz") reports) in its loop step, and *seconds is the difference of the two stamps;
+ * 0 when the device does not tell the clock's rate. */
 int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps,
                       int32_t *out_tokens, int32_t *n_out, double *seconds);
 
@@ -144,8 +148,11 @@ int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int
  * exactly, an fp32 activation is cut exactly into three bf16, the products are exact and the sums fp32 (the fp32
  * classifier runs on the fp32 matrix cores); sums are formed in another order than in the single-sequence path, so
  * logits agree to rounding, not bit for bit.  The first call makes a second copy of the quantized matrices on the
- * device, in the order this path reads them (freed by l2j_destroy); every call allocates its own activation buffers
- * and a KV cache of n_seq x steps rows per layer and frees them when it returns; the context's cache is not touched.
+ * device, in the order this path reads them (as large as the matrices themselves: 6.9 GB at the 7B shape), its
+ * activation buffers, a KV cache of n_seq x steps rows per layer and the captured graph of a step; the context keeps
+ * them until l2j_destroy, so later calls allocate and capture nothing unless they ask for another n_seq, more steps or
+ * longer prompts (then the set is replaced).  The context's own cache is not touched.  L2J_E_OOM when the device
+ * memory does not suffice (n_seq x n_layers x steps x kv_dim x 8 bytes of cache).
  * Needs dim and hidden_dim in whole groups of 256 and head_size 64, 128 or 256.
  * *seconds (may be NULL): GPU time from the end of the first step to the end of the last. */
 int l2j_decode_greedy_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,
@@ -227,13 +234,20 @@ int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
  * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
  * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
 int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
-/* l2j_running_sums for callers that cannot allocate device memory (code under hipGraph capture, serving loops,
- * harnesses that forbid it); it has no counterpart in the reference.  Same results, but the terms and sums pass
- * through a fixed 144 KB device array of the library (one per GPU, held until the process ends) instead of a buffer
- * allocated per call: n <= 36864, else L2J_E_SIZE.  No hipMalloc / hipFree is made.  Every call on a GPU shares that
- * GPU's array, so calls that overlapped would race: the library runs them one after the other.  The array keeps the last
- * call's contents; a call reads none of them (it only reads the n terms it has just copied in). */
+/* l2j_running_sums for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, code that runs while another thread captures a graph); it has no counterpart in the reference.  Same
+ * results, but the terms and sums pass through a fixed 144 KB device array of the library (one per GPU, held until the
+ * process ends) instead of a buffer allocated per call: n <= 36864, else L2J_E_SIZE.  No hipMalloc / hipFree is made;
+ * the call does copy from and to the caller's host memory and synchronizes the context's stream, so it is not itself
+ * something to record into a capture.  Every call on a GPU shares that GPU's array, so calls that overlapped would race:
+ * the library runs them one after the other.  The array keeps the last call's contents; a call reads none of them (it
+ * only reads the n terms it has just copied in). */
 int l2j_running_sums_noalloc(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
+/* Test: l2j_decode_greedy_batch that also returns the logits of every step, (steps, n_seq, vocab_size) floats, so that
+ * the batched path's arithmetic can be compared with the single-sequence path's and the CPU's step by step (they pass
+ * through a device buffer of that size, allocated for the call). */
+int l2j_decode_greedy_batch_logits(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,
+                                   int32_t prompt_stride, int32_t steps, int32_t *out_tokens, float *logits);
 /* Measurement and test of the matrix-core kernel for several sequences at once (the reference has none: "parallel
  * processing of multiple queries" is on its wish-list, README.md:347): y[b][r] = sum_k dequant(W[r][k]) * x[b][k] for
  * sixteen activation vectors x (16 x K floats) against one layer's matrix of a quantized matrix tensor (L2J_WQ..L2J_W3;

@@ -115,6 +115,7 @@ def _signatures():
         "l2j_time_kernel": (C.c_int, [vp, C.c_int, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]),
         "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
         "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
+        "l2j_decode_greedy_batch_logits": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, fp]),
         "l2j_batch_matmul": (C.c_int, [vp, C.c_int, C.c_int, fp, fp, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
         "l2j_bytes_per_token": (C.c_uint64, [cfgp, C.c_int32]),
         "l2j_quant_nbytes": (C.c_uint64, [C.c_uint64]),
@@ -420,10 +421,11 @@ class Transformer:
         self._check(lib().l2j_running_sums_noalloc(self._h, _fp(terms), terms.size, _fp(out)))
         return out
 
-    def decode_greedy_batch(self, prompts, steps, n_seq=None):
+    def decode_greedy_batch(self, prompts, steps, n_seq=None, want_logits=False):
         """Sixteen or thirty-two greedy token loops at once (l2j_decode_greedy_batch).  prompts: up to n_seq id sequences
         (missing ones run without a prompt; n_seq defaults to 16, or 32 for more than sixteen prompts); returns (tokens of
-        shape (n_seq, steps), seconds after the first step)."""
+        shape (n_seq, steps), seconds after the first step), or with want_logits (tokens, logits of shape (steps, n_seq,
+        vocab_size)) through l2j_decode_greedy_batch_logits."""
         if n_seq is None:
             n_seq = 16 if len(prompts) <= 16 else 32
         assert len(prompts) <= n_seq
@@ -434,6 +436,10 @@ class Transformer:
             ids[b, :len(p)] = p
             n[b] = len(p)
         out = np.zeros((n_seq, steps), dtype=np.int32)
+        if want_logits:
+            logits = np.empty((steps, n_seq, self.config.vocab_size), dtype=np.float32)
+            self._check(lib().l2j_decode_greedy_batch_logits(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), _fp(logits)))
+            return out, logits
         sec = C.c_double(0.0)
         self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), C.byref(sec)))
         return out, sec.value

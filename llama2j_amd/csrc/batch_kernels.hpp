@@ -47,7 +47,7 @@ __host__ __device__ inline int bg_units(int rows, int tiles) { return (rows + 16
 // (row by row a wave's instruction touches 16 rows, 64 bytes each: a third slower, measured); the blocks of a tile
 // follow each other group by group, then come those of the next tile.  The scales likewise: 16 (rm, min) per block.
 // One thread per 16 codes of the whole tensor (layers x rows x K); rows % 16 == 0, K % 256 == 0.
-__global__ void __launch_bounds__(256) k_btile(const uint8_t *__restrict__ codes, const float2 *__restrict__ gs, long n16, int rows, int K,
+static __global__ void __launch_bounds__(256) k_btile(const uint8_t *__restrict__ codes, const float2 *__restrict__ gs, long n16, int rows, int K,
                                                uint8_t *__restrict__ tcodes, float2 *__restrict__ tgs)
 {
     const long o = (long)blockIdx.x * 256 + threadIdx.x;   // index of the 16 codes in the tiled copy
@@ -399,7 +399,7 @@ struct BatchState {
 };
 
 // x[b] = row token[b] of the embedding table (J/Run.java:72)
-__global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, const BatchState *st, float *__restrict__ x, int dim)
+static __global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, const BatchState *st, float *__restrict__ x, int dim)
 {
     const int b = blockIdx.x;
     const float4 *src = reinterpret_cast<const float4 *>(emb + (long)st->token[b] * dim);
@@ -409,7 +409,7 @@ __global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, c
 
 // xn[b] = w * (ss * x[b]), ss = 1 / sqrt(sum(x^2) / n + 1e-5) (K/RootMeanSquare.java:25-35, K/WeightNormalizeAndScale.java:73).
 // One workgroup of 1024 threads per sequence.
-__global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ xn, int n)
+static __global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ xn, int n)
 {
     __shared__ float red[16];
     const int b = blockIdx.x, tid = threadIdx.x, n4 = n >> 2;
@@ -436,7 +436,7 @@ __global__ void __launch_bounds__(1024) k_brms(const float *__restrict__ x, cons
 
 // x[b] += the slices of a product summed in order (K/Accum.java:26-30), then xn[b] as k_brms does: the
 // hand-over from Wo to W1/W3 and from W2 to the next layer's Wq/Wk/Wv (or to the classifier) in one kernel.
-__global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ part, int slices, float *__restrict__ x, const float *__restrict__ w,
+static __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ part, int slices, float *__restrict__ x, const float *__restrict__ w,
                                                    float *__restrict__ xn, int n)
 {
     __shared__ float red[16];
@@ -474,7 +474,7 @@ __global__ void __launch_bounds__(1024) k_bres_rms(const float *__restrict__ par
 
 // hb[b][r] = silu(h1) * h3 with the reference's sigmoid table (K/Silu.java:72-74), h1 and h3 the slices summed in order.
 // grid (hidden / 256, sequences), 256 threads.
-__global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p1, const float *__restrict__ p3, int slices, int hidden,
+static __global__ void __launch_bounds__(256) k_bepi_swiglu(const float *__restrict__ p1, const float *__restrict__ p3, int slices, int hidden,
                                                      const float *__restrict__ silu, int exact, float *__restrict__ hb)
 {
     const int b = blockIdx.y, rix = blockIdx.x * 256 + threadIdx.x;
@@ -607,7 +607,7 @@ struct BNext {
 // Logits of every sequence (the slices summed in order), first index of the maximum (J/Sampler.java:46-57) and the step of
 // the token loop (J/Run.java:635-642, 668, 680): forced prompt id or argmax.  One workgroup per sequence; the last
 // workgroup to finish advances the position.
-__global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *done)
+static __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *done)
 {
     __shared__ float bval[16];
     __shared__ int bidx[16];
@@ -647,7 +647,7 @@ __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *done)
 }
 
 // y[b][r] = sum over the slices, in slice order
-__global__ void __launch_bounds__(256) k_breduce(const float *__restrict__ part, float *__restrict__ y, int rows, int slices)
+static __global__ void __launch_bounds__(256) k_breduce(const float *__restrict__ part, float *__restrict__ y, int rows, int slices)
 {
     const long n = (long)kBatch * rows;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {

@@ -219,7 +219,7 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) { retur
 __device__ __forceinline__ float be_bits_to_float(uint32_t le_loaded) { return __builtin_bit_cast(float, __builtin_bswap32(le_loaded)); }
 
 // One 64-thread block per group: 264 reference bytes -> 256 codes + (rm, min) + (min, max).
-__global__ void __launch_bounds__(64) k_unpack_groups(const uint8_t *__restrict__ ref, long ngroups, uint8_t *__restrict__ codes,
+static __global__ void __launch_bounds__(64) k_unpack_groups(const uint8_t *__restrict__ ref, long ngroups, uint8_t *__restrict__ codes,
                                                       float2 *__restrict__ gs, float2 *__restrict__ mm)
 {
     for (long g = blockIdx.x; g < ngroups; g += gridDim.x) {
@@ -233,7 +233,7 @@ __global__ void __launch_bounds__(64) k_unpack_groups(const uint8_t *__restrict_
     }
 }
 
-__global__ void __launch_bounds__(64) k_pack_groups(uint8_t *__restrict__ ref, long ngroups, const uint8_t *__restrict__ codes,
+static __global__ void __launch_bounds__(64) k_pack_groups(uint8_t *__restrict__ ref, long ngroups, const uint8_t *__restrict__ codes,
                                                     const float2 *__restrict__ mm)
 {
     for (long g = blockIdx.x; g < ngroups; g += gridDim.x) {
@@ -262,7 +262,7 @@ __device__ __forceinline__ float synth_value(uint64_t base, long i, float scale)
     return __fmul_rn((float)s, scale);
 }
 
-__global__ void k_synth_f32(float *__restrict__ out, long n, uint64_t base, float scale)
+static __global__ void k_synth_f32(float *__restrict__ out, long n, uint64_t base, float scale)
 {
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
         out[i] = synth_value(base, i, scale);
@@ -270,7 +270,7 @@ __global__ void k_synth_f32(float *__restrict__ out, long n, uint64_t base, floa
 
 // Quant.encode (J/Quant.java:156-193), one 256-thread block per group.  Source is either fp32
 // data (src != null, float index 0 = first float of group `g0`) or the seeded generator.
-__global__ void __launch_bounds__(256) k_encode_groups(const float *__restrict__ src, long n_src, long g0, long ngroups,
+static __global__ void __launch_bounds__(256) k_encode_groups(const float *__restrict__ src, long n_src, long g0, long ngroups,
                                                        long tensor_floats, uint64_t synth_base, float synth_scale,
                                                        uint8_t *__restrict__ codes, float2 *__restrict__ gs, float2 *__restrict__ mm)
 {
@@ -307,7 +307,7 @@ __global__ void __launch_bounds__(256) k_encode_groups(const float *__restrict__
 }
 
 // Plain copy of n 16-byte words: the known-size kernel against which hardware byte counters are scaled.
-__global__ void __launch_bounds__(256) k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, long n)
+static __global__ void __launch_bounds__(256) k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, long n)
 {
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) dst[i] = src[i];
 }

@@ -1,0 +1,427 @@
+// libllama2j_hip.so: several sequences at once (l2j_decode_greedy_batch, l2j_batch_matmul).
+#include "l2j_internal.hpp"
+#include "batch_kernels.hpp"
+
+using namespace l2j;
+
+static bool matrix_shape(const l2j_config &cf, int tensor, int *rows, int *K)
+{
+    const int kvd = cf.dim / cf.n_heads * cf.n_kv_heads;
+    switch (tensor) {
+    case L2J_WQ: case L2J_WO: *rows = cf.dim; *K = cf.dim; return true;
+    case L2J_WK: case L2J_WV: *rows = kvd; *K = cf.dim; return true;
+    case L2J_W1: case L2J_W3: *rows = cf.hidden_dim; *K = cf.dim; return true;
+    case L2J_W2: *rows = cf.dim; *K = cf.hidden_dim; return true;
+    default: return false;
+    }
+}
+
+// The tile-ordered copy of `tensor` for the batched path (rows % 16 == 0 and K % 256 == 0 checked by the caller; the
+// caller holds the context's upload lock: an upload of the tensor marks the copy stale, invalidate_batch_tiles).
+static int ensure_batch_tiles(l2j_ctx *c, int tensor)
+{
+    if (c->bt_done[tensor]) return L2J_OK;
+    int rows = 0, K = 0;
+    if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
+    const QTensor &t = c->qt[tensor];
+    if (t.groups_loaded < t.ngroups) return fail(L2J_E_STATE, "tensor not uploaded");
+    const uint64_t n = (uint64_t)c->cfg.n_layers * rows * K;
+    int rc;
+    if (!c->bt_codes[tensor] && (rc = dev_alloc(&c->bt_codes[tensor], n))) return rc;
+    if (!c->bt_gs[tensor] && (rc = dev_alloc(&c->bt_gs[tensor], n / 256))) return rc;
+    const long n16 = (long)(n / 16);
+    hipLaunchKernelGGL(k_btile, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, c->stream, t.codes, t.gs, n16, rows, K, c->bt_codes[tensor],
+                       c->bt_gs[tensor]);
+    HIPCHK(hipGetLastError());
+    c->bt_done[tensor] = true;
+    return L2J_OK;
+}
+
+static QMat bqmat(const l2j_ctx *c, int t, uint64_t off)
+{
+    QMat m;
+    m.codes = c->bt_codes[t];
+    m.gs = c->bt_gs[t];
+    m.off = (long)off;
+    return m;
+}
+
+extern "C" {
+
+int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y, int32_t groups_per_slice, int32_t rounds,
+                     double *mean_us)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !x || !y) return fail(L2J_E_ARG, "null argument");
+        int rows = 0, K = 0;
+        if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
+        if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
+        if (K % 256 || rows % 16) return fail(L2J_E_SIZE, "the batched matrix product needs rows of whole groups (K % 256 == 0) and rows % 16 == 0");
+        const int ngroups = K / 256, gps = std::max(1, std::min(std::min(ngroups, kBgMaxGps), (int)groups_per_slice));
+        const int slices = (ngroups + gps - 1) / gps;
+        const size_t lds = bg_lds_bytes(gps, kBatch);
+        if (lds + sizeof(float) * kBatch * kBgMaxGps > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        {
+            std::lock_guard<std::mutex> lock(c->upload_mu);
+            const int trc = ensure_batch_tiles(c, tensor);
+            if (trc) return trc;
+        }
+        float *dx = nullptr, *dpart = nullptr, *dy = nullptr;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        auto release = [&]() {
+            (void)hipFree(dx); (void)hipFree(dpart); (void)hipFree(dy);
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+        };
+        hipError_t e = hipMalloc(reinterpret_cast<void **>(&dx), (size_t)kBatch * K * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dpart), (size_t)slices * kBatch * rows * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
+        if (e == hipSuccess) e = hipEventCreate(&e0);
+        if (e == hipSuccess) e = hipEventCreate(&e1);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        if (e == hipSuccess) {
+            BGemm a{};
+            a.m[0] = bqmat(c, tensor, (uint64_t)layer * rows * K);
+            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
+            const dim3 grid((bg_units(rows, 2) + 3) / 4, slices);
+            const int n = std::max(1, (int)rounds);
+            hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);   // warm
+            (void)hipEventRecord(e0, c->stream);
+            for (int i = 0; i < n; i++) hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);
+            (void)hipEventRecord(e1, c->stream);
+            hipLaunchKernelGGL(k_breduce, dim3(256), dim3(256), 0, c->stream, dpart, dy, rows, slices);
+            e = hipGetLastError();
+            if (e == hipSuccess) e = hipMemcpyAsync(y, dy, (size_t)kBatch * rows * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+            float ms = 0.0f;
+            if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+            if (mean_us) *mean_us = (double)ms * 1e3 / n;
+        }
+        release();
+        if (e != hipSuccess) return fail(e == hipErrorOutOfMemory ? L2J_E_OOM : L2J_E_HIP, std::string("batch matmul: ") + hipGetErrorString(e));
+        return L2J_OK;
+    }());
+}
+
+}  // extern "C"
+
+// ---- several sequences at once ----------------------------------------------------------------------------------
+
+// Device memory, pinned staging and the captured step of the batched decode.  The context owns one set, made by the first
+// l2j_decode_greedy_batch and kept until l2j_destroy; a call that needs more (other sequence count, more steps, longer
+// prompts) replaces it.  No call allocates or captures anything once the set fits.
+struct l2j::BatchBufs {
+    int nseq = 0, cap_steps = 0, cap_pstride = 0;   // what the buffers and the graph's kernel arguments are made for
+    float *x = nullptr, *xn = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
+    float *part[3] = {nullptr, nullptr, nullptr};
+    float *kc = nullptr, *vc = nullptr;             // (sequence, layer, cap_steps, kv_dim)
+    BatchState *st = nullptr;
+    int *prompts = nullptr, *out = nullptr;         // (sequence, cap_pstride), (sequence, cap_steps)
+    unsigned *done = nullptr;
+    int *h_pin = nullptr;   // pinned: every transfer of a call goes through it, as in the single-sequence loops
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    void release()
+    {
+        if (exec) (void)hipGraphExecDestroy(exec);
+        if (graph) (void)hipGraphDestroy(graph);
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+        void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
+        for (void *p : ps) (void)hipFree(p);
+        if (h_pin) (void)hipHostFree(h_pin);
+    }
+};
+
+void l2j::free_batch(l2j_ctx *c)
+{
+    if (c->batch) {
+        c->batch->release();
+        delete c->batch;
+        c->batch = nullptr;
+    }
+    for (int t = 0; t < L2J_TENSOR_COUNT; t++) {
+        (void)hipFree(c->bt_codes[t]);
+        (void)hipFree(c->bt_gs[t]);
+        c->bt_codes[t] = nullptr; c->bt_gs[t] = nullptr; c->bt_done[t] = false;
+    }
+    c->bt_ready = false;
+}
+
+void l2j::invalidate_batch_tiles(l2j_ctx *c, int tensor)
+{
+    c->bt_done[tensor] = false;
+    c->bt_ready = false;
+}
+
+namespace {
+
+constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
+
+int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
+size_t batch_lds(int nseq) { return bg_lds_bytes(kBatchGps, nseq); }   // k_bgemm: bf16 planes
+size_t batch_lds_f32(int nseq) { return (size_t)nseq * (kBatchGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
+// workgroups of k_bgemm a compute unit holds at once: its 160 KB of LDS, and at most three by their registers
+int batch_resident(int nseq) { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds(nseq) + sizeof(float) * nseq * kBgMaxGps)))); }
+
+// The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
+void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part, int nseq)
+{
+    BGemm a{};
+    int K = 0;
+    for (int tensor : tensors) {
+        int rows = 0;
+        matrix_shape(c->cfg, tensor, &rows, &K);
+        a.m[a.nmat] = bqmat(c, tensor, (uint64_t)layer * rows * K);
+        a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
+        a.nmat++;
+    }
+    a.K = K; a.x = x; a.gps = kBatchGps;
+    // All workgroups of the launch are resident at once (batch_resident() per compute unit); a wave takes one unit of 16 or 32 rows
+    // after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
+    // activations they fetch from LDS).
+    const int nb = nseq / kBatch, waves = 4 * nb;
+    const int S = batch_slices(K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
+    int tiles = 2, gx = 1, best = 1 << 30;
+    for (int t = 2; t >= 1; t--) {
+        int units = 0;
+        for (int i = 0; i < a.nmat; i++) units += bg_units(a.rows[i], t);
+        const int g = std::min(gmax, (units + waves - 1) / waves), iters = (units + waves * g - 1) / (waves * g);
+        if (iters * t < best) {
+            best = iters * t; tiles = t;
+            gx = (units + waves * iters - 1) / (waves * iters);   // no more workgroups than that many rounds need
+        }
+    }
+    const dim3 grid(gx, S), block(kBgThreads * nb);
+    const size_t lds = batch_lds(nseq);
+    if (nb == 1) {
+        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 1>), grid, block, lds, c->stream, a);
+        else hipLaunchKernelGGL((k_bgemm<2, 1>), grid, block, lds, c->stream, a);
+    } else {
+        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 2>), grid, block, lds, c->stream, a);
+        else hipLaunchKernelGGL((k_bgemm<2, 2>), grid, block, lds, c->stream, a);
+    }
+}
+
+// One position of all sequences: embedding, the layers, the classifier, the next tokens.
+void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride, int nseq)
+{
+    const l2j_config &cf = c->cfg;
+    const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim;
+    const int sd = batch_slices(dim), sh = batch_slices(hidden);
+    hipStream_t s = c->stream;
+    { hipLaunchKernelGGL(k_bembed, dim3(nseq), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
+    { hipLaunchKernelGGL(k_brms, dim3(nseq), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
+    for (int l = 0; l < L; l++) {
+        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part, nseq);
+        BAttn t{};
+        t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
+        t.kc = b.kc + (size_t)l * max_pos * kvd; t.vc = b.vc + (size_t)l * max_pos * kvd;
+        t.seq_stride = (long)L * max_pos; t.out = b.xb; t.st = b.st;
+        t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
+        t.sqrt_hs = sqrtf((float)hs);
+        const dim3 ag(cf.n_heads, nseq);
+        {
+            if (hs == 64) hipLaunchKernelGGL(k_battn<16>, ag, dim3(256), 0, s, t);
+            else if (hs == 128) hipLaunchKernelGGL(k_battn<32>, ag, dim3(256), 0, s, t);
+            else hipLaunchKernelGGL(k_battn<64>, ag, dim3(256), 0, s, t);
+        }
+        launch_bgemm(c, {L2J_WO}, l, b.xb, b.part, nseq);
+        { hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim); }
+        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.part, nseq);
+        { hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, nseq), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
+                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb); }
+        launch_bgemm(c, {L2J_W2}, l, b.hb, b.part, nseq);
+        // the residual, then the norm of what follows: the next layer's attention norm, or the final one (rmsw: att, ffn, final)
+        const float *wn = c->rmsw + (l + 1 < L ? (size_t)(l + 1) * dim : (size_t)2 * L * dim);
+        { hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, dim); }
+    }
+    {
+        BGemmF32 g{};
+        g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
+        const dim3 cg((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd);
+        if (nseq == kBatch) hipLaunchKernelGGL(k_bgemm_f32<1>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
+        else hipLaunchKernelGGL(k_bgemm_f32<2>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
+    }
+    BNext n{};
+    n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
+    n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
+    { hipLaunchKernelGGL(k_bnext, dim3(nseq), dim3(1024), 0, s, n, b.done); }
+}
+
+
+int hip_rc(hipError_t e, const char *what)
+{
+    return fail(e == hipErrorOutOfMemory ? L2J_E_OOM : L2J_E_HIP, std::string("batched decode: ") + what + ": " + hipGetErrorString(e));
+}
+
+// The context's buffers for n_seq sequences over `steps` positions with prompts of up to `pstride` ids: kept when they fit.
+int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
+{
+    BatchBufs *old = c->batch;
+    if (old && old->nseq == nseq && old->cap_steps >= steps && old->cap_pstride >= pstride) return L2J_OK;
+    if (old) {
+        hipError_t se = hipStreamSynchronize(c->stream);
+        if (se != hipSuccess) return hip_rc(se, "synchronize");
+        old->release();
+        delete old;
+        c->batch = nullptr;
+    }
+    const l2j_config &cf = c->cfg;
+    const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, kvd = c->kv_dim, vocab = cf.vocab_size;
+    const int sd = batch_slices(dim), sh = batch_slices(hidden);
+    const size_t part_floats = (size_t)nseq * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
+    const size_t cache_floats = (size_t)nseq * L * steps * kvd;
+    BatchBufs *b = new (std::nothrow) BatchBufs();
+    if (!b) return fail(L2J_E_OOM, "batched decode: host allocation failed");
+    b->nseq = nseq; b->cap_steps = steps; b->cap_pstride = pstride;
+    hipError_t e = hipSuccess;
+    auto alloc = [&](auto **p, size_t n) {
+        if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
+    };
+    alloc(&b->x, (size_t)nseq * dim); alloc(&b->xn, (size_t)nseq * std::max(dim, hidden));
+    alloc(&b->xb, (size_t)nseq * dim); alloc(&b->hb, (size_t)nseq * hidden); alloc(&b->logits, (size_t)nseq * vocab);
+    for (int i = 0; i < 3; i++) alloc(&b->part[i], part_floats);
+    alloc(&b->kc, cache_floats); alloc(&b->vc, cache_floats);
+    alloc(&b->st, 1); alloc(&b->prompts, (size_t)nseq * pstride); alloc(&b->out, (size_t)nseq * steps); alloc(&b->done, 1);
+    if (e == hipSuccess) e = hipEventCreate(&b->e0);
+    if (e == hipSuccess) e = hipEventCreate(&b->e1);
+    const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)nseq * pstride, out_ints = (size_t)nseq * steps;
+    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&b->h_pin), std::max(state_ints + prompt_ints, out_ints) * sizeof(int), hipHostMallocDefault);
+    const void *gemms[] = {(const void *)k_bgemm<1, 1>, (const void *)k_bgemm<2, 1>, (const void *)k_bgemm<1, 2>, (const void *)k_bgemm<2, 2>};
+    for (int i = 0; i < 4 && e == hipSuccess; i++)
+        e = hipFuncSetAttribute(gemms[i], hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(i < 2 ? kBatch : kMaxBatch));
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm_f32<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kBatch));
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm_f32<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kMaxBatch));
+    // one position as a graph: every kernel reads the position and the tokens from device memory, so the same nodes serve
+    // every step of every call ("graph" = 0: the kernels are launched one by one, for tools that do not follow graph launches)
+    if (e == hipSuccess && c->opt[OPT_GRAPH] != 0) {
+        e = hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            launch_batch_step(c, *b, steps, pstride, nseq);
+            const hipError_t le = hipGetLastError();
+            e = hipStreamEndCapture(c->stream, &b->graph);
+            if (e == hipSuccess) e = le;
+        }
+        if (e == hipSuccess) e = hipGraphInstantiate(&b->exec, b->graph, nullptr, nullptr, 0);
+    }
+    if (e != hipSuccess) {
+        b->release();
+        delete b;
+        return hip_rc(e, "set-up");
+    }
+    c->batch = b;
+    return L2J_OK;
+}
+
+// logits_log: null, or steps x n_seq x vocab_size floats of the caller that receive the logits of every step
+int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride, int32_t steps,
+                 int32_t *out_tokens, double *seconds, float *logits_log)
+{
+    if (!c || !n_prompt || !out_tokens || (prompt_stride > 0 && !prompts) || prompt_stride < 0) return fail(L2J_E_ARG, "bad argument");
+    if (!c->finalized) return fail(L2J_E_STATE, "decode before l2j_finalize");
+    if (n_seq != kBatch && n_seq != kMaxBatch) return fail(L2J_E_ARG, "n_seq must be 16 or 32");
+    const int nseq = n_seq;
+    const l2j_config &cf = c->cfg;
+    const int hs = c->head_size;
+    if (cf.dim % 256 || cf.hidden_dim % 256 || c->kv_dim % 16 || cf.vocab_size % 16 || (hs != 64 && hs != 128 && hs != 256))
+        return fail(L2J_E_SIZE, "batched decode needs dim and hidden_dim in whole groups of 256, kv_dim and vocab_size multiples of 16, "
+                                "head_size 64, 128 or 256");
+    if (steps <= 0 || steps > cf.seq_len) return fail(L2J_E_ARG, "steps must be 1..seq_len");
+    for (int b = 0; b < nseq; b++) {
+        if (n_prompt[b] < 0 || n_prompt[b] > prompt_stride) return fail(L2J_E_ARG, "n_prompt out of range");
+        for (int i = 0; i < n_prompt[b]; i++)
+            if (prompts[(size_t)b * prompt_stride + i] < 0 || prompts[(size_t)b * prompt_stride + i] >= cf.vocab_size)
+                return fail(L2J_E_ARG, "prompt id out of range");
+    }
+    HIPCHK(hipSetDevice(cf.device));
+    if (!c->bt_ready) {   // the matrices once more, in the order the batched products read them
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        for (int t : {L2J_WQ, L2J_WK, L2J_WV, L2J_WO, L2J_W1, L2J_W2, L2J_W3}) {
+            const int trc = ensure_batch_tiles(c, t);
+            if (trc) return trc;
+        }
+        c->bt_ready = true;
+    }
+    int rc = ensure_batch(c, nseq, steps, std::max(1, (int)prompt_stride));
+    if (rc) return rc;
+    BatchBufs &b = *c->batch;
+    const int vocab = cf.vocab_size, cap = b.cap_steps, pcap = b.cap_pstride;
+    const size_t state_ints = sizeof(BatchState) / sizeof(int);
+    float *dlog = nullptr;
+    if (logits_log) {
+        hipError_t me = hipMalloc(reinterpret_cast<void **>(&dlog), (size_t)steps * nseq * vocab * sizeof(float));
+        if (me != hipSuccess) return hip_rc(me, "logits of every step");
+    }
+    auto fail_hip = [&](hipError_t e, const char *what) {
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipFree(dlog);
+        return hip_rc(e, what);
+    };
+    BatchState h{};
+    h.pos = 0;
+    for (int i = 0; i < nseq; i++) { h.token[i] = 1; h.n_prompt[i] = n_prompt[i]; }   // BOS first (J/Run.java:612)
+    memcpy(b.h_pin, &h, sizeof(h));
+    memset(b.h_pin + state_ints, 0, (size_t)nseq * pcap * sizeof(int));
+    for (int s = 0; s < nseq && prompt_stride > 0; s++)
+        memcpy(b.h_pin + state_ints + (size_t)s * pcap, prompts + (size_t)s * prompt_stride, (size_t)n_prompt[s] * sizeof(int));
+    hipError_t e = hipMemcpyAsync(b.st, b.h_pin, sizeof(h), hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(b.prompts, b.h_pin + state_ints, (size_t)nseq * pcap * sizeof(int), hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(b.done, 0, sizeof(unsigned), c->stream);
+    if (e != hipSuccess) return fail_hip(e, "state upload");
+    for (int pos = 0; pos < steps && e == hipSuccess; pos++) {
+        if (b.exec) {
+            e = hipGraphLaunch(b.exec, c->stream);
+        } else {
+            launch_batch_step(c, b, cap, pcap, nseq);
+            e = hipGetLastError();
+        }
+        if (dlog && e == hipSuccess)
+            e = hipMemcpyAsync(dlog + (size_t)pos * nseq * vocab, b.logits, (size_t)nseq * vocab * sizeof(float), hipMemcpyDeviceToDevice, c->stream);
+        if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
+    }
+    if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(b.h_pin, b.out, (size_t)nseq * cap * sizeof(int), hipMemcpyDeviceToHost, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e != hipSuccess) return fail_hip(e, "step");
+    for (int s = 0; s < nseq; s++) memcpy(out_tokens + (size_t)s * steps, b.h_pin + (size_t)s * cap, (size_t)steps * sizeof(int));
+    if (dlog) {
+        e = hipMemcpy(logits_log, dlog, (size_t)steps * nseq * vocab * sizeof(float), hipMemcpyDeviceToHost);
+        (void)hipFree(dlog);
+        dlog = nullptr;
+        if (e != hipSuccess) return hip_rc(e, "logits read-back");
+    }
+    float ms = 0.0f;
+    if (steps > 1 && (e = hipEventElapsedTime(&ms, b.e0, b.e1)) != hipSuccess) return hip_rc(e, "timing");
+    if (seconds) *seconds = (double)ms * 1e-3;
+    return L2J_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride,
+                            int32_t steps, int32_t *out_tokens, double *seconds)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        return decode_batch(c, prompts, n_prompt, n_seq, prompt_stride, steps, out_tokens, seconds, nullptr);
+    }());
+}
+
+int l2j_decode_greedy_batch_logits(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride,
+                                   int32_t steps, int32_t *out_tokens, float *logits)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!logits) return fail(L2J_E_ARG, "null argument");
+        return decode_batch(c, prompts, n_prompt, n_seq, prompt_stride, steps, out_tokens, nullptr, logits);
+    }());
+}
+
+}  // extern "C"

@@ -1172,7 +1172,7 @@ struct ClsRun {
     }
 };
 
-__global__ void __launch_bounds__(1024) k_classifier(const ClsPhase a)
+static __global__ void __launch_bounds__(1024) k_classifier(const ClsPhase a)
 {
     extern __shared__ float4 smem4[];
     ClsRun run(a);
@@ -1324,7 +1324,7 @@ struct FillArgs {
     int nparts;
 };
 
-__global__ void k_fill_unset(const FillArgs a)
+static __global__ void k_fill_unset(const FillArgs a)
 {
     const float u = __uint_as_float(kUnset);
     const float4 u4 = make_float4(u, u, u, u);
@@ -1567,7 +1567,7 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
 
 // First index of the strict maximum (J/Sampler.java:46-57), then the token-loop step
 // (J/Run.java:635-642, 668, 680): forced prompt id or argmax, then advance.  One workgroup.
-__global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
+static __global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
 {
     __shared__ float bval[16];
     __shared__ int bidx[16];
@@ -1602,7 +1602,7 @@ __global__ void __launch_bounds__(1024) k_finish(const ClsPhase a)
 }
 
 // rmsnorm weights dequantized once (K/WeightNormalizeAndScale.java:71-72): value = byte / 255f * range + min
-__global__ void k_dequant_rms(const uint8_t *__restrict__ codes, const float2 *__restrict__ mm, long n, float *__restrict__ out)
+static __global__ void k_dequant_rms(const uint8_t *__restrict__ codes, const float2 *__restrict__ mm, long n, float *__restrict__ out)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {

@@ -18,19 +18,9 @@
 #pragma once
 
 #include "kernels.hpp"
+#include "sampler_state.hpp"
 
 namespace l2j {
-
-constexpr int kSampleMaxVocab = 36864;  // the most probabilities of one call that fit in LDS: 144 KB
-constexpr unsigned long long kJavaRandMult = 0x5DEECE66DULL, kJavaRandMask = (1ULL << 48) - 1;
-
-struct SamplerState {        // the reference's Sampler object, device resident
-    unsigned long long rng;  // java.util.Random's 48-bit state
-    int n0;                  // candidates of the current sample_topp call
-    int nan;                 // bit 0: a NaN among the probabilities (J/Sampler.java:88-90 throws); bit 1: no top-p candidate
-    int result;              // the token of the last call
-    int pad;
-};
 
 struct SampleArgs {
     float *logits;           // in: logits; out: the probabilities, as the reference leaves them (J/Run.java:647-659)
@@ -396,7 +386,7 @@ __device__ __forceinline__ int spec_first_over(const float *p, const SpecThread 
 // The element-wise front of the step spread over many workgroups (the double-precision exponential of 32000 logits
 // takes 0.04 ms on one compute unit): every workgroup divides all the logits by the temperature and takes the maximum
 // (the same value everywhere: a maximum does not depend on the order), then exponentiates its own slice into expbuf.
-__global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
+static __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
 {
     __shared__ float red[16];
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
@@ -705,7 +695,7 @@ __global__ void __launch_bounds__(1024) k_running_sums(float *x, int n, int scan
 constexpr int kSortTile = 256, kSortRun = 4096, kSortTilesPerRun = kSortRun / kSortTile;
 
 // grid: padded n / 256 workgroups of 256 threads
-__global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
+static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
                                                           float *__restrict__ kout, int *__restrict__ vout)
 {
     __shared__ __align__(16) float keys[kSortTile];
@@ -729,7 +719,7 @@ __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restric
 // grid: (padded n / 4096, 16) workgroups of 256 threads: a workgroup holds the keys of its run in LDS and places a
 // sixteenth of them, one per thread.  The fifteen binary searches of a pair advance together, step by step (their LDS reads are
 // independent: one after the other they cost fifteen times the latency).
-__global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
+static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
                                                      int *__restrict__ vout)
 {
     __shared__ __align__(16) float keys[kSortRun];
@@ -767,7 +757,7 @@ __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ k
 constexpr int kSortMaxRuns = (kSampleMaxVocab + kSortRun - 1) / kSortRun;
 
 // grid: padded n / 256 workgroups of 256 threads; dynamic LDS: padded n floats.  Only the first n pairs are written.
-__global__ void __launch_bounds__(256) k_merge_runs(const float *__restrict__ kin, const int *__restrict__ vin, int n, int npad,
+static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restrict__ kin, const int *__restrict__ vin, int n, int npad,
                                                      float *__restrict__ kout, int *__restrict__ vout)
 {
     extern __shared__ __align__(16) float keys[];
@@ -813,7 +803,7 @@ __global__ void __launch_bounds__(256) k_merge_runs(const float *__restrict__ ki
 // grid: padded n / 256 workgroups of 256 threads; run_len and group_len are powers of two, npad a multiple of 256.
 constexpr int kSortFanIn = 16;
 
-__global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
+static __global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
                                                     int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
@@ -851,7 +841,7 @@ __global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin
 }
 
 // J/Sampler.java:46-57 on an array given by the caller: first index of the strict maximum.  One workgroup.
-__global__ void __launch_bounds__(1024) k_argmax_logits(const float *__restrict__ x, int n, SamplerState *ss)
+static __global__ void __launch_bounds__(1024) k_argmax_logits(const float *__restrict__ x, int n, SamplerState *ss)
 {
     __shared__ float bval[16];
     __shared__ int bidx[16];

@@ -10,6 +10,30 @@ from llama2j_amd.binding import L2JError
 
 pytestmark = pytest.mark.gpu
 
+LOGIT_TOL = 1e-3   # per step: max |logit - oracle's| / max |oracle's logit|, the bar of the single-sequence path
+
+
+def rel_err(got, want):
+    return float(np.abs(got.astype(np.float64) - want).max() / np.abs(want).max())
+
+
+def oracle_of(orc, shape, seed):
+    m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
+                  vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
+    m.fill_synth(seed, 0.02)
+    return m
+
+
+def check_against_oracle(m, prompt, steps, tokens, logits, what):
+    """The oracle's own greedy loop from the same prompt: the same tokens (until it stops at token 1; the batch runs on), and at
+    every one of those steps the batched path's logits within the bar of the oracle's."""
+    m.reset()
+    want_tok, want_logits, _ = m.generate_greedy(prompt, steps, want_logits=True)
+    np.testing.assert_array_equal(tokens[:len(want_tok)], want_tok, err_msg=what)
+    worst = max(rel_err(logits[pos], want_logits[pos]) for pos in range(len(want_tok)))
+    assert worst < LOGIT_TOL, (what, worst)
+    return worst
+
 SHAPES = [
     (512, 1024, 4, 8, 8, 1008, 64, 1),      # head 64, shared classifier
     (512, 1024, 2, 8, 2, 1008, 64, 0),      # grouped-query attention: 8 heads on 2 kv heads
@@ -58,21 +82,21 @@ def test_every_sequence_gets_what_it_gets_alone(orc, shape, n_seq):
     prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 9))).astype(np.int32) for _ in range(n_seq - 3)]   # three without a prompt
     got, sec = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
     assert got.shape == (n_seq, steps) and sec > 0
+    got2, logits = g.decode_greedy_batch(prompts, steps, n_seq=n_seq, want_logits=True)   # (the same buffers and graph again)
+    np.testing.assert_array_equal(got2, got)
     for b in range(n_seq):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
         g.reset()
         want, _ = g.decode_greedy(p, steps)          # stops after token 1; the batch runs on
         np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d" % b)
         np.testing.assert_array_equal(got[b, :len(p)], p)
-    # two of them against the oracle as well
-    m = orc.Model(dim=shape[0], hidden_dim=shape[1], n_layers=shape[2], n_heads=shape[3], n_kv_heads=shape[4],
-                  vocab_size=shape[5], seq_len=shape[6], shared_weights=shape[7])
-    m.fill_synth(9, 0.02)
-    for b in (0, n_seq - 1):
+    # every sequence against the oracle as well: its tokens, and the logits of every step
+    m = oracle_of(orc, shape, 9)
+    worst = 0.0
+    for b in range(n_seq):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
-        m.reset()
-        want, _, _ = m.generate_greedy(p, steps)
-        np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d against the oracle" % b)
+        worst = max(worst, check_against_oracle(m, p, steps, got[b], logits[:, b], "sequence %d against the oracle" % b))
+    print("batched logits vs oracle: worst max|d|/max|logit| = %.3g over %d sequences x %d steps" % (worst, n_seq, steps), flush=True)
     # the context's own cache and loop state are untouched: a single decode after the batch is what it was before
     g.reset()
     again, _ = g.decode_greedy(prompts[0], steps)
@@ -85,20 +109,60 @@ def test_every_sequence_gets_what_it_gets_alone(orc, shape, n_seq):
     ((4096, 11008, 3, 32, 32, 32000, 48, 0), 16, 40),
     ((8192, 28672, 2, 64, 8, 32000, 32, 0), 32, 24),       # the widths of Llama-2-70B: 64 heads on 8 kv heads, rows of 32 and 112 groups
 ])
-def test_published_widths_match_the_single_decode(shape, n_seq, steps):
+def test_published_widths_match_the_single_decode_and_the_oracle(orc, shape, n_seq, steps):
     """At the matrix sizes of the published models (a few layers of them) every sequence of a batch gets the tokens of its
-    own single-sequence decode; the single-sequence path is pinned against the oracle at these widths in test_gpu_parity.py."""
+    own single-sequence decode, and four of them (the first, two in the middle, the one without a prompt) the oracle's
+    tokens and, step by step, its logits."""
     g = l2j.Transformer(l2j.Config(*shape))
     g.fill_synthetic(21, 0.02)
     g.finalize()
     rng = np.random.default_rng(n_seq + shape[0])
     prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, 7))).astype(np.int32) for _ in range(n_seq - 1)]
-    got, _ = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
+    got, logits = g.decode_greedy_batch(prompts, steps, n_seq=n_seq, want_logits=True)
     for b in range(n_seq):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
         g.reset()
         want, _ = g.decode_greedy(p, steps)
         np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d" % b)
+    g.close()
+    m = oracle_of(orc, shape, 21)
+    worst = 0.0
+    for b in (0, n_seq // 3, n_seq // 2 + 1, n_seq - 1):
+        p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
+        worst = max(worst, check_against_oracle(m, p, steps, got[b], logits[:, b], "sequence %d against the oracle" % b))
+    print("batched logits vs oracle at widths %s: worst max|d|/max|logit| = %.3g" % (shape[:2], worst), flush=True)
+    m.close()
+
+
+def test_buffers_and_graph_are_kept_between_calls_and_replaced_when_they_do_not_fit():
+    """The context owns the batched path's buffers: a second call with fewer steps and other prompts runs in them (other
+    strides than its own arguments'), a call with more steps or another sequence count replaces them."""
+    shape = (512, 1024, 2, 8, 2, 1008, 96, 0)
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(5, 0.02)
+    g.finalize()
+    rng = np.random.default_rng(11)
+    for n_seq, steps, longest in ((32, 48, 9), (32, 20, 4), (32, 64, 12), (16, 30, 6), (16, 30, 1)):
+        prompts = [rng.integers(2, shape[5], size=int(rng.integers(0, longest + 1))).astype(np.int32) for _ in range(n_seq)]
+        got, _ = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
+        for b in (0, 1, n_seq - 1):
+            g.reset()
+            want, _ = g.decode_greedy(prompts[b], steps)
+            np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="%d sequences, %d steps, sequence %d" % (n_seq, steps, b))
+    g.close()
+
+
+def test_a_new_upload_replaces_the_tile_ordered_copy():
+    """The batched products read a second copy of the matrices; uploading a tensor again must not leave the old copy in use."""
+    shape = (512, 1024, 1, 8, 8, 1008, 16, 1)
+    g = l2j.Transformer(l2j.Config(*shape))
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((16, 512)).astype(np.float32)
+    for seed in (1, 2):
+        g.fill_synthetic(seed, 0.02)      # (uploads are legal until finalize; the product does not need a finalized context)
+        got, _ = g.batch_matmul(TENSOR.WQ, 0, x, 512)
+        want = x.astype(np.float64) @ dequantized(g, TENSOR.WQ, 0, 512, 512).T
+        assert (np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)).max() < 5e-6, seed
     g.close()
 
 

@@ -622,7 +622,7 @@ def test_checkpoint_loader_and_quant_caches(orc, tmp_path):
 
 # ------------------------------------------------------------------ whole model, the five benchmark configurations
 
-def run_config(orc, name, shape, seed, n_prompt, n_steps, n_logit_steps):
+def run_config(orc, name, shape, seed, n_prompt, n_steps, n_logit_steps, late=None):
     """Greedy decode on both sides: identical tokens; per-step logits for the first n_logit_steps."""
     say("[%s] building seed=%d shape=%s" % (name, seed, shape))
     t0 = time.time()
@@ -650,6 +650,28 @@ def run_config(orc, name, shape, seed, n_prompt, n_steps, n_logit_steps):
     say("[%s] worst max|dlogit|/max|logit| = %.3g over %d steps; min relative top-2 gap = %.3g" %
         (name, worst, min(n_logit_steps, len(want_tok)), min_gap))
     assert worst < LOGIT_TOL
+    if late:
+        # The configuration's full length: the GPU decodes all of it, the rows its decode left in the KV cache are copied
+        # into the oracle, and the oracle's single forwards at the last positions must give the GPU's logits and the token
+        # the GPU's own loop emitted there (the oracle would need minutes to get there by itself).
+        n_total, positions = late
+        L, kvd = shape[2], shape[0] // shape[3] * shape[4]
+        g.reset()
+        toks, sec = g.decode_greedy(prompt, n_total)
+        assert len(toks) == n_total, "the decode stopped early (token 1): pick another seed"
+        np.testing.assert_array_equal(toks[:len(want_tok)], want_tok)
+        kc, vc = m.buffer(orc.B_KCACHE).reshape(L, shape[6], kvd), m.buffer(orc.B_VCACHE).reshape(L, shape[6], kvd)
+        for l in range(L):
+            kc[l, :n_total] = g.read(BUFFER.KCACHE, layer=l, off=0, n=n_total * kvd).reshape(n_total, kvd)
+            vc[l, :n_total] = g.read(BUFFER.VCACHE, layer=l, off=0, n=n_total * kvd).reshape(n_total, kvd)
+        for pos in positions:
+            tok = int(toks[pos - 1])
+            want = m.forward(tok, pos).copy()
+            got = g.forward(tok, pos)
+            e = rel_err(got, want)
+            say("[%s] %d steps at %.1f tok/s; pos %d: max|dlogit|/max|logit| = %.3g" % (name, n_total, (n_total - 1) / sec, pos, e))
+            assert e < LOGIT_TOL, pos
+            assert int(np.argmax(want)) == int(np.argmax(got)) == int(toks[pos]), pos
     m.close(); g.close()
 
 
@@ -659,14 +681,16 @@ def test_config1_stories15m_shape(orc, launch_mode):
 
 
 def test_config2_stories110m_shape(orc, launch_mode):
-    run_config(orc, "110M", (768, 2048, 12, 12, 12, 32000, 1024, 1), seed=102, n_prompt=16, n_steps=16 + 128,
-               n_logit_steps=16 + 128)
+    # the configuration's full length: 16 prompt ids + 512 greedy tokens, logits at all 528 steps
+    run_config(orc, "110M", (768, 2048, 12, 12, 12, 32000, 1024, 1), seed=102, n_prompt=16, n_steps=16 + 512,
+               n_logit_steps=16 + 512)
 
 
 def test_config3_llama2_7b_shape(orc):
     # 32 prompt ids + 64 greedy tokens against the oracle (the oracle takes ~0.3 s per token per 16 cores)
+    # then the configuration's 32 + 256 on the GPU, and the oracle on the GPU's cache at the last positions
     run_config(orc, "7B", (4096, 11008, 32, 32, 32, 32000, 4096, 0), seed=103, n_prompt=32, n_steps=32 + 64,
-               n_logit_steps=32 + 64)
+               n_logit_steps=32 + 64, late=(32 + 256, (160, 285, 286, 287)))
 
 
 def test_config4_long_context_attention(orc):
@@ -755,4 +779,4 @@ def test_config5_llama2_13b_shape(orc):
     # the reference's int offsets overflow at this size (J/TransformerWeights.java:89); 64-bit here.
     # 32 prompt ids + the first 64 greedy tokens, logits at all 96 steps (the oracle runs at ~3.7 tok/s on 16 cores)
     run_config(orc, "13B", (5120, 13824, 40, 40, 40, 32000, 4096, 0), seed=105, n_prompt=32, n_steps=32 + 64,
-               n_logit_steps=32 + 64)
+               n_logit_steps=32 + 64, late=(32 + 256, (286, 287)))
