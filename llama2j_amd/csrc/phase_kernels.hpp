@@ -871,7 +871,7 @@ struct AttnRun {
     {
         float *sm_m = smem;           // nent
         float *sm_l = sm_m + nent;    // nent
-        float *sm_w = sm_l + nent;    // nent + 4: the slots' weights, then their common maximum (and padding)
+        float *sm_w = sm_l + nent;    // nent + 4 (unused: the fold keeps the weights in registers)
         float *sm_acc = sm_w + nent + 4;  // nent * hs
         int &s_last = *reinterpret_cast<int *>(sm_acc + nent * hs);
 
@@ -941,38 +941,31 @@ struct AttnRun {
                 }
                 m = mb;
             }
-            __syncthreads();  // LDS reuse across items
+            if (it != (int)blockIdx.x) __syncthreads();  // LDS reuse across items (the first finds it free)
             if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
             if (active) *reinterpret_cast<float4 *>(sm_acc + slot * hs + 4 * j) = acc;
             __syncthreads();
-            // Fold the row slots in a fixed order, so the result does not depend on timing.  The slots' weights
-            // exp(m_e - M) come from one lane each (at most 64 slots); the fold itself then only reads LDS.
-            if (tid < 64) {
-                const float me = tid < nent ? sm_m[tid] : -3.402823466e+38f;
-                const float mx = wave_max(me);
-                if (tid < nent) sm_w[tid] = expf(me - mx);  // empty slots: exp(-huge) = 0
-                if (tid == 0) sm_w[nent] = mx;
-            }
-            __syncthreads();
-            const float M = sm_w[nent];
-            float L = 0.0f, o = 0.0f;
-            if (tid < hs) {
-                // four slots per step: the LDS reads of a step are issued together, the additions keep slot order
-                const float *ap = sm_acc + tid;
+            // Fold the row slots (at most 64) in a fixed order, so the result does not depend on timing.  Each of the waves
+            // that hold the head's elements does the whole fold for itself, without another workgroup barrier: lane e
+            // takes slot e's maximum and sum and computes its weight exp(m_e - M), the weighted sums are added across the
+            // wave, and every thread folds its element over the slots with the weights read lane by lane.
+            float M = 0.0f, L = 0.0f, o = 0.0f;
+            if (tid < 64 * store_waves()) {
+                const float me = lane < nent ? sm_m[lane] : -3.402823466e+38f;
+                const float le = lane < nent ? sm_l[lane] : 0.0f;
+                M = wave_max(me);
+                const float w = expf(me - M);  // empty slots: exp(-huge) = 0
+                L = wave_sum(le * w);
+                const float *ap = sm_acc + min(tid, hs - 1);
                 int e = 0;
-                for (; (nent & 3) == 0 && e < nent; e += 4) {  // (16-byte LDS reads need nent % 4 == 0)
-                    const float4 w4 = *reinterpret_cast<const float4 *>(sm_w + e), l4 = *reinterpret_cast<const float4 *>(sm_l + e);
+                for (; e + 4 <= nent; e += 4) {  // four slots per step: their LDS reads are issued together
                     const float a0 = ap[(e + 0) * hs], a1 = ap[(e + 1) * hs], a2 = ap[(e + 2) * hs], a3 = ap[(e + 3) * hs];
-                    L = fmaf(l4.x, w4.x, L); o = fmaf(a0, w4.x, o);
-                    L = fmaf(l4.y, w4.y, L); o = fmaf(a1, w4.y, o);
-                    L = fmaf(l4.z, w4.z, L); o = fmaf(a2, w4.z, o);
-                    L = fmaf(l4.w, w4.w, L); o = fmaf(a3, w4.w, o);
+                    o = fmaf(a0, readlane_f(w, e), o);
+                    o = fmaf(a1, readlane_f(w, e + 1), o);
+                    o = fmaf(a2, readlane_f(w, e + 2), o);
+                    o = fmaf(a3, readlane_f(w, e + 3), o);
                 }
-                for (; e < nent; e++) {
-                    const float w = sm_w[e];
-                    L = fmaf(sm_l[e], w, L);
-                    o = fmaf(ap[e * hs], w, o);
-                }
+                for (; e < nent; e++) o = fmaf(ap[e * hs], readlane_f(w, e), o);
             }
             if (nact == 1) {
                 if (tid < hs) {
