@@ -30,12 +30,11 @@ size_t attn_smem_for(const l2j_ctx *c, int threads)
 
 size_t attn_smem(const l2j_ctx *c) { return attn_smem_for(c, c->attn_threads); }
 
-// k_token: the largest LDS need of its phases (rounded to 16 bytes), then its arrival counters
-size_t phase_smem(const l2j_ctx *c)
+// k_token: the largest LDS need of its phases
+size_t layer_smem(const l2j_ctx *c)
 {
-    return (std::max(mv_smem(std::max(c->cfg.dim, c->cfg.hidden_dim)), attn_smem_for(c, c->pk_threads)) + 15) / 16 * 16;
+    return std::max(mv_smem(std::max(c->cfg.dim, c->cfg.hidden_dim)), attn_smem_for(c, c->pk_threads));
 }
-size_t layer_smem(const l2j_ctx *c) { return phase_smem(c) + kTokenLdsExtra; }
 
 static_assert(K_QKV == L2J_K_QKV && K_ATT == L2J_K_ATTENTION && K_WO == L2J_K_WO && K_W13 == L2J_K_W13 && K_W2 == L2J_K_W2 &&
               K_CLS == L2J_K_CLASSIFIER, "kernel classes of the C ABI and of the device code must agree");
@@ -106,8 +105,7 @@ auto with_token_kernel(const l2j_ctx *c, F f)
     const int tud = tu_for(c->cfg.dim), tuh = tu_for(c->cfg.hidden_dim);
     const bool special = c->opt[OPT_TOKEN_SPECIAL] != 0;
     if (special && c->opt[OPT_FAST_STEPS] != 0 && lpr == 32 && c->cfg.dim == 1024 * tud && c->cfg.dim % 256 == 0) {
-        // (its Wo phase stages one 16-byte word per thread and folds one item per wave: run_by_quarters)
-        if (tud == kTU && c->pk_threads == 1024 && 16 * c->pk_grid >= c->cfg.dim / 2) return f(k_token<32, kTU, kTU, true>);
+        if (tud == kTU) return f(k_token<32, kTU, kTU, true>);
         if (tud == 5) return f(k_token<32, 5, kTU, true>);
     }
     if (special && lpr == 16 && tud == 1 && tuh == 1) return f(k_token<16, 1, 1>);
@@ -128,7 +126,6 @@ hipError_t launch_layers(const l2j_ctx *c, int l0, int l1, hipStream_t s, hipEve
     a.attn_rows = c->fused_attn_rows;
     a.attn_splits = fused_splits(c);
     a.maxspin = std::max(0, c->opt[OPT_BARRIER_SPINS]);  // each poll is a memory round trip, >= 1 us
-    a.ctr_off = (int)(phase_smem(c) / sizeof(float));
     a.by_value = c->by_value ? 1 : 0;
     a.self_contained = l0 == 0 && l1 == c->cfg.n_layers ? c->self_contained : 0;
     const dim3 grid(c->pk_grid), block(c->pk_threads);
@@ -476,9 +473,8 @@ int l2j::setup_forward(l2j_ctx *c)
         c->attn_nsplit = std::max(1, o[OPT_ATTN_NSPLIT]);
         c->attn_grid = c->cfg.n_heads * c->attn_nsplit;
         c->fused_attn_rows = std::max(1, o[OPT_FUSED_ATTN_ROWS]);
-        if (std::max(mv_smem(nmax), attn_smem(c)) > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
-        // (a whole-token kernel whose LDS would exceed the compute unit's is not used, see below)
-        const size_t need = std::min<size_t>(160 * 1024, std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c)));
+        const size_t need = std::max(std::max(mv_smem(nmax), attn_smem(c)), layer_smem(c));
+        if (need > 160 * 1024) return fail(L2J_E_ARG, "hidden_dim does not fit the 160 KB LDS");
         if (need > 64 * 1024) {
             const void *ks[] = {reinterpret_cast<const void *>(k_matvec<PH_QKV>), reinterpret_cast<const void *>(k_matvec<PH_W13>),
                                 reinterpret_cast<const void *>(k_matvec<PH_RES>), reinterpret_cast<const void *>(k_matvec<PH_ROW>),
@@ -509,7 +505,6 @@ int l2j::setup_forward(l2j_ctx *c)
         const uint64_t layer_floats = 2ull * c->cfg.dim * c->cfg.dim + 2ull * c->cfg.dim * c->kv_dim + 3ull * c->cfg.dim * c->cfg.hidden_dim;
         c->fused = (c->opt[OPT_FUSE] != kAuto ? c->opt[OPT_FUSE] : layer_floats >= (4ull << 20) ? 1 : 0) != 0;
         c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, c->opt[OPT_LAYERS_PER_LAUNCH] != kAuto ? c->opt[OPT_LAYERS_PER_LAUNCH] : c->cfg.n_layers));
-        if (c->fused && layer_smem(c) > 160 * 1024) c->fused = false;
         if (c->fused) {
             const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
             int per_cu = 0;

@@ -221,19 +221,7 @@ struct MatvecPhase {
     int threads;    // workgroup size (a kernel argument: reading it from the dispatch costs a vector load per phase)
     Poll poll;      // how the input vector and the residual are read
     float *knew, *vnew;  // QKV with poll.on: this token's k and v rows once more, where attention waits for them
-    int ctr_off;    // k_token: four arrival counters in dynamic LDS behind the phases' own, in floats (run_by_quarters)
-    int ctr_target; // ... and what they read once this phase's input is staged
 };
-
-#ifndef L2J_WO_QUARTERS
-#define L2J_WO_QUARTERS 1
-#endif
-__device__ __forceinline__ float *dyn_lds()
-{
-    extern __shared__ float4 l2j_dyn_lds_[];
-    return reinterpret_cast<float *>(l2j_dyn_lds_);
-}
-constexpr size_t kTokenLdsExtra = 64;  // bytes of k_token's dynamic LDS behind its phases' own: the arrival counters
 
 // ---- activation vector -> LDS ------------------------------------------------------------------
 // LDS layout for an n-float vector (nch = n/16 chunks): float4 xs[q*nch + c] holds x[16c+4q .. 16c+4q+3],
@@ -647,60 +635,6 @@ struct MatvecRun {
                 if (p1) *p1 = v1;
             }
         }
-    }
-
-    // The Wo phase of k_token at the 7B width (rows of 4096 codes, 1024 threads, at most one item per wave).  Its input, the
-    // attention output, arrives head by head as the heads' last splits finish, up to a microsecond apart, and the phase has
-    // nothing else to wait for: its weights are in the registers.  So instead of one workgroup barrier behind the slowest
-    // head, each quarter of the vector (the 1024 floats that chunk u of every lane multiplies; the four waves 4u..4u+3 stage
-    // it) has an arrival counter in LDS, and a wave folds chunk u as soon as that quarter is there: the multiply-adds of
-    // the early quarters are done when the last head arrives.  The sums are added in chunk order as always.
-    __device__ __forceinline__ void run_by_quarters(float4 *smem4, int token, int pos)
-    {
-        static_assert(FAST && MODE == PH_RES && TU == 4, "rows of 4096 codes in pairs");
-        float4 *xs = smem4;
-        float *sumx = reinterpret_cast<float *>(smem4 + 4 * nch);
-        const float *res = d.res_emb ? d.emb + (long)token * n : d.res_src;
-        unsigned *cnt = reinterpret_cast<unsigned *>(dyn_lds() + d.ctr_off);
-        const int tid = phase_tid();
-        {
-            const float4 xv = wait_word(d.xin + 4 * tid, d.poll);
-            const float s0 = (xv.x + xv.y) + (xv.z + xv.w);
-            const float s1 = dpp_f<0x55>(s0), s2 = dpp_f<0xAA>(s0), s3 = dpp_f<0xFF>(s0);  // quad lanes 1, 2, 3
-            xs[(tid & 3) * nch + (tid >> 2)] = xv;
-            if ((tid & 3) == 0) sumx[tid >> 2] = ((s0 + s1) + s2) + s3;
-            asm volatile("" ::: "memory");  // (the LDS performs a wave's instructions in order: the count follows the data)
-            if (lane == 0) __hip_atomic_fetch_add(cnt + (wave >> 2), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
-        if (item >= nitems) return;
-        if (!first) {
-            resolve(item);
-            issue(0);
-        }
-        first = false;
-        float resv0, resv1, acc0 = 0.0f, acc1 = 0.0f;
-        residual(res, resv0, resv1);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-        const float4 *xp = xs + lane;
-        const float *sp = sumx + lane;
-        const unsigned want = (unsigned)d.ctr_target;
-#pragma unroll
-        for (int u = 0; u < TU; u++) {
-            int spins = 0;
-            while (__hip_atomic_load(cnt + u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < want) {
-                if (++spins > (1 << 22)) break;  // (a producer that gave up has flagged the fault)
-                __builtin_amdgcn_s_sleep(1);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            const uint4 a0 = w0[u], a1 = w1[u];
-            const float2 g0 = s0[u], g1 = s1[u];
-            const float4 x0 = xp[64 * u], x1 = xp[nch + 64 * u], x2 = xp[2 * nch + 64 * u], x3 = xp[3 * nch + 64 * u];
-            const float sx = sp[64 * u];
-            acc0 += fmaf(g0.x, dot16(a0, x0, x1, x2, x3), g0.y * sx);
-            acc1 += fmaf(g1.x, dot16(a1, x0, x1, x2, x3), g1.y * sx);
-        }
-        finish<true>(item, which, r, acc0, acc1, resv0, resv1, pos, 1.0f);
-        item = nitems;
     }
 
     // smem: 4*nch float4 (vector), nch floats (chunk sums), 16 floats (reduction).
@@ -1301,7 +1235,6 @@ struct TokenArgs {
     int attn_rows;          // cache rows per attention split in this kernel (more when the splits run out)
     int attn_splits;        // at most this many splits per head: one (head, split) item per workgroup
     int maxspin;
-    int ctr_off;            // dynamic LDS behind the phases' own (kTokenLdsExtra bytes) starts here, in floats
     int by_value;           // 1: consumers wait for the data itself (activations pre-filled with kUnset); 0: grid barriers
     int self_contained;     // (with by_value, the whole token in this launch) bit 0: the kernel alternates between two sets of
                             // activation vectors and marks the other one unwritten for the next token (no k_fill_unset
@@ -1369,8 +1302,6 @@ __device__ __forceinline__ MatvecPhase token_phase(int kclass, int l, int set)
 {
     MatvecPhase d = matvec_phase_of(token_args()->g, kclass, l, set);
     d.poll = token_poll();
-    d.ctr_off = token_args()->ctr_off;
-    d.ctr_target = 4 * (l - token_args()->l0 + 1);
     if (d.poll.on && kclass == K_QKV) {
         d.knew = token_args()->g.knew + set * token_args()->g.set_stride + l * token_args()->g.skv;
         d.vnew = token_args()->g.vnew + set * token_args()->g.set_stride + l * token_args()->g.skv;
@@ -1435,11 +1366,7 @@ __device__ __forceinline__ void token_wo_w13(const GridBar &b, int l, int set, f
     } else {
         handoff(b, 5 * l + 1, wo);
     }
-    if constexpr (L2J_WO_QUARTERS && FAST && WO_MODE == PH_RES && TUD == 4) {
-        wo.run_by_quarters(smem4, token, pos);  // (1024 threads and at most one item per wave: checked on the host)
-    } else {
-        wo.template run<true>(smem4, token, pos);
-    }
+    wo.template run<true>(smem4, token, pos);
     if constexpr (WO_MODE == PH_RES && LEND) {
         TakeRegisters<W13Run, WoRun> second{w13, wo, lend};
         handoff(b, 5 * l + 2, second);
@@ -1508,7 +1435,6 @@ __global__ void __launch_bounds__(1024) k_token(const TokenArgs)
     const int wo_mode = row_mode(t->g.dim), w2_mode = row_mode(t->g.hidden);
     GridBar b;
     b.ctr = t->g.bar_ctr; b.fault = t->g.fault; b.ngroups = t->by_value ? 0 : kBarGroups; b.maxspin = t->maxspin;
-    if (threadIdx.x < 4) reinterpret_cast<unsigned *>(dyn_lds() + t->ctr_off)[threadIdx.x] = 0u;  // (published by the first workgroup barrier)
     for (int l = l0; l < l1; l++) {
         {
             MatvecRun<PH_QKV, TUD, FASTD> qkv(token_phase(K_QKV, l, set));
