@@ -55,7 +55,7 @@ def synth_prompt(seed, n, vocab):
 # profiles/hbm_traffic_llama2-7b.md (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for a
 # 256 MiB copy kernel); it is reported with its source and only for the workload and kernel it was collected on.
 COUNTER_TRAFFIC = {
-    "llama2-7b-shape": {"hbm_bytes_per_launch": 7460326598, "positions": "0-287 (median launch: 144)",
+    "llama2-7b-shape": {"hbm_bytes_per_launch": 7460859757, "positions": "0-287 (median launch: 144)",
                         "algorithmic_bytes_at_those_positions": 7356051584,
                         "source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), profiles/hbm_traffic_llama2-7b.md",
                         "collected": "2026-11-25"},
