@@ -577,6 +577,12 @@ def test_options_override_the_process_defaults(orc, monkeypatch):
         g.finalize()
         for p in range(4):
             assert rel_err(g.forward(3 + p, p), want[p]) < LOGIT_TOL, (opts, p)
+        # the decode loop times itself with the device's wall clock: the rate is known here, and a run has a duration
+        assert g.get_option("wall_clock_khz") > 0
+        toks, sec = g.decode_greedy(np.array([3, 4], dtype=np.int32), 6)
+        assert len(toks) > 1 and 0.0 < sec < 1.0
+        with pytest.raises(l2j.L2JError):
+            g.set_option("wall_clock_khz", 5)        # read-only
         g.close()
     m.close()
 
