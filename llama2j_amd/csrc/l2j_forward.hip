@@ -499,11 +499,12 @@ int l2j::setup_forward(l2j_ctx *c)
         HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&c->h_fault), sizeof(int), hipHostMallocDefault));
         *c->h_fault = 0;
         // k_token needs its whole grid resident at once (grid barriers): at most what the occupancy allows.
-        // One launch per token pays off when a layer streams enough to hide its five hand-overs (7B shape, 208 MB a
-        // layer: 645 vs 511 tok/s; 110M shape, 7 MB: 3240 vs 3080); the smallest models run faster as one launch per
-        // phase (15M shape, 1 MB a layer: 6300 vs 5400 tok/s).
+        // One launch per token pays off when a hand-over inside the kernel costs less than a kernel boundary of the
+        // replayed graph: measured whole-token / one launch per phase, 7B shape (208 MB a layer) 1.44 / 1.96 ms per token,
+        // 110M shape (7 MB) 0.241 / 0.278 ms, 15M shape (1 MB) 0.123 / 0.134 ms.  Below half a million weights a layer
+        // (test models) the phases stay separate launches.
         const uint64_t layer_floats = 2ull * c->cfg.dim * c->cfg.dim + 2ull * c->cfg.dim * c->kv_dim + 3ull * c->cfg.dim * c->cfg.hidden_dim;
-        c->fused = (c->opt[OPT_FUSE] != kAuto ? c->opt[OPT_FUSE] : layer_floats >= (4ull << 20) ? 1 : 0) != 0;
+        c->fused = (c->opt[OPT_FUSE] != kAuto ? c->opt[OPT_FUSE] : layer_floats >= (1ull << 19) ? 1 : 0) != 0;
         c->layers_per_launch = std::max(1, std::min(c->cfg.n_layers, c->opt[OPT_LAYERS_PER_LAUNCH] != kAuto ? c->opt[OPT_LAYERS_PER_LAUNCH] : c->cfg.n_layers));
         if (c->fused) {
             const void *kl = with_token_kernel(c, [](auto kernel) { return reinterpret_cast<const void *>(kernel); });
