@@ -318,7 +318,9 @@ def main():
     if long_context:
         out["cpu_baseline"] = lc_cpu
     elif a.cpu_steps > 1:
-        out["cpu_baseline"] = cpu_baseline(shape, seed, prompt, g_tokens, min(a.cpu_steps, steps))
+        # (a bounded sample of its own length, about 10-30 s of CPU work: it does not shrink with a short timed run; the
+        # tokens compared are the generated positions both runs have)
+        out["cpu_baseline"] = cpu_baseline(shape, seed, prompt, g_tokens, min(a.cpu_steps, shape[6]))
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out), flush=True)
