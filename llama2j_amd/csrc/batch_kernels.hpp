@@ -24,6 +24,35 @@ constexpr int kXPadH = 8;           // the same for the bf16 planes of k_bgemm (
 typedef float v4f32 __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
 
+// Device-coherent 16-byte accesses for what the workgroups of one launch hand to each other (a load per float would
+// fetch the same lines once per float: such loads do not stay in the L2).  Loads and their wait are one statement: the
+// compiler must not touch the destination registers in between.
+__device__ __forceinline__ void ld_coh64x2(const float *p0, const float *p1, float (&v0)[16], float (&v1)[16])   // 64 bytes at p0, 64 bytes at p1
+{
+    float4 v[8];
+    asm volatile("global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %8, off offset:16 sc1\n\t"
+                 "global_load_dwordx4 %2, %8, off offset:32 sc1\n\tglobal_load_dwordx4 %3, %8, off offset:48 sc1\n\t"
+                 "global_load_dwordx4 %4, %9, off sc1\n\tglobal_load_dwordx4 %5, %9, off offset:16 sc1\n\t"
+                 "global_load_dwordx4 %6, %9, off offset:32 sc1\n\tglobal_load_dwordx4 %7, %9, off offset:48 sc1\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+                 : "v"(p0), "v"(p1)
+                 : "memory");
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        v0[4 * q] = v[q].x; v0[4 * q + 1] = v[q].y; v0[4 * q + 2] = v[q].z; v0[4 * q + 3] = v[q].w;
+        v1[4 * q] = v[4 + q].x; v1[4 * q + 1] = v[4 + q].y; v1[4 * q + 2] = v[4 + q].z; v1[4 * q + 3] = v[4 + q].w;
+    }
+}
+
+// write-through; acknowledged by the next s_waitcnt vmcnt(0).  (The wait states are part of the statement: a store of more
+// than 8 bytes reads its data registers after it has issued, and the compiler, which does not look inside the statement,
+// would let the next instruction overwrite them.)
+__device__ __forceinline__ void st_coh16(float *p, v4f32 v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
+}
+
 // y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].  Up to three matrices that
 // share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
 constexpr int kBgMaxMat = 3;
@@ -106,19 +135,22 @@ struct BgWave {
         int rows;
         bool two;
     };
-    const BGemm &a;
+    const BGemm *ap;   // (a pointer, so that a kernel with several products can aim one BgWave at each in turn)
+    long layer;        // the matrices of this layer: layer * rows * K codes behind m.off
     int by, lane, r, s, ngroups, g0, g1, total, stride, u;
     Unit cur;
     uint4 w0[4], w1[4];
 
-    __device__ __forceinline__ BgWave(const BGemm &a_) : a(a_) {}
+    __device__ __forceinline__ BgWave(const BGemm &a_) : ap(&a_), layer(0) {}
 
     __device__ __forceinline__ Unit locate(int unit) const
     {
+        const BGemm &a = *ap;
         int mi = 0;
         while (mi + 1 < a.nmat && unit >= bg_units(a.rows[mi], TILES)) { unit -= bg_units(a.rows[mi], TILES); mi++; }
-        const QMat mat = a.m[mi];
+        QMat mat = a.m[mi];
         const int rows = a.rows[mi], row0 = unit * 16 * TILES;
+        mat.off += layer * rows * a.K;
         Unit n;
         n.rows = rows;
         n.two = TILES == 2 && row0 + 16 < rows;
@@ -142,6 +174,7 @@ struct BgWave {
     // the activations would arrive with them).
     __device__ __forceinline__ void begin(int bx, int by_, int gx, bool first)
     {
+        const BGemm &a = *ap;
         const int tid = threadIdx.x;
         by = by_;
         lane = tid & 63;
@@ -164,6 +197,7 @@ struct BgWave {
     template <bool COH>
     __device__ __forceinline__ void run(unsigned short *xh, float (*sxs)[kBgMaxGps], bool requested)
     {
+        const BGemm &a = *ap;
         const int tid = threadIdx.x, nk = (g1 - g0) << 8;
         // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
         // offsets) and their three bf16 parts.
@@ -171,12 +205,11 @@ struct BgWave {
         const int sb = tid >> 4, pt = tid & 15;
         const float *xsrc = a.x + (long)sb * a.K + (g0 << 8) + 16 * pt;
         float xa[2][16];
+        if (COH) {   // (one trip to memory for both groups; a slice of one group reads its 64 bytes twice)
+            ld_coh64x2(xsrc, xsrc + (g1 - g0 > 1 ? 256 : 0), xa[0], xa[1]);
+        } else {
 #pragma unroll
-        for (int gi = 0; gi < 2; gi++) {
-            if (COH) {
-#pragma unroll
-                for (int e = 0; e < 16; e++) xa[gi][e] = gi < g1 - g0 ? ld_coh(xsrc + 256 * gi + e) : 0.0f;
-            } else {
+            for (int gi = 0; gi < 2; gi++) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const float4 v = gi < g1 - g0 ? reinterpret_cast<const float4 *>(xsrc + 256 * gi)[q] : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -211,8 +244,13 @@ struct BgWave {
         if (g1 - g0 > 1) stage(1, xa[1]);
         for (int gi = 2; gi < g1 - g0; gi++) {
             float v[16];
+            if (COH) {
+                float twice[16];
+                ld_coh64x2(xsrc + 256 * gi, xsrc + 256 * gi, v, twice);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 16; e++) v[e] = COH ? ld_coh(xsrc + 256 * gi + e) : xsrc[256 * gi + e];
+                for (int e = 0; e < 16; e++) v[e] = xsrc[256 * gi + e];
+            }
             stage(gi, v);
         }
         __syncthreads();
@@ -280,8 +318,8 @@ struct BgWave {
             for (int nb = 0; nb < NB; nb++) {
                 float *o = cur.out + (long)nb * 16 * cur.rows;
                 if (COH) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++) { st_coh(o + i, y0[nb][i]); if (cur.two) st_coh(o + 16 + i, y1[nb][i]); }
+                    st_coh16(o, y0[nb]);
+                    if (cur.two) st_coh16(o + 16, y1[nb]);
                 } else {
                     *reinterpret_cast<v4f32 *>(o) = y0[nb];
                     if (cur.two) *reinterpret_cast<v4f32 *>(o + 16) = y1[nb];
@@ -398,10 +436,13 @@ struct BatchState {
     int n_prompt[kMaxBatch];
 };
 
-// x[b] = row token[b] of the embedding table (J/Run.java:72)
-static __global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, const BatchState *st, float *__restrict__ x, int dim)
+// x[b] = row token[b] of the embedding table (J/Run.java:72).  As the first kernel of a step it also clears the
+// counters of the grid barrier of k_bstep (bar_ctr: null without that kernel).
+static __global__ void __launch_bounds__(256) k_bembed(const float *__restrict__ emb, const BatchState *st, float *__restrict__ x, int dim,
+                                                unsigned *bar_ctr)
 {
     const int b = blockIdx.x;
+    if (bar_ctr && b == 0 && threadIdx.x < 1 + kBarGroups) bar_ctr[64 * threadIdx.x] = 0u;
     const float4 *src = reinterpret_cast<const float4 *>(emb + (long)st->token[b] * dim);
     float4 *dst = reinterpret_cast<float4 *>(x + (long)b * dim);
     for (int i = threadIdx.x; i < (dim >> 2); i += blockDim.x) dst[i] = src[i];

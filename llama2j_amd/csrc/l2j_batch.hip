@@ -1,6 +1,7 @@
 // libllama2j_hip.so: several sequences at once (l2j_decode_greedy_batch, l2j_batch_matmul).
 #include "l2j_internal.hpp"
 #include "batch_kernels.hpp"
+#include "batch_step.hpp"
 
 using namespace l2j;
 
@@ -121,6 +122,13 @@ struct l2j::BatchBufs {
     BatchState *st = nullptr;
     int *prompts = nullptr, *out = nullptr;         // (sequence, cap_pstride), (sequence, cap_steps)
     unsigned *done = nullptr;
+    unsigned *bar_ctr = nullptr;   // k_bstep: the counters of its grid barrier,
+    int *fault = nullptr;          // the flag a bounded wait sets when it runs out,
+    float *ssq = nullptr;          // the sums of squares behind the two norms of a layer,
+    BStep *step_args = nullptr;    // its argument (fixed for the life of the buffers)
+    int step_grid = 0;             // workgroups of k_bstep (0: the layers run as eight launches each)
+    int fuse_opt = 0;              // option batch_fuse when the step was planned
+    int h_fault = 0;
     int *h_pin = nullptr;   // pinned: every transfer of a call goes through it, as in the single-sequence loops
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -131,7 +139,7 @@ struct l2j::BatchBufs {
         if (graph) (void)hipGraphDestroy(graph);
         if (e0) (void)hipEventDestroy(e0);
         if (e1) (void)hipEventDestroy(e1);
-        void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done};
+        void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done, bar_ctr, fault, ssq, step_args};
         for (void *p : ps) (void)hipFree(p);
         if (h_pin) (void)hipHostFree(h_pin);
     }
@@ -168,8 +176,8 @@ size_t batch_lds_f32(int nseq) { return (size_t)nseq * (kBatchGps * 256 + kXPad)
 // workgroups of k_bgemm a compute unit holds at once: its 160 KB of LDS, and at most three by their registers
 int batch_resident(int nseq) { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds(nseq) + sizeof(float) * nseq * kBgMaxGps)))); }
 
-// The products of one layer's matrices `tensors` (the same input, the same row length) in one launch.
-void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part, int nseq)
+// The product of one layer's matrices `tensors` (the same input, the same row length) as one k_bgemm argument.
+BGemm bgemm_args(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part)
 {
     BGemm a{};
     int K = 0;
@@ -181,21 +189,36 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
         a.nmat++;
     }
     a.K = K; a.x = x; a.gps = kBatchGps;
-    // All workgroups of the launch are resident at once (batch_resident() per compute unit); a wave takes one unit of 16 or 32 rows
-    // after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
-    // activations they fetch from LDS).
-    const int nb = nseq / kBatch, waves = 4 * nb;
-    const int S = batch_slices(K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
-    int tiles = 2, gx = 1, best = 1 << 30;
+    return a;
+}
+
+// With at most gmax workgroups per slice of K (all of a launch resident at once) a wave takes one unit of 16 or 32 rows
+// after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
+// activations they fetch from LDS; bit t - 1 of `tiles_allowed`: units of t tiles may be used).  Returns the workgroups per slice.
+int bgemm_shape(const BGemm &a, int waves, int gmax, int tiles_allowed, int *tiles)
+{
+    int gx = 1, best = 1 << 30;
     for (int t = 2; t >= 1; t--) {
+        if (!(tiles_allowed & (1 << (t - 1)))) continue;
         int units = 0;
         for (int i = 0; i < a.nmat; i++) units += bg_units(a.rows[i], t);
         const int g = std::min(gmax, (units + waves - 1) / waves), iters = (units + waves * g - 1) / (waves * g);
         if (iters * t < best) {
-            best = iters * t; tiles = t;
+            best = iters * t; *tiles = t;
             gx = (units + waves * iters - 1) / (waves * iters);   // no more workgroups than that many rounds need
         }
     }
+    return gx;
+}
+
+// The products of one layer's matrices in one launch.
+void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part, int nseq)
+{
+    const BGemm a = bgemm_args(c, tensors, layer, x, part);
+    const int nb = nseq / kBatch;
+    const int S = batch_slices(a.K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
+    int tiles = 2;
+    const int gx = bgemm_shape(a, 4 * nb, gmax, 3, &tiles);
     const dim3 grid(gx, S), block(kBgThreads * nb);
     const size_t lds = batch_lds(nseq);
     if (nb == 1) {
@@ -207,6 +230,56 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
     }
 }
 
+// The grid of k_bstep: one workgroup per compute unit, all resident (by the runtime's count for the kernel and its LDS);
+// 0 when the shape does not fit (a product with more slices of K than workgroups) or the option is off.
+hipError_t plan_bstep(l2j_ctx *c, BatchBufs &b, int nseq)
+{
+    b.step_grid = 0;
+    if (!c->opt[OPT_BATCH_FUSE]) return hipSuccess;
+    const void *kernel = nseq == kBatch ? (const void *)k_bstep<1> : (const void *)k_bstep<2>;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(nseq));
+    if (e != hipSuccess) return e;
+    int per_cu = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBgThreads * (nseq / kBatch), batch_lds(nseq));
+    if (e != hipSuccess) return e;
+    if (per_cu < 1 || c->n_cu < batch_slices(c->cfg.hidden_dim) || c->n_cu < batch_slices(c->cfg.dim)) return hipSuccess;
+    b.step_grid = c->n_cu;
+    return hipSuccess;
+}
+
+// The argument of k_bstep for these buffers.
+BStep bstep_args(l2j_ctx *c, BatchBufs &b, int max_pos, int nseq)
+{
+    const l2j_config &cf = c->cfg;
+    const int nb = nseq / kBatch;
+    BStep a{};
+    a.g[BS_QKV] = bgemm_args(c, {L2J_WQ, L2J_WK, L2J_WV}, 0, b.xn, b.part);
+    a.g[BS_WO] = bgemm_args(c, {L2J_WO}, 0, b.xb, b.part);
+    a.g[BS_W13] = bgemm_args(c, {L2J_W1, L2J_W3}, 0, b.xn, b.part);
+    a.g[BS_W2] = bgemm_args(c, {L2J_W2}, 0, b.hb, b.part);
+    for (int k = 0; k < 4; k++) {
+        int tiles = 1;
+        a.gx[k] = bgemm_shape(a.g[k], 4 * nb, std::max(1, b.step_grid / batch_slices(a.g[k].K)), 1, &tiles);
+    }
+    a.n_layers = cf.n_layers; a.nseq = nseq; a.dim = cf.dim; a.hidden = cf.hidden_dim; a.n_heads = cf.n_heads;
+    a.kv_mul = cf.n_heads / cf.n_kv_heads; a.head_size = c->head_size; a.kv_dim = c->kv_dim;
+    a.sqrt_hs = sqrtf((float)c->head_size);
+    a.rope = c->rope; a.kc = b.kc; a.vc = b.vc; a.seq_stride = (long)cf.n_layers * max_pos; a.layer_stride = max_pos; a.st = b.st;
+    a.x = b.x; a.xn = b.xn; a.xb = b.xb; a.hb = b.hb; a.rmsw = c->rmsw; a.ssq = b.ssq;
+    a.silu = c->silu; a.exact = (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0;
+    a.bar.ctr = b.bar_ctr; a.bar.fault = b.fault; a.bar.ngroups = kBarGroups; a.bar.maxspin = c->opt[OPT_BARRIER_SPINS];
+    return a;
+}
+
+// All layers of a step in one launch.
+void launch_bstep(l2j_ctx *c, BatchBufs &b, int nseq)
+{
+    const dim3 grid(b.step_grid), block(kBgThreads * (nseq / kBatch));
+    const BStep *args = b.step_args;
+    if (nseq == kBatch) hipLaunchKernelGGL(k_bstep<1>, grid, block, batch_lds(nseq), c->stream, args);
+    else hipLaunchKernelGGL(k_bstep<2>, grid, block, batch_lds(nseq), c->stream, args);
+}
+
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
 void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride, int nseq)
 {
@@ -214,9 +287,13 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
     const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim;
     const int sd = batch_slices(dim), sh = batch_slices(hidden);
     hipStream_t s = c->stream;
-    { hipLaunchKernelGGL(k_bembed, dim3(nseq), dim3(256), 0, s, c->emb, b.st, b.x, dim); }
+    { hipLaunchKernelGGL(k_bembed, dim3(nseq), dim3(256), 0, s, c->emb, b.st, b.x, dim, b.step_grid > 0 ? b.bar_ctr : nullptr); }
     { hipLaunchKernelGGL(k_brms, dim3(nseq), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim); }
-    for (int l = 0; l < L; l++) {
+    if (b.step_grid > 0) {
+        launch_bstep(c, b, nseq);
+        { hipLaunchKernelGGL(k_brms, dim3(nseq), dim3(1024), 0, s, b.x, c->rmsw + (size_t)2 * L * dim, b.xn, dim); }   // the final norm
+    }
+    for (int l = 0; l < L && b.step_grid == 0; l++) {
         launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part, nseq);
         BAttn t{};
         t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
@@ -263,7 +340,7 @@ int hip_rc(hipError_t e, const char *what)
 int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
 {
     BatchBufs *old = c->batch;
-    if (old && old->nseq == nseq && old->cap_steps >= steps && old->cap_pstride >= pstride) return L2J_OK;
+    if (old && old->nseq == nseq && old->cap_steps >= steps && old->cap_pstride >= pstride && old->fuse_opt == c->opt[OPT_BATCH_FUSE]) return L2J_OK;
     if (old) {
         hipError_t se = hipStreamSynchronize(c->stream);
         if (se != hipSuccess) return hip_rc(se, "synchronize");
@@ -278,7 +355,7 @@ int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
     const size_t cache_floats = (size_t)nseq * L * steps * kvd;
     BatchBufs *b = new (std::nothrow) BatchBufs();
     if (!b) return fail(L2J_E_OOM, "batched decode: host allocation failed");
-    b->nseq = nseq; b->cap_steps = steps; b->cap_pstride = pstride;
+    b->nseq = nseq; b->cap_steps = steps; b->cap_pstride = pstride; b->fuse_opt = c->opt[OPT_BATCH_FUSE];
     hipError_t e = hipSuccess;
     auto alloc = [&](auto **p, size_t n) {
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(p), n * sizeof(**p));
@@ -288,6 +365,15 @@ int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
     for (int i = 0; i < 3; i++) alloc(&b->part[i], part_floats);
     alloc(&b->kc, cache_floats); alloc(&b->vc, cache_floats);
     alloc(&b->st, 1); alloc(&b->prompts, (size_t)nseq * pstride); alloc(&b->out, (size_t)nseq * steps); alloc(&b->done, 1);
+    alloc(&b->bar_ctr, (size_t)kBarStride); alloc(&b->fault, 1); alloc(&b->ssq, (size_t)2 * nseq * (dim / 256));
+    if (e == hipSuccess) e = hipMemsetAsync(b->bar_ctr, 0, kBarStride * sizeof(unsigned), c->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(b->fault, 0, sizeof(int), c->stream);
+    alloc(&b->step_args, 1);
+    if (e == hipSuccess) e = plan_bstep(c, *b, nseq);
+    if (e == hipSuccess && b->step_grid > 0) {
+        const BStep a = bstep_args(c, *b, steps, nseq);
+        e = hipMemcpy(b->step_args, &a, sizeof(a), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess) e = hipEventCreate(&b->e0);
     if (e == hipSuccess) e = hipEventCreate(&b->e1);
     const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)nseq * pstride, out_ints = (size_t)nseq * steps;
@@ -394,6 +480,15 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
         (void)hipFree(dlog);
         dlog = nullptr;
         if (e != hipSuccess) return hip_rc(e, "logits read-back");
+    }
+    if (b.step_grid > 0) {
+        int fault = 0;
+        if ((e = hipMemcpy(&fault, b.fault, sizeof(int), hipMemcpyDeviceToHost)) != hipSuccess) return hip_rc(e, "fault flag");
+        if (fault) {
+            (void)hipMemset(b.fault, 0, sizeof(int));
+            return fail(L2J_E_HIP, "batched decode: a bounded wait at a grid barrier ran out (is another process using the GPU?); "
+                                   "option batch_fuse = 0 runs the same step without grid barriers");
+        }
     }
     float ms = 0.0f;
     if (steps > 1 && (e = hipEventElapsedTime(&ms, b.e0, b.e1)) != hipSuccess) return hip_rc(e, "timing");

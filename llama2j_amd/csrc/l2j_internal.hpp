@@ -55,7 +55,7 @@ struct QTensor {
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_BATCH_FUSE, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -83,6 +83,7 @@ inline const OptionDef kOptions[OPT_COUNT] = {
     {"graph_tokens", 32, false},       // tokens per replay of the decode loops' graph (1: only the one-token graph)
     {"fast_steps", 1, false},          // k_token folds rows of dim codes without clamping when they are exactly one step
     {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
+    {"batch_fuse", 1, true},           // batched decode: the layers of a step in one launch with grid barriers (0: eight launches per layer)
 };
 
 inline int option_from_env(int i)

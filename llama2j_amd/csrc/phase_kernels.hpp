@@ -1043,7 +1043,7 @@ struct ClsRun {
         uv.x = uv.y = uv.z = uv.w = u;
         const long step = (long)G * a.threads;
         for (long i = (long)blockIdx.x * a.threads + 64 * wave + lane; i < a.unset_n4; i += step)
-            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(a.unset_p + i), "v"(uv) : "memory");
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 2" ::"v"(a.unset_p + i), "v"(uv) : "memory");   // (wait states: a 16-byte store reads its data registers after it has issued)
     }
 
     // smem: as for a matvec phase, then 16 floats and 16 ints for the per-wave maxima
