@@ -130,7 +130,7 @@ struct BgWave {
     static constexpr int NSEQ = kBatch * NB, WAVES = 4 * NB;
     struct Unit {   // 16 * TILES rows of one matrix: where this lane's codes, scales and results are
         const uint4 *c0, *c1;
-        const float2 *gs0, *gs1;
+        const float4 *gs0, *gs1;   // (rm, min) of rows 4 s + (0..3) of the tile: 32 bytes
         float *out;
         int rows;
         bool two;
@@ -138,33 +138,53 @@ struct BgWave {
     const BGemm *ap;   // (a pointer, so that a kernel with several products can aim one BgWave at each in turn)
     long layer;        // the matrices of this layer: layer * rows * K codes behind m.off
     int by, lane, r, s, ngroups, g0, g1, total, stride, u;
+    // The product's matrices, read from the argument once per product: looked up there for every unit (the argument
+    // lies in memory, and a kernel whose other phases contain memory barriers reads it again each time), finding a
+    // unit's addresses cost 1.2 us per unit, measured.
+    struct Mat {
+        const uint8_t *codes;
+        const float2 *gs;
+        float *part;
+        int rows, units;
+    };
+    Mat m0, m1, m2;   // (named, not an array: indexed by a variable the wave's whole state would move to scratch memory)
+    int nmat;
     Unit cur;
     uint4 w0[4], w1[4];
+    float4 ws0[2], ws1[2];   // the scales of the group whose codes are in w0, w1
 
     __device__ __forceinline__ BgWave(const BGemm &a_) : ap(&a_), layer(0) {}
 
     __device__ __forceinline__ Unit locate(int unit) const
     {
-        const BGemm &a = *ap;
-        int mi = 0;
-        while (mi + 1 < a.nmat && unit >= bg_units(a.rows[mi], TILES)) { unit -= bg_units(a.rows[mi], TILES); mi++; }
-        QMat mat = a.m[mi];
-        const int rows = a.rows[mi], row0 = unit * 16 * TILES;
-        mat.off += layer * rows * a.K;
+        Mat m = m0;
+        if (nmat > 1 && unit >= m0.units) {
+            unit -= m0.units;
+            m = m1;
+            if (nmat > 2 && unit >= m1.units) { unit -= m1.units; m = m2; }
+        }
+        const uint8_t *codes = m.codes;
+        const float2 *gs = m.gs;
+        float *part = m.part;
+        const int rows = m.rows, row0 = unit * 16 * TILES;
         Unit n;
         n.rows = rows;
         n.two = TILES == 2 && row0 + 16 < rows;
         const long block = (long)(row0 >> 4) * ngroups + g0;   // the tile's first block of this slice
-        n.c0 = reinterpret_cast<const uint4 *>(mat.codes + mat.off + (block << 12)) + lane;
+        n.c0 = reinterpret_cast<const uint4 *>(codes + (block << 12)) + lane;
         n.c1 = n.c0 + (n.two ? (long)ngroups << 8 : 0L);   // the next tile: ngroups blocks of 256 16-byte words on
-        n.gs0 = mat.gs + (mat.off >> 8) + (block << 4) + 4 * s;
-        n.gs1 = n.gs0 + (n.two ? (long)ngroups << 4 : 0L);
-        n.out = a.part[mi] + ((long)by * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
+        n.gs0 = reinterpret_cast<const float4 *>(gs + (block << 4) + 4 * s);
+        n.gs1 = n.gs0 + (n.two ? (long)ngroups << 3 : 0L);
+        n.out = part + ((long)by * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
         return n;
     }
 
-    __device__ __forceinline__ void request(const Unit &n)   // one group of the unit's codes
+    // One group of the unit: its scales, then its codes (a wave's loads return in order: requested behind the codes of
+    // the group after it, the scales would only arrive with those).
+    __device__ __forceinline__ void request(const Unit &n)
     {
+#pragma unroll
+        for (int i = 0; i < 2; i++) { ws0[i] = n.gs0[i]; if (TILES == 2) ws1[i] = n.gs1[i]; }
 #pragma unroll
         for (int T = 0; T < 4; T++) { w0[T] = load_stream(n.c0 + 64 * T); if (TILES == 2) w1[T] = load_stream(n.c1 + 64 * T); }
     }
@@ -181,8 +201,21 @@ struct BgWave {
         r = lane & 15; s = lane >> 4;
         ngroups = a.K >> 8;
         g0 = by * a.gps; g1 = min(ngroups, g0 + a.gps);
-        total = 0;
-        for (int i = 0; i < a.nmat; i++) total += bg_units(a.rows[i], TILES);
+        nmat = a.nmat;
+        auto matrix = [&](int i) {
+            Mat m{};
+            if (i < a.nmat) {
+                const long off = a.m[i].off + layer * a.rows[i] * a.K;
+                m.codes = a.m[i].codes + off;
+                m.gs = a.m[i].gs + (off >> 8);
+                m.part = a.part[i];
+                m.rows = a.rows[i];
+                m.units = bg_units(a.rows[i], TILES);
+            }
+            return m;
+        };
+        m0 = matrix(0); m1 = matrix(1); m2 = matrix(2);
+        total = m0.units + m1.units + m2.units;
         stride = gx * WAVES;
         u = bx * WAVES + (tid >> 6);
         cur = Unit{};
@@ -190,6 +223,18 @@ struct BgWave {
             cur = locate(u);
             if (first) request(cur);
         }
+    }
+
+    // The three planes of sequence r (+ 16 per column block) at k = 64 T + 16 s + j of group gi of the slice: [nb][j < 8, j >= 8][plane]
+    __device__ __forceinline__ void fetch_x(const unsigned short *xk, int plane, int pitch, int T, v8bf16 (&bx)[NB][2][3]) const
+    {
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) {
+                bx[nb][0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
+                bx[nb][1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
+            }
     }
 
     // requested = begin(.., true) was called.  COH: the activations were written by other workgroups of this launch and
@@ -262,47 +307,58 @@ struct BgWave {
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) y0[nb] = y1[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
             for (int g = g0; g < g1; g++) {
+                const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
+                // The activations of a block of 64 k are fetched from LDS while the block before it is multiplied:
+                // fetched where they are used, every few MFMAs waited for LDS, and these reads were two thirds of a
+                // group's time, measured.
+                v8bf16 bxa[NB][2][3];
+                fetch_x(xk, plane, pitch, 0, bxa);
                 uint4 u0[4], u1[4];
+                float4 us0[2], us1[2];
 #pragma unroll
                 for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
-                // the next group's codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
+#pragma unroll
+                for (int i = 0; i < 2; i++) { us0[i] = ws0[i]; us1[i] = ws1[i]; }
+                // the next group's scales and codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
                 if (g + 1 < g1) {
-                    cur.c0 += 256; cur.c1 += 256;
+                    cur.c0 += 256; cur.c1 += 256; cur.gs0 += 8; cur.gs1 += 8;
                     request(cur);
                 } else if (more) {
                     request(nxt);
                 }
-                float2 sc0[4], sc1[4];   // (rm, min) of rows 4 s + (0..3) of the tile
-#pragma unroll
-                for (int i = 0; i < 4; i++) { sc0[i] = cur.gs0[i]; if (TILES == 2) sc1[i] = cur.gs1[i]; }
                 v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
-                const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
 #pragma unroll
-                for (int T = 0; T < 4; T++) {
+                for (int T = 0; T < 4; T++) {   // blocks of 64 k
+                    v8bf16 bx[NB][2][3];
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                        for (int h = 0; h < 2; h++)
+#pragma unroll
+                            for (int pl = 0; pl < 3; pl++) bx[nb][h][pl] = bxa[nb][h][pl];
+                    if (T + 1 < 4) fetch_x(xk, plane, pitch, T + 1, bxa);   // (the compiler renames the registers: the copy above costs nothing)
                     const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
                     v8bf16 a10 = a00, a11 = a01;
                     if (TILES == 2) { a10 = codes_bf16(u1[T].x, u1[T].y); a11 = codes_bf16(u1[T].z, u1[T].w); }
 #pragma unroll
                     for (int nb = 0; nb < NB; nb++) {
-                        v8bf16 bx[2][3];   // [j < 8, j >= 8][plane]
-#pragma unroll
-                        for (int pl = 0; pl < 3; pl++) {
-                            bx[0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
-                            bx[1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
-                        }
 #pragma unroll
                         for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
-                            acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[0][pl], acc0[nb], 0, 0, 0);
-                            acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[1][pl], acc2[nb], 0, 0, 0);
+                            acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[nb][0][pl], acc0[nb], 0, 0, 0);
+                            acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[nb][1][pl], acc2[nb], 0, 0, 0);
                             if (TILES == 2) {
-                                acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[0][pl], acc1[nb], 0, 0, 0);
-                                acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[1][pl], acc3[nb], 0, 0, 0);
+                                acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[nb][0][pl], acc1[nb], 0, 0, 0);
+                                acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[nb][1][pl], acc3[nb], 0, 0, 0);
                             }
                         }
                     }
                 }
+                const float2 sc0[4] = {make_float2(us0[0].x, us0[0].y), make_float2(us0[0].z, us0[0].w), make_float2(us0[1].x, us0[1].y),
+                                       make_float2(us0[1].z, us0[1].w)};
+                const float2 sc1[4] = {make_float2(us1[0].x, us1[0].y), make_float2(us1[0].z, us1[0].w), make_float2(us1[1].x, us1[1].y),
+                                       make_float2(us1[1].z, us1[1].w)};
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
                     const float sxv = sxs[16 * nb + r][g - g0];   // this lane's column is sequence 16 nb + r
@@ -312,7 +368,6 @@ struct BgWave {
                         if (TILES == 2) y1[nb][i] += fmaf(sc1[i].x, acc1[nb][i] + acc3[nb][i], sc1[i].y * sxv);
                     }
                 }
-                cur.gs0 += 16; cur.gs1 += 16;
             }
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) {

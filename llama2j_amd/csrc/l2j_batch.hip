@@ -218,7 +218,7 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
     const int nb = nseq / kBatch;
     const int S = batch_slices(a.K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
     int tiles = 2;
-    const int gx = bgemm_shape(a, 4 * nb, gmax, 3, &tiles);
+    const int gx = bgemm_shape(a, 4 * nb, gmax, 1, &tiles);
     const dim3 grid(gx, S), block(kBgThreads * nb);
     const size_t lds = batch_lds(nseq);
     if (nb == 1) {
