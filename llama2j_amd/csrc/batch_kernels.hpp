@@ -16,10 +16,9 @@ namespace l2j {
 constexpr int kBatch = 16;          // sequences per column block: the 16 columns of one MFMA
 constexpr int kMaxBatch = 32;       // sequences per step: one or two column blocks
 constexpr int kBgThreads = 256;     // threads per column block: four waves per 16 sequences share the staged activations
-constexpr int kBgRowsPerWave = 32;  // two 16-row tiles share the activations fetched from LDS
+constexpr int kBgRowsPerWave = 32;  // k_bgemm_f32: two 16-row tiles share the activations fetched from LDS
 constexpr int kBgRowsPerWG = kBgRowsPerWave * (kBgThreads / 64);
 constexpr int kXPad = 4;            // floats between the slices of two sequences in LDS: a quarter wave's 16-byte reads then cover every bank once
-constexpr int kXPadH = 8;           // the same for the bf16 planes of k_bgemm (16 bytes)
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf16 __attribute__((ext_vector_type(8)));
@@ -56,7 +55,8 @@ __device__ __forceinline__ void st_coh16(float *p, v4f32 v)
 // y[b][r] = sum_k dequant(W[r][k]) * x[b][k], split over slices of K: part[slice][b][r].  Up to three matrices that
 // share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
 constexpr int kBgMaxMat = 3;
-constexpr int kBgMaxGps = 16;       // most groups per slice
+constexpr int kBgGroups = 4;        // groups of 256 codes per slice of K: one per wave (16 sequences) or per pair of waves (32)
+constexpr int kBgDepth = 4;         // tiles whose codes a wave has in flight (divides the number of waves: a tile's register set is known at compile time)
 struct BGemm {
     QMat m[kBgMaxMat];        // the tensor's copy in tile order (k_btile), m.off: the layer's matrix (a multiple of 4096)
     int rows[kBgMaxMat];      // rows % 16 == 0
@@ -64,11 +64,9 @@ struct BGemm {
     int nmat;
     int K;                    // K % 256 == 0
     const float *x;           // (nseq, K)
-    int gps;                  // groups of 256 codes per slice
 };
 
-
-__host__ __device__ inline int bg_units(int rows, int tiles) { return (rows + 16 * tiles - 1) / (16 * tiles); }
+__host__ __device__ inline int bg_slices(int K) { return ((K >> 8) + kBgGroups - 1) / kBgGroups; }
 
 // The batched path keeps its own copy of the quantized matrices, in the order its waves read them: the 16 rows x 256
 // codes of a (tile of 16 rows, group) block are 4 KB in a row, [T][lane][16 codes] with lane = r + 16 s holding row r of
@@ -92,8 +90,13 @@ static __global__ void __launch_bounds__(256) k_btile(const uint8_t *__restrict_
         tgs[(layer * (long)rows * K >> 8) + (long)block * 16 + in] = gs[((layer * (long)rows * K + (long)(16 * tile + in) * K) >> 8) + g];
 }
 
-// LDS of k_bgemm for slices of gps groups: three bf16 planes of (nseq, gps * 256 + kXPadH)
-__host__ __device__ inline size_t bg_lds_bytes(int gps, int nseq) { return (size_t)3 * nseq * (gps * 256 + kXPadH) * sizeof(unsigned short); }
+// LDS of k_bgemm: the sums of a batch of tiles (as many tiles as the workgroup has waves; per tile, wave and column block
+// 64 lanes x 16 bytes), then every wave's sums of its activations per sequence
+__host__ __device__ inline size_t bg_lds_bytes(int nseq, int hv)
+{
+    const size_t nb = nseq / kBatch, waves = 4 * hv;
+    return waves * waves * nb * 1024 + waves * nseq * sizeof(float);
+}
 
 // eight codes (two words of a row) as eight bf16: the upper halves of the codes' floats, two to a register
 __device__ __forceinline__ v8bf16 codes_bf16(uint32_t d0, uint32_t d1)
@@ -116,91 +119,87 @@ __device__ __forceinline__ void split_bf16(float x, uint32_t h[3])
     h[0] = b0 >> 16; h[1] = b1 >> 16; h[2] = __float_as_uint(r2) >> 16;
 }
 
-// Workgroup (by: one slice of K; bx of gx: a share of the rows): the slice of the 16 NB activation vectors is staged in LDS
-// once, as three bf16 planes, then every wave takes units of 16 * TILES rows (of all the launch's matrices, in order) in
-// turn: unit bx * 4 NB + wave, then every gx * 4 NB-th.  A lane (r = lane % 16, s = lane / 16) holds the codes of
-// row r at k = 64 T + 16 s + j (T < 4, j < 16: four 16-byte loads per group and tile, from the copy in tile order); one MFMA
-// multiplies the 16 rows by 16 sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane and
-// column block.  After the 24 NB MFMAs of a group the 16 x 16 sums get the group's scale and offset.  TILES = 2: two
-// tiles share the activations fetched from LDS; NB = 2: two column blocks share the converted codes.  256 NB threads.
+// Workgroup (by: one slice of K, four groups of 256; bx of gx: a share of the 16-row tiles of the launch's matrices, in
+// order: tile bx, then every gx-th).  The ACTIVATIONS stay in registers and the codes stream past them: a wave owns one
+// group of the slice (with 32 sequences, NB = 2: half a group; two waves per group) and holds, for every one of its 64-k
+// blocks, the three bf16 planes of its 16 NB sequences as MFMA operands (96 registers); all waves of the workgroup take
+// the same tiles, each the part of the tile's codes that belongs to its k (4 KB, or 2 KB: [T][lane][16 codes] in tile
+// order, lane (r = lane % 16, s = lane / 16) holding row r at k = 64 T + 16 s + j; one MFMA multiplies the 16 rows by 16
+// sequences over the eight k (j < 8, or j >= 8) of each of the four s, once per plane and column block), kBgDepth
+// tiles' codes in flight.  The waves' 16 x 16 sums of a tile meet in LDS: after every batch of as many tiles as the
+// workgroup has waves, wave w adds up tile w of the batch: per group the halves, times the group's scale, plus its
+// offset times the sum of the activations, group after group (K/MatMul.java:137-147), and writes the slice's partial
+// sums.  (A first version staged the activations in LDS as bf16 planes and every wave fetched them from there for every
+// tile: 12 bytes of LDS reads per byte of codes, two thirds of the time of a group, measured with time stamps in the
+// kernel; here LDS carries 2 bytes per byte of codes.)
 // The work of one wave, in two steps so that a kernel with several phases can request the first codes of a product
 // before the phase (and the grid barrier) that produces its activations: begin(), then run().
-template <int TILES, int NB>
+template <int NB, int HV>   // HV: waves per group (1: a wave takes the group's 256 k, 2: 128 k)
 struct BgWave {
-    static constexpr int NSEQ = kBatch * NB, WAVES = 4 * NB;
-    struct Unit {   // 16 * TILES rows of one matrix: where this lane's codes, scales and results are
-        const uint4 *c0, *c1;
-        const float4 *gs0, *gs1;   // (rm, min) of rows 4 s + (0..3) of the tile: 32 bytes
-        float *out;
-        int rows;
-        bool two;
-    };
-    const BGemm *ap;   // (a pointer, so that a kernel with several products can aim one BgWave at each in turn)
-    long layer;        // the matrices of this layer: layer * rows * K codes behind m.off
-    int by, lane, r, s, ngroups, g0, g1, total, stride, u;
-    // The product's matrices, read from the argument once per product: looked up there for every unit (the argument
-    // lies in memory, and a kernel whose other phases contain memory barriers reads it again each time), finding a
-    // unit's addresses cost 1.2 us per unit, measured.
+    static constexpr int NSEQ = kBatch * NB, WAVES = 4 * HV, TB = 4 / HV;   // TB: blocks of 64 k per wave
     struct Mat {
         const uint8_t *codes;
         const float2 *gs;
         float *part;
-        int rows, units;
+        int rows, tiles;
     };
-    Mat m0, m1, m2;   // (named, not an array: indexed by a variable the wave's whole state would move to scratch memory)
-    int nmat;
-    Unit cur;
-    uint4 w0[4], w1[4];
-    float4 ws0[2], ws1[2];   // the scales of the group whose codes are in w0, w1
+    struct Tile {   // a 16-row tile of one of the matrices
+        const uint8_t *codes;   // its first block (group 0)
+        const float2 *gs;
+        float *out;             // row0 of sequence 0 of this slice
+        int rows;
+    };
+    const BGemm *ap;   // (a pointer, so that a kernel with several products can aim one BgWave at each in turn)
+    long layer;        // the matrices of this layer: layer * rows * K codes behind m.off
+    Mat m0, m1, m2;    // (named, not an array: indexed by a variable the wave's whole state would move to scratch memory)
+    int nmat, ntiles, by, lane, c, s, wave, gq, h, ngroups, g0, ng, first, gx, cnt;
+    bool active;       // this wave's group exists (the last slice of K may have fewer than four)
+    uint4 cw[kBgDepth][TB];
 
     __device__ __forceinline__ BgWave(const BGemm &a_) : ap(&a_), layer(0) {}
 
-    __device__ __forceinline__ Unit locate(int unit) const
+    __device__ __forceinline__ Tile locate(int tile) const
     {
         Mat m = m0;
-        if (nmat > 1 && unit >= m0.units) {
-            unit -= m0.units;
+        if (nmat > 1 && tile >= m0.tiles) {
+            tile -= m0.tiles;
             m = m1;
-            if (nmat > 2 && unit >= m1.units) { unit -= m1.units; m = m2; }
+            if (nmat > 2 && tile >= m1.tiles) { tile -= m1.tiles; m = m2; }
         }
-        const uint8_t *codes = m.codes;
-        const float2 *gs = m.gs;
-        float *part = m.part;
-        const int rows = m.rows, row0 = unit * 16 * TILES;
-        Unit n;
-        n.rows = rows;
-        n.two = TILES == 2 && row0 + 16 < rows;
-        const long block = (long)(row0 >> 4) * ngroups + g0;   // the tile's first block of this slice
-        n.c0 = reinterpret_cast<const uint4 *>(codes + (block << 12)) + lane;
-        n.c1 = n.c0 + (n.two ? (long)ngroups << 8 : 0L);   // the next tile: ngroups blocks of 256 16-byte words on
-        n.gs0 = reinterpret_cast<const float4 *>(gs + (block << 4) + 4 * s);
-        n.gs1 = n.gs0 + (n.two ? (long)ngroups << 3 : 0L);
-        n.out = part + ((long)by * NSEQ + r) * rows + row0 + 4 * s;   // rows row0 + 4 s + (0..3) of sequence r (+ 16 per column block)
-        return n;
+        Tile t;
+        t.rows = m.rows;
+        const long block = (long)tile * ngroups;
+        t.codes = m.codes + (block << 12);
+        t.gs = m.gs + (block << 4);
+        t.out = m.part + (long)by * NSEQ * m.rows + 16 * tile;
+        return t;
     }
 
-    // One group of the unit: its scales, then its codes (a wave's loads return in order: requested behind the codes of
-    // the group after it, the scales would only arrive with those).
-    __device__ __forceinline__ void request(const Unit &n)
+    // The codes of this wave's k of the i-th tile of the workgroup into register set `slot`.  Unconditionally (past the
+    // workgroup's last tile: that tile again; a wave without a group: the slice's last group): after a load that may or
+    // may not have been issued the compiler can only wait for all loads, and the sets in flight would be waited for too.
+    __device__ __forceinline__ void request(int slot, int i)
     {
+        const Tile t = locate(min(first + min(i, cnt - 1) * gx, ntiles - 1));
+        const uint4 *p = reinterpret_cast<const uint4 *>(t.codes + ((long)(g0 + min(gq, ng - 1)) << 12)) + (h * TB) * 64 + lane;
 #pragma unroll
-        for (int i = 0; i < 2; i++) { ws0[i] = n.gs0[i]; if (TILES == 2) ws1[i] = n.gs1[i]; }
-#pragma unroll
-        for (int T = 0; T < 4; T++) { w0[T] = load_stream(n.c0 + 64 * T); if (TILES == 2) w1[T] = load_stream(n.c1 + 64 * T); }
+        for (int T = 0; T < TB; T++) cw[slot][T] = load_stream(p + 64 * T);
     }
 
     // This wave's share of workgroup (bx, by) of a gx-wide grid; first = false: the first codes are not requested yet
-    // (run() does it once the first activations are requested: a wave's loads return in order, and behind 8 KB of codes
-    // the activations would arrive with them).
-    __device__ __forceinline__ void begin(int bx, int by_, int gx, bool first)
+    // (run() does it once the activations are requested: a wave's loads return in order, and behind the codes the
+    // activations would arrive with them).
+    __device__ __forceinline__ void begin(int bx, int by_, int gx_, bool first_codes)
     {
         const BGemm &a = *ap;
         const int tid = threadIdx.x;
         by = by_;
-        lane = tid & 63;
-        r = lane & 15; s = lane >> 4;
+        lane = tid & 63; wave = tid >> 6;
+        c = lane & 15; s = lane >> 4;
+        gq = wave / HV; h = wave % HV;
         ngroups = a.K >> 8;
-        g0 = by * a.gps; g1 = min(ngroups, g0 + a.gps);
+        g0 = by * kBgGroups; ng = min(kBgGroups, ngroups - g0);
+        active = gq < ng;
         nmat = a.nmat;
         auto matrix = [&](int i) {
             Mat m{};
@@ -210,190 +209,159 @@ struct BgWave {
                 m.gs = a.m[i].gs + (off >> 8);
                 m.part = a.part[i];
                 m.rows = a.rows[i];
-                m.units = bg_units(a.rows[i], TILES);
+                m.tiles = a.rows[i] >> 4;
             }
             return m;
         };
         m0 = matrix(0); m1 = matrix(1); m2 = matrix(2);
-        total = m0.units + m1.units + m2.units;
-        stride = gx * WAVES;
-        u = bx * WAVES + (tid >> 6);
-        cur = Unit{};
-        if (u < total) {
-            cur = locate(u);
-            if (first) request(cur);
+        ntiles = m0.tiles + m1.tiles + m2.tiles;
+        first = bx; gx = gx_;
+        cnt = bx < ntiles ? (ntiles - bx + gx - 1) / gx : 0;
+        if (first_codes) {
+#pragma unroll
+            for (int d = 0; d < kBgDepth; d++) request(d, d);
         }
-    }
-
-    // The three planes of sequence r (+ 16 per column block) at k = 64 T + 16 s + j of group gi of the slice: [nb][j < 8, j >= 8][plane]
-    __device__ __forceinline__ void fetch_x(const unsigned short *xk, int plane, int pitch, int T, v8bf16 (&bx)[NB][2][3]) const
-    {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int pl = 0; pl < 3; pl++) {
-                bx[nb][0][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T);
-                bx[nb][1][pl] = *reinterpret_cast<const v8bf16 *>(xk + pl * plane + nb * 16 * pitch + 64 * T + 8);
-            }
     }
 
     // requested = begin(.., true) was called.  COH: the activations were written by other workgroups of this launch and
     // the partial sums are read by other workgroups of it (device-coherent loads, write-through stores).
+    // lds: bg_lds_bytes(NSEQ, HV) bytes, free when the workgroup's waves get here.
     template <bool COH>
-    __device__ __forceinline__ void run(unsigned short *xh, float (*sxs)[kBgMaxGps], bool requested)
+    __device__ __forceinline__ void run(float *lds, bool requested)
     {
         const BGemm &a = *ap;
-        const int tid = threadIdx.x, nk = (g1 - g0) << 8;
-        // Staging: 16 threads per sequence, 16 consecutive activations of every group each: their sum (for the groups'
-        // offsets) and their three bf16 parts.
-        const int pitch = nk + kXPadH, plane = NSEQ * pitch;
-        const int sb = tid >> 4, pt = tid & 15;
-        const float *xsrc = a.x + (long)sb * a.K + (g0 << 8) + 16 * pt;
-        float xa[2][16];
-        if (COH) {   // (one trip to memory for both groups; a slice of one group reads its 64 bytes twice)
-            ld_coh64x2(xsrc, xsrc + (g1 - g0 > 1 ? 256 : 0), xa[0], xa[1]);
-        } else {
+        v4f32 *raw = reinterpret_cast<v4f32 *>(lds);                      // [tile of the batch][wave][column block][lane]
+        float *sxw = lds + (size_t)WAVES * WAVES * NB * 256;              // [wave][sequence]
+        // This wave's activations: sequence c (+ 16 per column block) at k = 64 T + 16 s + j of its blocks T, as the
+        // three bf16 planes, eight k (j < 8, j >= 8) to an MFMA operand; and their sum per sequence.
+        v8bf16 bx[NB][TB][2][3];
 #pragma unroll
-            for (int gi = 0; gi < 2; gi++) {
+        for (int nb = 0; nb < NB; nb++) {
+            const float *xsrc = a.x + (long)(16 * nb + c) * a.K + ((long)(g0 + (active ? gq : 0)) << 8) + h * (64 * TB) + 16 * s;
+            float t = 0.0f;
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const float4 v = gi < g1 - g0 ? reinterpret_cast<const float4 *>(xsrc + 256 * gi)[q] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    xa[gi][4 * q] = v.x; xa[gi][4 * q + 1] = v.y; xa[gi][4 * q + 2] = v.z; xa[gi][4 * q + 3] = v.w;
+            for (int T2 = 0; T2 < TB; T2 += 2) {
+                float v[2][16];
+                if (COH) {
+                    ld_coh64x2(xsrc + 64 * T2, xsrc + 64 * (T2 + 1), v[0], v[1]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 2; e++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const float4 f = reinterpret_cast<const float4 *>(xsrc + 64 * (T2 + e))[q];
+                            v[e][4 * q] = f.x; v[e][4 * q + 1] = f.y; v[e][4 * q + 2] = f.z; v[e][4 * q + 3] = f.w;
+                        }
+                }
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const float (&w)[16] = v[e];
+                    t += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7])) + ((w[8] + w[9]) + (w[10] + w[11])) +
+                         ((w[12] + w[13]) + (w[14] + w[15]));
+#pragma unroll
+                    for (int hf = 0; hf < 2; hf++) {
+                        uint32_t pk[3][4];
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            uint32_t lo[3], hi[3];
+                            split_bf16(w[8 * hf + 2 * q], lo);
+                            split_bf16(w[8 * hf + 2 * q + 1], hi);
+#pragma unroll
+                            for (int pl = 0; pl < 3; pl++) pk[pl][q] = lo[pl] | (hi[pl] << 16);
+                        }
+#pragma unroll
+                        for (int pl = 0; pl < 3; pl++)
+                            bx[nb][T2 + e][hf][pl] = __builtin_bit_cast(v8bf16, make_uint4(pk[pl][0], pk[pl][1], pk[pl][2], pk[pl][3]));
+                    }
                 }
             }
+            t += __shfl_xor(t, 16);
+            t += __shfl_xor(t, 32);
+            if (s == 0) sxw[wave * NSEQ + 16 * nb + c] = active ? t : 0.0f;
         }
-        if (!requested && u < total) request(cur);
-        auto stage = [&](int gi, const float (&v)[16]) {
-            float t = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7])) + ((v[8] + v[9]) + (v[10] + v[11])) +
-                      ((v[12] + v[13]) + (v[14] + v[15]));
+        if (!requested) {
 #pragma unroll
-            for (int off = 8; off > 0; off >>= 1) t += __shfl_xor(t, off);
-            if (pt == 0) sxs[sb][gi] = t;
-            uint32_t pk[3][8];
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                uint32_t lo[3], hi[3];
-                split_bf16(v[2 * e], lo);
-                split_bf16(v[2 * e + 1], hi);
-#pragma unroll
-                for (int pl = 0; pl < 3; pl++) pk[pl][e] = lo[pl] | (hi[pl] << 16);
-            }
-            unsigned short *dst = xh + sb * pitch + (gi << 8) + 16 * pt;
-#pragma unroll
-            for (int pl = 0; pl < 3; pl++) {
-                reinterpret_cast<uint4 *>(dst + pl * plane)[0] = make_uint4(pk[pl][0], pk[pl][1], pk[pl][2], pk[pl][3]);
-                reinterpret_cast<uint4 *>(dst + pl * plane)[1] = make_uint4(pk[pl][4], pk[pl][5], pk[pl][6], pk[pl][7]);
-            }
-        };
-        stage(0, xa[0]);
-        if (g1 - g0 > 1) stage(1, xa[1]);
-        for (int gi = 2; gi < g1 - g0; gi++) {
-            float v[16];
-            if (COH) {
-                float twice[16];
-                ld_coh64x2(xsrc + 256 * gi, xsrc + 256 * gi, v, twice);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 16; e++) v[e] = xsrc[256 * gi + e];
-            }
-            stage(gi, v);
+            for (int d = 0; d < kBgDepth; d++) request(d, d);
         }
         __syncthreads();
-        for (; u < total; u += stride) {
-            const bool more = u + stride < total;
-            Unit nxt{};
-            if (more) nxt = locate(u + stride);
-            v4f32 y0[NB], y1[NB];
+        for (int i0 = 0; i0 < cnt; i0 += WAVES) {
+            const int nbatch = min(WAVES, cnt - i0);
+            // the scales of the tile this wave will add up, requested ahead of the batch's codes
+            float4 sc[kBgGroups][2];
+            const Tile mine = locate(min(first + min(i0 + wave, cnt - 1) * gx, ntiles - 1));   // (unconditionally, as the codes)
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) y0[nb] = y1[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
-            for (int g = g0; g < g1; g++) {
-                const unsigned short *xk = xh + r * pitch + ((g - g0) << 8) + 16 * s;   // sequence r (+ 16 per column block), k = 64 T + 16 s + j
-                // The activations of a block of 64 k are fetched from LDS while the block before it is multiplied:
-                // fetched where they are used, every few MFMAs waited for LDS, and these reads were two thirds of a
-                // group's time, measured.
-                v8bf16 bxa[NB][2][3];
-                fetch_x(xk, plane, pitch, 0, bxa);
-                uint4 u0[4], u1[4];
-                float4 us0[2], us1[2];
+            for (int q = 0; q < kBgGroups; q++) {
+                const float4 *gp = reinterpret_cast<const float4 *>(mine.gs + ((g0 + min(q, ng - 1)) << 4) + 4 * s);   // (rm, min) of rows 4 s + (0..3)
+                sc[q][0] = gp[0]; sc[q][1] = gp[1];
+            }
 #pragma unroll
-                for (int T = 0; T < 4; T++) { u0[T] = w0[T]; u1[T] = w1[T]; }
+            for (int ii = 0; ii < WAVES; ii++) {
+                // (the register set of a tile is fixed: moving sets along as in a queue would wait for the loads in flight)
+                uint4 (&cu)[TB] = cw[ii % kBgDepth];
+                v8bf16 a0[TB], a1[TB];
 #pragma unroll
-                for (int i = 0; i < 2; i++) { us0[i] = ws0[i]; us1[i] = ws1[i]; }
-                // the next group's scales and codes (of this unit, or the first of the wave's next one) are requested before this one is multiplied
-                if (g + 1 < g1) {
-                    cur.c0 += 256; cur.c1 += 256; cur.gs0 += 8; cur.gs1 += 8;
-                    request(cur);
-                } else if (more) {
-                    request(nxt);
-                }
-                v4f32 acc0[NB], acc1[NB], acc2[NB], acc3[NB];
+                for (int T = 0; T < TB; T++) { a0[T] = codes_bf16(cu[T].x, cu[T].y); a1[T] = codes_bf16(cu[T].z, cu[T].w); }
+                request(ii % kBgDepth, i0 + ii + kBgDepth);   // the set is free: the tile four further on
+                if (active && ii < nbatch) {
+                    // two sums per column block: independent chains of MFMAs (one chain: 9 % slower, measured); each chain's
+                    // first MFMA takes a zero as the sum it adds to
+                    v4f32 acc0[NB], acc1[NB];
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) acc0[nb] = acc1[nb] = acc2[nb] = acc3[nb] = v4f32{0.f, 0.f, 0.f, 0.f};
+                    for (int T = 0; T < TB; T++) {
 #pragma unroll
-                for (int T = 0; T < 4; T++) {   // blocks of 64 k
-                    v8bf16 bx[NB][2][3];
+                        for (int nb = 0; nb < NB; nb++) {
+                            const v4f32 zero = {0.f, 0.f, 0.f, 0.f};
+                            acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[T], bx[nb][T][0][2], T == 0 ? zero : acc0[nb], 0, 0, 0);   // the small parts first
+                            acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[T], bx[nb][T][1][2], T == 0 ? zero : acc1[nb], 0, 0, 0);
 #pragma unroll
-                    for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-                        for (int h = 0; h < 2; h++)
-#pragma unroll
-                            for (int pl = 0; pl < 3; pl++) bx[nb][h][pl] = bxa[nb][h][pl];
-                    if (T + 1 < 4) fetch_x(xk, plane, pitch, T + 1, bxa);   // (the compiler renames the registers: the copy above costs nothing)
-                    const v8bf16 a00 = codes_bf16(u0[T].x, u0[T].y), a01 = codes_bf16(u0[T].z, u0[T].w);
-                    v8bf16 a10 = a00, a11 = a01;
-                    if (TILES == 2) { a10 = codes_bf16(u1[T].x, u1[T].y); a11 = codes_bf16(u1[T].z, u1[T].w); }
-#pragma unroll
-                    for (int nb = 0; nb < NB; nb++) {
-#pragma unroll
-                        for (int pl = 2; pl >= 0; pl--) {   // two sums per tile: independent chains of MFMAs; the small parts first
-                            acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a00, bx[nb][0][pl], acc0[nb], 0, 0, 0);
-                            acc2[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a01, bx[nb][1][pl], acc2[nb], 0, 0, 0);
-                            if (TILES == 2) {
-                                acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a10, bx[nb][0][pl], acc1[nb], 0, 0, 0);
-                                acc3[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a11, bx[nb][1][pl], acc3[nb], 0, 0, 0);
+                            for (int pl = 1; pl >= 0; pl--) {
+                                acc0[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[T], bx[nb][T][0][pl], acc0[nb], 0, 0, 0);
+                                acc1[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[T], bx[nb][T][1][pl], acc1[nb], 0, 0, 0);
                             }
                         }
                     }
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++) raw[((ii * WAVES + wave) * NB + nb) * 64 + lane] = acc0[nb] + acc1[nb];
                 }
-                const float2 sc0[4] = {make_float2(us0[0].x, us0[0].y), make_float2(us0[0].z, us0[0].w), make_float2(us0[1].x, us0[1].y),
-                                       make_float2(us0[1].z, us0[1].w)};
-                const float2 sc1[4] = {make_float2(us1[0].x, us1[0].y), make_float2(us1[0].z, us1[0].w), make_float2(us1[1].x, us1[1].y),
-                                       make_float2(us1[1].z, us1[1].w)};
+            }
+            __syncthreads();
+            if (wave < nbatch) {   // this lane: rows 4 s + (0..3) of sequence c (+ 16 per column block) of tile `wave` of the batch
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) {
-                    const float sxv = sxs[16 * nb + r][g - g0];   // this lane's column is sequence 16 nb + r
+                    v4f32 y = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        y0[nb][i] += fmaf(sc0[i].x, acc0[nb][i] + acc2[nb][i], sc0[i].y * sxv);
-                        if (TILES == 2) y1[nb][i] += fmaf(sc1[i].x, acc1[nb][i] + acc3[nb][i], sc1[i].y * sxv);
+                    for (int q = 0; q < kBgGroups; q++) {
+                        if (q < ng) {
+                            v4f32 t = raw[((wave * WAVES + q * HV) * NB + nb) * 64 + lane];
+                            float sx = sxw[(q * HV) * NSEQ + 16 * nb + c];
+                            if (HV == 2) {
+                                t += raw[((wave * WAVES + q * HV + 1) * NB + nb) * 64 + lane];
+                                sx += sxw[(q * HV + 1) * NSEQ + 16 * nb + c];
+                            }
+                            y[0] += fmaf(sc[q][0].x, t[0], sc[q][0].y * sx);
+                            y[1] += fmaf(sc[q][0].z, t[1], sc[q][0].w * sx);
+                            y[2] += fmaf(sc[q][1].x, t[2], sc[q][1].y * sx);
+                            y[3] += fmaf(sc[q][1].z, t[3], sc[q][1].w * sx);
+                        }
                     }
+                    float *o = mine.out + (long)(16 * nb + c) * mine.rows + 4 * s;
+                    if (COH) st_coh16(o, y);
+                    else *reinterpret_cast<v4f32 *>(o) = y;
                 }
             }
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                float *o = cur.out + (long)nb * 16 * cur.rows;
-                if (COH) {
-                    st_coh16(o, y0[nb]);
-                    if (cur.two) st_coh16(o + 16, y1[nb]);
-                } else {
-                    *reinterpret_cast<v4f32 *>(o) = y0[nb];
-                    if (cur.two) *reinterpret_cast<v4f32 *>(o + 16) = y1[nb];
-                }
-            }
-            cur = nxt;
+            __syncthreads();   // (the next batch writes the same LDS)
         }
     }
 };
 
-// grid (workgroups per slice, slices of K), 256 NB threads; dynamic LDS: bg_lds_bytes(gps, 16 NB)
-template <int TILES, int NB>
-__global__ void __launch_bounds__(kBgThreads * NB) k_bgemm(const BGemm a)
+// grid (workgroups per slice, slices of K), 256 HV threads; dynamic LDS: bg_lds_bytes(16 NB, HV)
+template <int NB, int HV>
+__global__ void __launch_bounds__(kBgThreads * HV) k_bgemm(const BGemm a)
 {
-    extern __shared__ __align__(16) unsigned short xh[];   // xh[(plane * NSEQ + b) * pitch + k]
-    __shared__ float sxs[kBatch * NB][kBgMaxGps];
-    BgWave<TILES, NB> w(a);
+    extern __shared__ __align__(16) float bg_lds[];
+    BgWave<NB, HV> w(a);
     w.begin(blockIdx.x, blockIdx.y, gridDim.x, false);
-    w.template run<false>(xh, sxs, false);
+    w.template run<false>(bg_lds, false);
 }
 
 // ---- the classifier: fp32 weights (K/MatMul.java:37-60), the same tiling -------------------------------------------

@@ -134,7 +134,7 @@ __device__ __forceinline__ void bstep_attention(const BStep &a, int l, float *ld
     const int pos = a.st->pos;
     const int items = a.n_heads * a.nseq, G = gridDim.x;
     const int rounds = (items + G * IPW - 1) / (G * IPW);
-    const int S = ((a.g[BS_QKV].K >> 8) + a.g[BS_QKV].gps - 1) / a.g[BS_QKV].gps;
+    const int S = bg_slices(a.g[BS_QKV].K);
     float *kc = a.kc + l * a.layer_stride * a.kv_dim, *vc = a.vc + l * a.layer_stride * a.kv_dim;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     float *mine = lds + it * (hs + 4);   // of this pair of waves: m, l, then the head's accumulators
@@ -258,7 +258,7 @@ __device__ __forceinline__ void bstep_residual(const BStep &a, const float *part
 __device__ __forceinline__ void bstep_swiglu(const BStep &a, const float *ss_lds)
 {
     const long n = (long)a.nseq * a.hidden, n4 = n >> 2;
-    const int S = ((a.g[BS_W13].K >> 8) + a.g[BS_W13].gps - 1) / a.g[BS_W13].gps;
+    const int S = bg_slices(a.g[BS_W13].K);
     const float *p1 = a.g[BS_W13].part[0], *p3 = a.g[BS_W13].part[1];
     for (long f = (long)blockIdx.x * blockDim.x + threadIdx.x; f < n4; f += (long)gridDim.x * blockDim.x) {
         const long i = 4 * f;
@@ -273,8 +273,6 @@ __device__ __forceinline__ void bstep_swiglu(const BStep &a, const float *ss_lds
     }
 }
 
-__device__ __forceinline__ int bstep_slices(const BGemm &g) { return ((g.K >> 8) + g.gps - 1) / g.gps; }
-
 // grid: as many workgroups of 256 NB threads as are resident at once (one per compute unit); dynamic LDS as k_bgemm.
 // Before: x = the embeddings, xn = their rmsnorm (normalized: the first attention multiplies by no ss), the barrier
 // counters zero.  After: x = the residual stream after the last layer (the final norm is the caller's).
@@ -283,28 +281,27 @@ __global__ void __launch_bounds__(kBgThreads * NB) k_bstep(const BStep *__restri
 {
     const BStep &a = *args;   // (in device memory: the kernel aims pointers at its parts, which an argument passed by value would be copied to scratch memory for)
     constexpr int NSEQ = kBatch * NB;
-    extern __shared__ __align__(16) unsigned short xh[];
-    __shared__ float sxs[NSEQ][kBgMaxGps];
+    extern __shared__ __align__(16) float lds[];   // the products' (bg_lds_bytes); the attention's hand-over between two waves
     __shared__ float ss_lds[NSEQ];
     const int wg = blockIdx.x, nch = a.dim >> 8;
     unsigned nbar = 0;
-    BgWave<1, NB> w(a.g[BS_QKV]);   // aimed at the four products of the argument in turn (the argument is never copied)
-    int S = bstep_slices(a.g[BS_QKV]);
+    BgWave<NB, NB> w(a.g[BS_QKV]);   // aimed at the four products of the argument in turn (the argument is never copied)
+    int S = bg_slices(a.g[BS_QKV].K);
     bool in = wg < a.gx[BS_QKV] * S;
     if (in) w.begin(wg / S, wg % S, a.gx[BS_QKV], true);
     for (int l = 0; l < a.n_layers; l++) {
 #pragma unroll 1
         for (int k = 0; k < 4; k++) {
-            if (in) w.template run<true>(xh, sxs, true);
+            if (in) w.template run<true>(lds, true);
             wait_own_stores();
             step_barrier(a.bar, nbar++);
             const bool last = l + 1 == a.n_layers;
             switch (k) {
             case BS_QKV:
                 if (l > 0) bstep_scalars(a.ssq + a.nseq * nch, nch, a.dim, ss_lds);
-                if (a.head_size == 64) bstep_attention<16, NB>(a, l, reinterpret_cast<float *>(xh), l > 0 ? ss_lds : nullptr);
-                else if (a.head_size == 128) bstep_attention<32, NB>(a, l, reinterpret_cast<float *>(xh), l > 0 ? ss_lds : nullptr);
-                else bstep_attention<64, NB>(a, l, reinterpret_cast<float *>(xh), l > 0 ? ss_lds : nullptr);
+                if (a.head_size == 64) bstep_attention<16, NB>(a, l, lds, l > 0 ? ss_lds : nullptr);
+                else if (a.head_size == 128) bstep_attention<32, NB>(a, l, lds, l > 0 ? ss_lds : nullptr);
+                else bstep_attention<64, NB>(a, l, lds, l > 0 ? ss_lds : nullptr);
                 break;
             case BS_WO:
                 bstep_residual<NB>(a, a.g[BS_WO].part[0], S, a.rmsw + (long)(a.n_layers + l) * a.dim, a.ssq, false);
@@ -322,7 +319,7 @@ __global__ void __launch_bounds__(kBgThreads * NB) k_bstep(const BStep *__restri
             wait_own_stores();
             w.ap = &a.g[nk];
             w.layer = l + (k == BS_W2 ? 1 : 0);
-            S = bstep_slices(a.g[nk]);
+            S = bg_slices(a.g[nk].K);
             in = wg < a.gx[nk] * S;
             if (in) w.begin(wg / S, wg % S, a.gx[nk], true);   // the first codes travel while the others arrive
             step_barrier(a.bar, nbar++);

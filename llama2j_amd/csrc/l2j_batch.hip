@@ -59,10 +59,9 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (!matrix_shape(c->cfg, tensor, &rows, &K)) return fail(L2J_E_ARG, "not a matrix tensor");
         if (layer < 0 || layer >= c->cfg.n_layers) return fail(L2J_E_ARG, "layer out of range");
         if (K % 256 || rows % 16) return fail(L2J_E_SIZE, "the batched matrix product needs rows of whole groups (K % 256 == 0) and rows % 16 == 0");
-        const int ngroups = K / 256, gps = std::max(1, std::min(std::min(ngroups, kBgMaxGps), (int)groups_per_slice));
-        const int slices = (ngroups + gps - 1) / gps;
-        const size_t lds = bg_lds_bytes(gps, kBatch);
-        if (lds + sizeof(float) * kBatch * kBgMaxGps > 160 * 1024) return fail(L2J_E_SIZE, "groups_per_slice: the slice of the activations does not fit the LDS");
+        (void)groups_per_slice;   // (a slice of K is four groups since the activations stay in the waves' registers)
+        const int slices = bg_slices(K);
+        const size_t lds = bg_lds_bytes(kBatch, 2);
         HIPCHK(hipSetDevice(c->cfg.device));
         {
             std::lock_guard<std::mutex> lock(c->upload_mu);
@@ -81,17 +80,17 @@ int l2j_batch_matmul(l2j_ctx *c, int tensor, int layer, const float *x, float *y
         if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&dy), (size_t)kBatch * rows * sizeof(float));
         if (e == hipSuccess) e = hipEventCreate(&e0);
         if (e == hipSuccess) e = hipEventCreate(&e1);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess) e = hipMemcpyAsync(dx, x, (size_t)kBatch * K * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             BGemm a{};
             a.m[0] = bqmat(c, tensor, (uint64_t)layer * rows * K);
-            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx; a.gps = gps;
-            const dim3 grid((bg_units(rows, 2) + 3) / 4, slices);
+            a.rows[0] = rows; a.part[0] = dpart; a.nmat = 1; a.K = K; a.x = dx;
+            const dim3 grid(std::min(rows / 16, std::max(1, c->n_cu / slices)), slices);
             const int n = std::max(1, (int)rounds);
-            hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);   // warm
+            hipLaunchKernelGGL((k_bgemm<1, 2>), grid, dim3(2 * kBgThreads), lds, c->stream, a);   // warm
             (void)hipEventRecord(e0, c->stream);
-            for (int i = 0; i < n; i++) hipLaunchKernelGGL((k_bgemm<2, 1>), grid, dim3(kBgThreads), lds, c->stream, a);
+            for (int i = 0; i < n; i++) hipLaunchKernelGGL((k_bgemm<1, 2>), grid, dim3(2 * kBgThreads), lds, c->stream, a);
             (void)hipEventRecord(e1, c->stream);
             hipLaunchKernelGGL(k_breduce, dim3(256), dim3(256), 0, c->stream, dpart, dy, rows, slices);
             e = hipGetLastError();
@@ -168,13 +167,15 @@ void l2j::invalidate_batch_tiles(l2j_ctx *c, int tensor)
 
 namespace {
 
-constexpr int kBatchGps = 2;   // groups of 256 codes per slice of K (measured: 1, 2, 4 -> 26, 24, 30 us for W1 of the 7B shape)
+constexpr int kClsGps = 2;   // k_bgemm_f32: groups of 256 floats per slice of K
 
-int batch_slices(int K) { return (K / 256 + kBatchGps - 1) / kBatchGps; }
-size_t batch_lds(int nseq) { return bg_lds_bytes(kBatchGps, nseq); }   // k_bgemm: bf16 planes
-size_t batch_lds_f32(int nseq) { return (size_t)nseq * (kBatchGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
-// workgroups of k_bgemm a compute unit holds at once: its 160 KB of LDS, and at most three by their registers
-int batch_resident(int nseq) { return std::max(1, std::min(3, (int)((160 * 1024) / (batch_lds(nseq) + sizeof(float) * nseq * kBgMaxGps)))); }
+int batch_slices(int K) { return bg_slices(K); }
+int cls_slices(int K) { return (K / 256 + kClsGps - 1) / kClsGps; }
+size_t batch_lds(int nseq) { return bg_lds_bytes(nseq, 2); }                 // k_bgemm: two waves per group for 16 and for 32 sequences
+size_t step_lds(int nseq) { return bg_lds_bytes(nseq, nseq / kBatch); }       // k_bstep: 256 threads per 16 sequences
+size_t batch_lds_f32(int nseq) { return (size_t)nseq * (kClsGps * 256 + kXPad) * sizeof(float); }   // k_bgemm_f32: floats
+// workgroups of k_bgemm a compute unit holds at once (eight waves each: two per SIMD by their registers)
+int batch_resident(int) { return 1; }
 
 // The product of one layer's matrices `tensors` (the same input, the same row length) as one k_bgemm argument.
 BGemm bgemm_args(l2j_ctx *c, std::initializer_list<int> tensors, int layer, const float *x, float *const *part)
@@ -188,27 +189,18 @@ BGemm bgemm_args(l2j_ctx *c, std::initializer_list<int> tensors, int layer, cons
         a.rows[a.nmat] = rows; a.part[a.nmat] = part[a.nmat];
         a.nmat++;
     }
-    a.K = K; a.x = x; a.gps = kBatchGps;
+    a.K = K; a.x = x;
     return a;
 }
 
-// With at most gmax workgroups per slice of K (all of a launch resident at once) a wave takes one unit of 16 or 32 rows
-// after the other.  Whichever unit size gives a wave fewer rows in all is taken (32 on a tie: two tiles share the
-// activations they fetch from LDS; bit t - 1 of `tiles_allowed`: units of t tiles may be used).  Returns the workgroups per slice.
-int bgemm_shape(const BGemm &a, int waves, int gmax, int tiles_allowed, int *tiles)
+// The workgroups per slice of K: at most gmax (all of a launch resident at once); every workgroup takes every gx-th tile of
+// 16 rows, in batches of as many tiles as it has waves, so no more workgroups than the number of rounds needs.
+int bgemm_shape(const BGemm &a, int gmax)
 {
-    int gx = 1, best = 1 << 30;
-    for (int t = 2; t >= 1; t--) {
-        if (!(tiles_allowed & (1 << (t - 1)))) continue;
-        int units = 0;
-        for (int i = 0; i < a.nmat; i++) units += bg_units(a.rows[i], t);
-        const int g = std::min(gmax, (units + waves - 1) / waves), iters = (units + waves * g - 1) / (waves * g);
-        if (iters * t < best) {
-            best = iters * t; *tiles = t;
-            gx = (units + waves * iters - 1) / (waves * iters);   // no more workgroups than that many rounds need
-        }
-    }
-    return gx;
+    int tiles = 0;
+    for (int i = 0; i < a.nmat; i++) tiles += a.rows[i] / 16;
+    const int g = std::max(1, std::min(gmax, tiles)), iters = (tiles + g - 1) / g;
+    return (tiles + iters - 1) / iters;
 }
 
 // The products of one layer's matrices in one launch.
@@ -217,17 +209,9 @@ void launch_bgemm(l2j_ctx *c, std::initializer_list<int> tensors, int layer, con
     const BGemm a = bgemm_args(c, tensors, layer, x, part);
     const int nb = nseq / kBatch;
     const int S = batch_slices(a.K), gmax = std::max(1, batch_resident(nseq) * c->n_cu / S);
-    int tiles = 2;
-    const int gx = bgemm_shape(a, 4 * nb, gmax, 1, &tiles);
-    const dim3 grid(gx, S), block(kBgThreads * nb);
-    const size_t lds = batch_lds(nseq);
-    if (nb == 1) {
-        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 1>), grid, block, lds, c->stream, a);
-        else hipLaunchKernelGGL((k_bgemm<2, 1>), grid, block, lds, c->stream, a);
-    } else {
-        if (tiles == 1) hipLaunchKernelGGL((k_bgemm<1, 2>), grid, block, lds, c->stream, a);
-        else hipLaunchKernelGGL((k_bgemm<2, 2>), grid, block, lds, c->stream, a);
-    }
+    const dim3 grid(bgemm_shape(a, gmax), S), block(kBgThreads * 2);
+    if (nb == 1) hipLaunchKernelGGL((k_bgemm<1, 2>), grid, block, batch_lds(nseq), c->stream, a);
+    else hipLaunchKernelGGL((k_bgemm<2, 2>), grid, block, batch_lds(nseq), c->stream, a);
 }
 
 // The grid of k_bstep: one workgroup per compute unit, all resident (by the runtime's count for the kernel and its LDS);
@@ -237,10 +221,10 @@ hipError_t plan_bstep(l2j_ctx *c, BatchBufs &b, int nseq)
     b.step_grid = 0;
     if (!c->opt[OPT_BATCH_FUSE]) return hipSuccess;
     const void *kernel = nseq == kBatch ? (const void *)k_bstep<1> : (const void *)k_bstep<2>;
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(nseq));
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)step_lds(nseq));
     if (e != hipSuccess) return e;
     int per_cu = 0;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBgThreads * (nseq / kBatch), batch_lds(nseq));
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kBgThreads * (nseq / kBatch), step_lds(nseq));
     if (e != hipSuccess) return e;
     if (per_cu < 1 || c->n_cu < batch_slices(c->cfg.hidden_dim) || c->n_cu < batch_slices(c->cfg.dim)) return hipSuccess;
     b.step_grid = c->n_cu;
@@ -251,16 +235,12 @@ hipError_t plan_bstep(l2j_ctx *c, BatchBufs &b, int nseq)
 BStep bstep_args(l2j_ctx *c, BatchBufs &b, int max_pos, int nseq)
 {
     const l2j_config &cf = c->cfg;
-    const int nb = nseq / kBatch;
     BStep a{};
     a.g[BS_QKV] = bgemm_args(c, {L2J_WQ, L2J_WK, L2J_WV}, 0, b.xn, b.part);
     a.g[BS_WO] = bgemm_args(c, {L2J_WO}, 0, b.xb, b.part);
     a.g[BS_W13] = bgemm_args(c, {L2J_W1, L2J_W3}, 0, b.xn, b.part);
     a.g[BS_W2] = bgemm_args(c, {L2J_W2}, 0, b.hb, b.part);
-    for (int k = 0; k < 4; k++) {
-        int tiles = 1;
-        a.gx[k] = bgemm_shape(a.g[k], 4 * nb, std::max(1, b.step_grid / batch_slices(a.g[k].K)), 1, &tiles);
-    }
+    for (int k = 0; k < 4; k++) a.gx[k] = bgemm_shape(a.g[k], std::max(1, b.step_grid / batch_slices(a.g[k].K)));
     a.n_layers = cf.n_layers; a.nseq = nseq; a.dim = cf.dim; a.hidden = cf.hidden_dim; a.n_heads = cf.n_heads;
     a.kv_mul = cf.n_heads / cf.n_kv_heads; a.head_size = c->head_size; a.kv_dim = c->kv_dim;
     a.sqrt_hs = sqrtf((float)c->head_size);
@@ -276,8 +256,8 @@ void launch_bstep(l2j_ctx *c, BatchBufs &b, int nseq)
 {
     const dim3 grid(b.step_grid), block(kBgThreads * (nseq / kBatch));
     const BStep *args = b.step_args;
-    if (nseq == kBatch) hipLaunchKernelGGL(k_bstep<1>, grid, block, batch_lds(nseq), c->stream, args);
-    else hipLaunchKernelGGL(k_bstep<2>, grid, block, batch_lds(nseq), c->stream, args);
+    if (nseq == kBatch) hipLaunchKernelGGL(k_bstep<1>, grid, block, step_lds(nseq), c->stream, args);
+    else hipLaunchKernelGGL(k_bstep<2>, grid, block, step_lds(nseq), c->stream, args);
 }
 
 // One position of all sequences: embedding, the layers, the classifier, the next tokens.
@@ -319,13 +299,13 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
     }
     {
         BGemmF32 g{};
-        g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kBatchGps;
-        const dim3 cg((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, sd);
+        g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kClsGps;
+        const dim3 cg((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, cls_slices(dim));
         if (nseq == kBatch) hipLaunchKernelGGL(k_bgemm_f32<1>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
         else hipLaunchKernelGGL(k_bgemm_f32<2>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
     }
     BNext n{};
-    n.part = b.part[0]; n.slices = sd; n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
+    n.part = b.part[0]; n.slices = cls_slices(dim); n.vocab = cf.vocab_size; n.logits = b.logits; n.st = b.st; n.prompts = b.prompts;
     n.prompt_stride = prompt_stride; n.out_tokens = b.out; n.out_stride = max_pos;
     { hipLaunchKernelGGL(k_bnext, dim3(nseq), dim3(1024), 0, s, n, b.done); }
 }
@@ -351,7 +331,7 @@ int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
     const l2j_config &cf = c->cfg;
     const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, kvd = c->kv_dim, vocab = cf.vocab_size;
     const int sd = batch_slices(dim), sh = batch_slices(hidden);
-    const size_t part_floats = (size_t)nseq * std::max({(size_t)sd * std::max(hidden, vocab), (size_t)sh * dim});
+    const size_t part_floats = (size_t)nseq * std::max({(size_t)sd * hidden, (size_t)cls_slices(dim) * vocab, (size_t)sh * dim, (size_t)sd * dim});
     const size_t cache_floats = (size_t)nseq * L * steps * kvd;
     BatchBufs *b = new (std::nothrow) BatchBufs();
     if (!b) return fail(L2J_E_OOM, "batched decode: host allocation failed");
@@ -378,9 +358,8 @@ int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
     if (e == hipSuccess) e = hipEventCreate(&b->e1);
     const size_t state_ints = sizeof(BatchState) / sizeof(int), prompt_ints = (size_t)nseq * pstride, out_ints = (size_t)nseq * steps;
     if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void **>(&b->h_pin), std::max(state_ints + prompt_ints, out_ints) * sizeof(int), hipHostMallocDefault);
-    const void *gemms[] = {(const void *)k_bgemm<1, 1>, (const void *)k_bgemm<2, 1>, (const void *)k_bgemm<1, 2>, (const void *)k_bgemm<2, 2>};
-    for (int i = 0; i < 4 && e == hipSuccess; i++)
-        e = hipFuncSetAttribute(gemms[i], hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(i < 2 ? kBatch : kMaxBatch));
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<1, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kBatch));
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds(kMaxBatch));
     if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm_f32<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kBatch));
     if (e == hipSuccess) e = hipFuncSetAttribute((const void *)k_bgemm_f32<2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)batch_lds_f32(kMaxBatch));
     // one position as a graph: every kernel reads the position and the tokens from device memory, so the same nodes serve

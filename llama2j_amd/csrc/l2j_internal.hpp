@@ -83,7 +83,7 @@ inline const OptionDef kOptions[OPT_COUNT] = {
     {"graph_tokens", 32, false},       // tokens per replay of the decode loops' graph (1: only the one-token graph)
     {"fast_steps", 1, false},          // k_token folds rows of dim codes without clamping when they are exactly one step
     {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
-    {"batch_fuse", 1, true},           // batched decode: the layers of a step in one launch with grid barriers (0: eight launches per layer)
+    {"batch_fuse", 0, true},           // batched decode: 1: the layers of a step in one launch with grid barriers (slower, measured); 0: eight launches per layer
 };
 
 inline int option_from_env(int i)
