@@ -554,8 +554,9 @@ struct BAttn {
     const float *pq, *pk, *pv;   // partial products of Wq, Wk, Wv: (slices, sequences, dim | kv_dim)
     int slices;
     const float2 *rope;          // (seq_len, head_size / 2) cos, sin
-    float *kc, *vc;              // this layer's rows of the batch cache: + (b * seq_stride + pos) * kv_dim
-    long seq_stride;             // cache rows between two sequences
+    float *kc, *vc;              // this layer's part of the batch cache, head-major: + b * seq_stride + (kv head * cap + pos) * head_size
+    long seq_stride;             // floats between two sequences
+    int cap;                     // positions the cache holds
     float *out;                  // (sequences, dim)
     const BatchState *st;
     int n_heads, kv_mul, head_size, kv_dim, dim;
@@ -598,7 +599,7 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
             sm_qkv[which][2 * idx] = v0;
             sm_qkv[which][2 * idx + 1] = v1;
             if (which > 0 && h % a.kv_mul == 0)
-                *reinterpret_cast<float2 *>((which == 1 ? a.kc : a.vc) + ((long)b * a.seq_stride + pos) * a.kv_dim + kvh * hs + 2 * idx) =
+                *reinterpret_cast<float2 *>((which == 1 ? a.kc : a.vc) + (long)b * a.seq_stride + ((long)kvh * a.cap + pos) * hs + 2 * idx) =
                     make_float2(v0, v1);
         }
     }
@@ -608,17 +609,17 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
     const float4 q4 = on ? *reinterpret_cast<const float4 *>(&sm_qkv[0][4 * j]) : zero;
     const float4 kp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[1][4 * j]) : zero;   // the row of this position
     const float4 vp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[2][4 * j]) : zero;
-    const long base = (long)b * a.seq_stride * a.kv_dim + kvh * hs + 4 * j;
+    const long base = (long)b * a.seq_stride + (long)kvh * a.cap * hs + 4 * j;   // the head's rows lie one after the other
     float m = -3.0e38f, l = 0.0f;
     float4 acc = zero;
     for (int t0 = slot; t0 < len; t0 += 2 * NSLOT) {   // two rows in flight per slot
         const int t1 = t0 + NSLOT;
         const bool ok1 = t1 < len;
         const bool c0 = on && t0 < pos, c1 = on && t1 < pos;   // rows of earlier positions come from the cache
-        float4 k0 = c0 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t0 * a.kv_dim) : zero;
-        float4 v0 = c0 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t0 * a.kv_dim) : zero;
-        float4 k1 = c1 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t1 * a.kv_dim) : zero;
-        float4 v1 = c1 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t1 * a.kv_dim) : zero;
+        float4 k0 = c0 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t0 * hs) : zero;
+        float4 v0 = c0 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t0 * hs) : zero;
+        float4 k1 = c1 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t1 * hs) : zero;
+        float4 v1 = c1 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t1 * hs) : zero;
         if (t0 == pos) { k0 = kp; v0 = vp; }
         if (t1 == pos) { k1 = kp; v1 = vp; }
         float s0 = (q4.x * k0.x + q4.y * k0.y) + (q4.z * k0.z + q4.w * k0.w);

@@ -20,8 +20,9 @@ struct BStep {
     int n_layers, nseq, dim, hidden, n_heads, kv_mul, head_size, kv_dim;
     float sqrt_hs;
     const float2 *rope;       // (seq_len, head_size / 2) cos, sin
-    float *kc, *vc;           // the batch cache: row ((b * seq_stride) + l * layer_stride + pos) * kv_dim
-    long seq_stride, layer_stride;
+    float *kc, *vc;           // the batch cache, head-major: b * seq_stride + l * layer_stride + (kv head * cap + pos) * head_size
+    long seq_stride, layer_stride;   // floats
+    int cap;
     const BatchState *st;
     float *x;                 // residual stream (nseq, dim): always read and written by the same wave
     float *xn, *xb, *hb;      // inputs of the products: g * x (nseq, dim), attention output (nseq, dim), SwiGLU output (nseq, hidden)
@@ -135,7 +136,7 @@ __device__ __forceinline__ void bstep_attention(const BStep &a, int l, float *ld
     const int items = a.n_heads * a.nseq, G = gridDim.x;
     const int rounds = (items + G * IPW - 1) / (G * IPW);
     const int S = bg_slices(a.g[BS_QKV].K);
-    float *kc = a.kc + l * a.layer_stride * a.kv_dim, *vc = a.vc + l * a.layer_stride * a.kv_dim;
+    float *kc = a.kc + l * a.layer_stride, *vc = a.vc + l * a.layer_stride;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     float *mine = lds + it * (hs + 4);   // of this pair of waves: m, l, then the head's accumulators
     for (int rd = 0; rd < rounds; rd++) {
@@ -160,10 +161,10 @@ __device__ __forceinline__ void bstep_attention(const BStep &a, int l, float *ld
             const float4 cs = *reinterpret_cast<const float4 *>(a.rope + (long)pos * half + 2 * j);   // (cos, sin) of pairs 2 j and 2 j + 1
             rope_pair(q4.x, q4.y, cs.x, cs.y); rope_pair(q4.z, q4.w, cs.z, cs.w);
             rope_pair(k4.x, k4.y, cs.x, cs.y); rope_pair(k4.z, k4.w, cs.z, cs.w);
-            const long base = (long)b * a.seq_stride * a.kv_dim + kvh * hs + 4 * j;
+            const long base = (long)b * a.seq_stride + (long)kvh * a.cap * hs + 4 * j;
             if (slot == 0 && h % a.kv_mul == 0) {   // J/Run.java:95-99
-                *reinterpret_cast<float4 *>(kc + base + (long)pos * a.kv_dim) = k4;
-                *reinterpret_cast<float4 *>(vc + base + (long)pos * a.kv_dim) = v4;
+                *reinterpret_cast<float4 *>(kc + base + (long)pos * hs) = k4;
+                *reinterpret_cast<float4 *>(vc + base + (long)pos * hs) = v4;
             }
             for (int t0 = 0; t0 < pos; t0 += NSL * U) {
                 float4 kk[U], vv[U];
@@ -172,8 +173,8 @@ __device__ __forceinline__ void bstep_attention(const BStep &a, int l, float *ld
                 for (int u = 0; u < U; u++) {
                     const int t = t0 + u * NSL + slot;
                     ok[u] = t < pos;
-                    kk[u] = ok[u] ? *reinterpret_cast<const float4 *>(kc + base + (long)t * a.kv_dim) : zero;
-                    vv[u] = ok[u] ? *reinterpret_cast<const float4 *>(vc + base + (long)t * a.kv_dim) : zero;
+                    kk[u] = ok[u] ? *reinterpret_cast<const float4 *>(kc + base + (long)t * hs) : zero;
+                    vv[u] = ok[u] ? *reinterpret_cast<const float4 *>(vc + base + (long)t * hs) : zero;
                 }
                 float s[U];
 #pragma unroll

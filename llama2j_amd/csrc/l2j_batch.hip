@@ -117,7 +117,7 @@ struct l2j::BatchBufs {
     int nseq = 0, cap_steps = 0, cap_pstride = 0;   // what the buffers and the graph's kernel arguments are made for
     float *x = nullptr, *xn = nullptr, *xb = nullptr, *hb = nullptr, *logits = nullptr;
     float *part[3] = {nullptr, nullptr, nullptr};
-    float *kc = nullptr, *vc = nullptr;             // (sequence, layer, cap_steps, kv_dim)
+    float *kc = nullptr, *vc = nullptr;             // (sequence, layer, kv head, cap_steps, head_size)
     BatchState *st = nullptr;
     int *prompts = nullptr, *out = nullptr;         // (sequence, cap_pstride), (sequence, cap_steps)
     unsigned *done = nullptr;
@@ -244,7 +244,7 @@ BStep bstep_args(l2j_ctx *c, BatchBufs &b, int max_pos, int nseq)
     a.n_layers = cf.n_layers; a.nseq = nseq; a.dim = cf.dim; a.hidden = cf.hidden_dim; a.n_heads = cf.n_heads;
     a.kv_mul = cf.n_heads / cf.n_kv_heads; a.head_size = c->head_size; a.kv_dim = c->kv_dim;
     a.sqrt_hs = sqrtf((float)c->head_size);
-    a.rope = c->rope; a.kc = b.kc; a.vc = b.vc; a.seq_stride = (long)cf.n_layers * max_pos; a.layer_stride = max_pos; a.st = b.st;
+    a.rope = c->rope; a.kc = b.kc; a.vc = b.vc; a.seq_stride = (long)cf.n_layers * max_pos * c->kv_dim; a.layer_stride = (long)max_pos * c->kv_dim; a.cap = max_pos; a.st = b.st;
     a.x = b.x; a.xn = b.xn; a.xb = b.xb; a.hb = b.hb; a.rmsw = c->rmsw; a.ssq = b.ssq;
     a.silu = c->silu; a.exact = (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0;
     a.bar.ctr = b.bar_ctr; a.bar.fault = b.fault; a.bar.ngroups = kBarGroups; a.bar.maxspin = c->opt[OPT_BARRIER_SPINS];
@@ -278,7 +278,7 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
         BAttn t{};
         t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
         t.kc = b.kc + (size_t)l * max_pos * kvd; t.vc = b.vc + (size_t)l * max_pos * kvd;
-        t.seq_stride = (long)L * max_pos; t.out = b.xb; t.st = b.st;
+        t.seq_stride = (long)L * max_pos * kvd; t.cap = max_pos; t.out = b.xb; t.st = b.st;
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
         const dim3 ag(cf.n_heads, nseq);
