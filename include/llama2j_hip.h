@@ -252,10 +252,10 @@ int l2j_decode_greedy_batch_logits(l2j_ctx *ctx, const int32_t *prompts, const i
  * processing of multiple queries" is on its wish-list, README.md:347): y[b][r] = sum_k dequant(W[r][k]) * x[b][k] for
  * sixteen activation vectors x (16 x K floats) against one layer's matrix of a quantized matrix tensor (L2J_WQ..L2J_W3;
  * K a multiple of 256), in the arithmetic of K/MatMul.java:117-151 (exact products, fp32 sums, group scale and offset;
- * see l2j_decode_greedy_batch).  y: 16 x rows floats.  groups_per_slice: groups of 256 codes per slice of K (a workgroup
- * stages that slice of the activations in LDS as three bf16 planes, 24 KB per group: at most 6).  The call makes the
- * tile-ordered copy of the tensor if the context has none yet.  *mean_us (may be NULL): mean time of `rounds` launches
- * of the product kernel. */
+ * see l2j_decode_greedy_batch).  y: 16 x rows floats.  groups_per_slice is ignored (a slice of K is four groups of 256
+ * codes since the kernel keeps the activations in its waves' registers; the argument remains for callers built against
+ * the earlier kernel).  The call makes the tile-ordered copy of the tensor if the context has none yet.  *mean_us (may be
+ * NULL): mean time of `rounds` launches of the product kernel. */
 int l2j_batch_matmul(l2j_ctx *ctx, int tensor, int layer, const float *x, float *y, int32_t groups_per_slice,
                      int32_t rounds, double *mean_us);
 /* Measurement: launches one kernel class `rounds` times at position `pos`, back to back on the context's stream,
