@@ -91,7 +91,9 @@ int l2j_device_count(void);
  * "token_special", "graph" (0: launch kernel by kernel instead of replaying captured hipGraphs), "graph_tokens" (tokens per
  * replay in the decode loops).  At any time: "sampler_scan", "sampler_exp_wgs", "fallback" (1: when a bounded wait of the
  * whole-token kernel runs out, because something else holds compute units of the GPU, the context switches to one launch
- * per phase for good and repeats the call; 0: the call returns L2J_E_HIP).  l2j_get_option reads the value in force
+ * per phase for good and repeats the call; 0: the call returns L2J_E_HIP), "batch_fuse" (l2j_decode_greedy_batch: 1 runs the
+ * layers of a step in one resident kernel with grid barriers instead of eight launches per layer; the same results,
+ * slower as measured, 0 by default; a bounded wait of that kernel that runs out is L2J_E_HIP).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
