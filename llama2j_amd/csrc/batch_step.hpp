@@ -1,7 +1,7 @@
-// All layers of a batched step in one launch: the four products of a layer (k_bgemm's waves) and what lies between
-// them (attention, residual + rmsnorm, SwiGLU) as eight phases with a grid barrier after each, all workgroups resident.
-// A kernel of the batched chain costs 5-6 us before it streams (launch, staging, first codes); here the first codes of a
-// product are requested before the barrier that precedes it, and the phases between the products spread over all
+// All layers of a batched step in one launch (option batch_fuse; slower than the eight launches per layer it replaces,
+// measured, and off by default): the four products of a layer (k_bgemm's waves) and what lies between them (attention,
+// residual + rmsnorm, SwiGLU) as eight phases with a grid barrier after each, all workgroups resident.  The first codes
+// of a product are requested before the barrier that precedes it, and the phases between the products spread over all
 // workgroups: the rmsnorm scalar is deferred (sum_k w_k (g_k ss x_k) = ss sum_k w_k g_k x_k), so a norm is no pass of one
 // workgroup over a vector but a sum of squares per 256 floats, written beside g x, and a multiplication by ss where the
 // product's partial sums are added up.  What one phase hands to the next goes through write-through stores and
