@@ -180,7 +180,7 @@ struct BgWave {
     // may not have been issued the compiler can only wait for all loads, and the sets in flight would be waited for too.
     __device__ __forceinline__ void request(int slot, int i)
     {
-        const Tile t = locate(min(first + min(i, cnt - 1) * gx, ntiles - 1));
+        const Tile t = locate(max(min(first + min(i, cnt - 1) * gx, ntiles - 1), 0));
         const uint4 *p = reinterpret_cast<const uint4 *>(t.codes + ((long)(g0 + min(gq, ng - 1)) << 12)) + (h * TB) * 64 + lane;
 #pragma unroll
         for (int T = 0; T < TB; T++) cw[slot][T] = load_stream(p + 64 * T);
@@ -288,7 +288,7 @@ struct BgWave {
             const int nbatch = min(WAVES, cnt - i0);
             // the scales of the tile this wave will add up, requested ahead of the batch's codes
             float4 sc[kBgGroups][2];
-            const Tile mine = locate(min(first + min(i0 + wave, cnt - 1) * gx, ntiles - 1));   // (unconditionally, as the codes)
+            const Tile mine = locate(max(min(first + min(i0 + wave, cnt - 1) * gx, ntiles - 1), 0));   // (unconditionally, as the codes)
 #pragma unroll
             for (int q = 0; q < kBgGroups; q++) {
                 const float4 *gp = reinterpret_cast<const float4 *>(mine.gs + ((g0 + min(q, ng - 1)) << 4) + 4 * s);   // (rm, min) of rows 4 s + (0..3)
