@@ -56,7 +56,8 @@ __device__ __forceinline__ void st_coh16(float *p, v4f32 v)
 // share the input (Wq, Wk, Wv; W1, W3) go into one launch: their row blocks follow each other in grid.x.
 constexpr int kBgMaxMat = 3;
 constexpr int kBgGroups = 4;        // groups of 256 codes per slice of K: one per wave (16 sequences) or per pair of waves (32)
-constexpr int kBgDepth = 4;         // tiles whose codes a wave has in flight (divides the number of waves: a tile's register set is known at compile time)
+constexpr int kBgDepth = 2;         // tiles whose codes a wave has in flight (divides the number of waves: a tile's register set is known at
+                                    // compile time).  Measured, 32 / 16 sequences: 1: 3.95 / 3.05 ms per step, 2: 3.84 / 2.97, 4: 3.85 / 3.07
 struct BGemm {
     QMat m[kBgMaxMat];        // the tensor's copy in tile order (k_btile), m.off: the layer's matrix (a multiple of 4096)
     int rows[kBgMaxMat];      // rows % 16 == 0
@@ -301,7 +302,7 @@ struct BgWave {
                 v8bf16 a0[TB], a1[TB];
 #pragma unroll
                 for (int T = 0; T < TB; T++) { a0[T] = codes_bf16(cu[T].x, cu[T].y); a1[T] = codes_bf16(cu[T].z, cu[T].w); }
-                request(ii % kBgDepth, i0 + ii + kBgDepth);   // the set is free: the tile four further on
+                request(ii % kBgDepth, i0 + ii + kBgDepth);   // the set is free: the tile kBgDepth further on
                 if (active && ii < nbatch) {
                     // two sums per column block: independent chains of MFMAs (one chain: 9 % slower, measured); each chain's
                     // first MFMA takes a zero as the sum it adds to
