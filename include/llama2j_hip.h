@@ -93,7 +93,9 @@ int l2j_device_count(void);
  * whole-token kernel runs out, because something else holds compute units of the GPU, the context switches to one launch
  * per phase for good and repeats the call; 0: the call returns L2J_E_HIP), "batch_fuse" (l2j_decode_greedy_batch: 1 runs the
  * layers of a step in one resident kernel with grid barriers instead of eight launches per layer; the same results,
- * slower as measured, 0 by default; a bounded wait of that kernel that runs out is L2J_E_HIP).  l2j_get_option reads the value in force
+ * slower as measured, 0 by default; a bounded wait of that kernel that runs out is L2J_E_HIP), "sampler_wide" (1, the default: a
+ * sampling step of a vocabulary of at most 36864 is one launch of a workgroup per 256 probabilities with grid barriers; a
+ * bounded wait of it that runs out is L2J_E_HIP; 0: one launch per stage, as larger vocabularies always take).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
@@ -236,6 +238,12 @@ int l2j_fill_synthetic(l2j_ctx *ctx, uint64_t seed, float sigma);
  * loops form them one addition after the other (sum += x, K/ExpSumNormalize.java:31-33; cdf += probabilities[i],
  * J/Sampler.java:37-40, 100-117), computed by the routine the device sampler uses.  sums[i] = terms[0] + ... + terms[i]. */
 int l2j_running_sums(l2j_ctx *ctx, const float *terms, int32_t n, float *sums);
+/* Measurement and test: the same sums as the one-launch sampling step forms them (option "sampler_wide"; many workgroups,
+ * 256 terms each), asked the questions the sampler asks (J/Sampler.java:37-40, 100-117): *total = the sum of the
+ * n <= 36864 non-negative terms added in element order; for every limit, index[q] = the first i whose running sum
+ * exceeds limits[q] (-1: none does) and sum[q] = that running sum.  n_limits <= 4096. */
+int l2j_sum_probe(l2j_ctx *ctx, const float *terms, int32_t n, const float *limits, int32_t n_limits, int32_t *index, float *sum,
+                  float *total);
 /* l2j_running_sums for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
  * hipMalloc, code that runs while another thread captures a graph); it has no counterpart in the reference.  Same
  * results, but the terms and sums pass through a fixed 144 KB device array of the library (one per GPU, held until the

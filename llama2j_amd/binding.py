@@ -107,6 +107,7 @@ def _signatures():
         "l2j_sample": (C.c_int, [vp, fp, C.c_float, C.c_float, C.c_float, i32p]),
         "l2j_running_sums": (C.c_int, [vp, fp, C.c_int32, fp]),
         "l2j_running_sums_noalloc": (C.c_int, [vp, fp, C.c_int32, fp]),
+        "l2j_sum_probe": (C.c_int, [vp, fp, C.c_int32, fp, C.c_int32, i32p, fp, fp]),
         "l2j_decode_sample": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, C.c_float, C.c_float, C.c_int64, i32p, i32p,
                                         C.POINTER(C.c_double)]),
         "l2j_read": (C.c_int, [vp, C.c_int, C.c_int, C.c_uint64, fp, C.c_uint64]),
@@ -461,6 +462,19 @@ class Transformer:
         out = np.empty_like(terms)
         self._check(lib().l2j_running_sums(self._h, _fp(terms), terms.size, _fp(out)))
         return out
+
+    def sum_probe(self, terms, limits):
+        """The sequential float32 sum of the terms as the one-launch sampling step forms it: (index, sum, total) with
+        index[q] the first i whose running sum exceeds limits[q] (-1: none), sum[q] that running sum, total the sum of
+        all terms."""
+        terms = np.ascontiguousarray(terms, dtype=np.float32)
+        limits = np.ascontiguousarray(limits, dtype=np.float32)
+        idx = np.empty(max(limits.size, 1), dtype=np.int32)
+        at = np.empty(max(limits.size, 1), dtype=np.float32)
+        total = np.empty(1, dtype=np.float32)
+        self._check(lib().l2j_sum_probe(self._h, _fp(terms), terms.size, _fp(limits), limits.size,
+                                        idx.ctypes.data_as(C.POINTER(C.c_int32)), _fp(at), _fp(total)))
+        return idx[:limits.size], at[:limits.size], float(total[0])
 
     def decode_sample(self, prompt, steps, temperature, topp, rng_seed):
         """The token loop of Run.main with its sampler (J/Run.java:611-685)."""

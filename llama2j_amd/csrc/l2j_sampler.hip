@@ -1,6 +1,7 @@
 // libllama2j_hip.so: host side of the device sampler (J/Sampler.java, J/Run.java:643-665) and the running sums.
 #include "l2j_internal.hpp"
 #include "sampler_kernels.hpp"
+#include "sampler_wide.hpp"
 
 using namespace l2j;
 
@@ -54,6 +55,8 @@ void l2j::free_sampler(l2j_ctx *c)
     }
     (void)hipFree(c->sample_exp);
     c->sample_exp = nullptr;
+    (void)hipFree(c->wide_mem);
+    c->wide_mem = nullptr;
     if (c->h_ss) (void)hipHostFree(c->h_ss);
     c->h_ss = nullptr;
 }
@@ -66,17 +69,49 @@ size_t sampler_lds_bytes(int n)
     return n <= kSampleMaxVocab ? (size_t)(((n + kChainStep - 1) & ~(kChainStep - 1)) + kChainStep) * sizeof(float) : 0;
 }
 
+// k_sample_wide's device memory, carved out of one allocation (WideWs says what is what)
+constexpr size_t kWideSync = 0, kWideSsum = (sizeof(WideSync) + 63) / 64 * 64, kWideSeg = kWideSsum + 8 * kWideMaxSlices,
+                 kWideCmask = kWideSeg + 16 * kWideMaxSlices, kWideT = kWideCmask + 32 * kWideMaxSlices, kWideD = kWideT + 3 * 8 * kWideMaxSlices, kWideBytes = kWideD + 3 * 8 * 64 * kWideMaxSlices;
+
+WideWs wide_ws(l2j_ctx *c)
+{
+    unsigned char *m = c->wide_mem;
+    WideWs w{};
+    w.sync = reinterpret_cast<WideSync *>(m + kWideSync);
+    w.ssum = reinterpret_cast<double *>(m + kWideSsum);
+    w.seg = reinterpret_cast<unsigned long long *>(m + kWideSeg);
+    w.cmask = reinterpret_cast<unsigned long long *>(m + kWideCmask);
+    int *t = reinterpret_cast<int *>(m + kWideT);
+    w.t_x0 = t; w.t_x1 = t + 2 * kWideMaxSlices; w.t_m = t + 4 * kWideMaxSlices;
+    int *d = reinterpret_cast<int *>(m + kWideD);
+    w.d_x0 = d; w.d_x1 = d + 2 * 64 * kWideMaxSlices; w.d_m = d + 4 * 64 * kWideMaxSlices;
+    w.maxspin = std::max(0, c->opt[OPT_BARRIER_SPINS]);
+    return w;
+}
+
+size_t wide_lds_bytes(int n)
+{
+    const size_t keys = (size_t)((n + kSortRun - 1) / kSortRun * kSortRun) * sizeof(float);
+    return std::max(keys, sizeof(WideWalk));
+}
+
 int alloc_sampler(l2j_ctx *c)
 {
     const int n = c->cfg.vocab_size;
+    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
     int rc;
     for (int i = 0; i < 2; i++) {
         if ((rc = dev_alloc(&c->pi_prob[i], (uint64_t)n + 4))) return rc;   // (read in 16-byte words: stage_terms)
         if ((rc = dev_alloc(&c->pi_idx[i], (uint64_t)n))) return rc;
     }
-    if ((rc = dev_alloc(&c->sample_exp, (uint64_t)n + 4))) return rc;
+    if ((rc = dev_alloc(&c->sample_exp, (uint64_t)npad + 4))) return rc;   // (k_sample_wide stores whole slices of 256)
     HIPCHK(hipHostMalloc((void **)&c->h_ss, sizeof(SamplerState), hipHostMallocDefault));
-    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+    if (n <= kSampleMaxVocab) {
+        if ((rc = dev_alloc(&c->wide_mem, kWideBytes))) return rc;
+        HIPCHK(hipMemset(c->wide_mem, 0, kWideBytes));
+        HIPCHK(hipFuncSetAttribute((const void *)k_sample_wide, hipFuncAttributeMaxDynamicSharedMemorySize, (int)wide_lds_bytes(n)));
+        HIPCHK(hipFuncSetAttribute((const void *)k_sum_probe, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(WideWalk)));
+    }
     for (int i = 0; i < 2; i++) {
         if ((rc = dev_alloc(&c->sort_k[i], (uint64_t)npad))) return rc;
         if ((rc = dev_alloc(&c->sort_v[i], (uint64_t)npad))) return rc;
@@ -140,6 +175,22 @@ hipError_t l2j::launch_sampler(l2j_ctx *c, float temperature, float topp, float 
     a.out_tokens = c->out_tokens;
     a.scan = c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0;
     const bool in_lds = n <= kSampleMaxVocab;   // else the kernels work in device memory, where k_sample_exp leaves the exponentials
+    if (in_lds && c->opt[OPT_SAMPLER_WIDE] != 0 && a.scan) {
+        WideArgs wa{};
+        wa.logits = c->logits; wa.n = n;
+        wa.temperature = temperature; wa.topp = topp; wa.coin = coin;
+        wa.plain = a.plain;
+        wa.ss = c->ss;
+        wa.old_prob = c->pi_prob[cur]; wa.old_idx = c->pi_idx[cur];
+        wa.new_prob = c->pi_prob[other]; wa.new_idx = c->pi_idx[other];
+        wa.k0 = c->sort_k[0]; wa.v0 = c->sort_v[0]; wa.k1 = c->sort_k[1]; wa.v1 = c->sort_v[1];
+        wa.expbuf = c->sample_exp;
+        wa.st = a.st; wa.out_tokens = a.out_tokens;
+        wa.w = wide_ws(c);
+        hipLaunchKernelGGL(k_sample_wide, dim3((n + kWideSlice - 1) / kWideSlice), dim3(kWideSlice), wide_lds_bytes(n), c->stream, wa);
+        if (!a.plain) c->pi_cur = other;   // the array stays there until the next call
+        return hipGetLastError();
+    }
     const int exp_wgs = std::min(1024, std::max(in_lds ? 0 : 1, c->opt[OPT_SAMPLER_EXP_WGS]));   // 0: the exponentials in k_sample_probs' one workgroup
     a.expbuf = exp_wgs > 0 ? c->sample_exp : nullptr;
     if (a.expbuf) {
@@ -190,6 +241,10 @@ int l2j::check_sampler_status(l2j_ctx *c)
     if (!st) return L2J_OK;
     c->h_ss->nan = 0;
     HIPCHK(hipMemcpy(&c->ss->nan, &c->h_ss->nan, sizeof(int), hipMemcpyHostToDevice));
+    if (st & 4) {   // (the counters of the launch are not where the next one expects them)
+        if (c->wide_mem) HIPCHK(hipMemset(c->wide_mem, 0, sizeof(WideSync)));
+        return fail(L2J_E_HIP, "sampler: a workgroup waited too long for the others (k_sample_wide needs a compute unit per 256 probabilities)");
+    }
     if (st & 1) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
     return fail(L2J_E_ARG, "sampler: no probability reaches the top-p cutoff (ArrayIndexOutOfBoundsException at J/Sampler.java:119)");
 }
@@ -269,6 +324,44 @@ int l2j_running_sums(l2j_ctx *c, const float *terms, int32_t n, float *sums)
         (void)hipFree(d);
         if (e != hipSuccess) return fail(L2J_E_HIP, std::string("running sums: ") + hipGetErrorString(e));
         return L2J_OK;
+    }());
+}
+
+int l2j_sum_probe(l2j_ctx *c, const float *terms, int32_t n, const float *limits, int32_t n_limits, int32_t *index_out, float *sum_out,
+                  float *total_out)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c || !terms || !total_out || (n_limits > 0 && (!limits || !index_out || !sum_out))) return fail(L2J_E_ARG, "null argument");
+        if (n <= 0 || n > kSampleMaxVocab) return fail(L2J_E_SIZE, "l2j_sum_probe: 1 to 36864 terms");
+        if (n_limits < 0 || n_limits > 4096) return fail(L2J_E_SIZE, "l2j_sum_probe: 0 to 4096 limits");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        int rc;
+        if (!c->ss && (rc = seed_sampler(c, 0))) return rc;
+        if (!c->wide_mem) return fail(L2J_E_STATE, "l2j_sum_probe: the context's vocabulary does not fit the one-launch sampler");
+        const int slices = (n + kWideSlice - 1) / kWideSlice;
+        // terms padded to whole slices | limits | sums at the hits | the total | the hits
+        const size_t nt = (size_t)slices * kWideSlice, nl = (size_t)std::max(n_limits, 1);
+        float *d = nullptr;
+        HIPCHK(hipMalloc(reinterpret_cast<void **>(&d), (nt + 2 * nl + 1) * sizeof(float) + nl * sizeof(int)));
+        float *d_lim = d + nt, *d_sum = d_lim + nl, *d_total = d_sum + nl;
+        int *d_idx = reinterpret_cast<int *>(d_total + 1);
+        hipError_t e = hipMemsetAsync(d, 0, nt * sizeof(float), c->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(d, terms, (size_t)n * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        if (e == hipSuccess && n_limits > 0) e = hipMemcpyAsync(d_lim, limits, (size_t)n_limits * sizeof(float), hipMemcpyHostToDevice, c->stream);
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(k_sum_probe, dim3(slices), dim3(kWideSlice), sizeof(WideWalk), c->stream, d, n, d_lim, n_limits, d_idx, d_sum,
+                               d_total, c->ss, wide_ws(c));
+            e = hipGetLastError();
+        }
+        if (e == hipSuccess && n_limits > 0) e = hipMemcpyAsync(index_out, d_idx, (size_t)n_limits * sizeof(int), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess && n_limits > 0) e = hipMemcpyAsync(sum_out, d_sum, (size_t)n_limits * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(total_out, d_total, sizeof(float), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(c->h_ss, c->ss, sizeof(SamplerState), hipMemcpyDeviceToHost, c->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+        (void)hipFree(d);
+        if (e != hipSuccess) return fail(L2J_E_HIP, std::string("sum probe: ") + hipGetErrorString(e));
+        return check_sampler_status(c);
     }());
 }
 

@@ -694,23 +694,33 @@ __global__ void __launch_bounds__(1024) k_running_sums(float *x, int n, int scan
 // Pairs past n (the array is padded to whole runs) carry the key -1 and sort behind everything.
 constexpr int kSortTile = 256, kSortRun = 4096, kSortTilesPerRun = kSortRun / kSortTile;
 
+// o >= k is o > the float just below k: a search that counts ">= k" in stretches that stood earlier and "> k" in later
+// ones then makes one comparison per probe, against sort_below(k) or k (two comparisons and a choice between their
+// results kept the compiler from issuing the probes of a step together).
+__device__ __forceinline__ float sort_below(float k)
+{
+    return __uint_as_float(k > 0.0f ? __float_as_uint(k) - 1u : k == 0.0f ? 0x80000001u : __float_as_uint(k) + 1u);
+}
+
 // grid: padded n / 256 workgroups of 256 threads
 static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
                                                           float *__restrict__ kout, int *__restrict__ vout)
 {
-    __shared__ __align__(16) float keys[kSortTile];
+    // a pair stands before another when its probability is greater, or equal and its position lower: one unsigned
+    // comparison of (probability bits, 255 - position); the bits of a non-negative float ascend with it, the padding's -1
+    // counts as 0 (it stands behind every position of the array anyway)
+    __shared__ __align__(16) unsigned long long keys[kSortTile];
     const int tid = threadIdx.x, i = blockIdx.x * kSortTile + tid;
     const float k = i < n ? kin[i] : -1.0f;
     const int v = i < n ? vin[i] : 0;
-    keys[tid] = k;
+    const unsigned long long mine = ((unsigned long long)(k < 0.0f ? 0u : __float_as_uint(k)) << 32) | (unsigned)(kSortTile - 1 - tid);
+    keys[tid] = mine;
     __syncthreads();
     int rank = 0;
-#pragma unroll 8
-    for (int j4 = 0; j4 < kSortTile / 4; j4++) {
-        const float4 o = *reinterpret_cast<const float4 *>(&keys[4 * j4]);
-        const int j = 4 * j4;
-        rank += (o.x > k || (o.x == k && j < tid)) + (o.y > k || (o.y == k && j + 1 < tid)) + (o.z > k || (o.z == k && j + 2 < tid)) +
-                (o.w > k || (o.w == k && j + 3 < tid));
+#pragma unroll 16
+    for (int j2 = 0; j2 < kSortTile / 2; j2++) {
+        const ulonglong2 o = *reinterpret_cast<const ulonglong2 *>(&keys[2 * j2]);
+        rank += (o.x > mine) + (o.y > mine);
     }
     kout[blockIdx.x * kSortTile + rank] = k;
     vout[blockIdx.x * kSortTile + rank] = v;
@@ -732,6 +742,7 @@ static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restr
     const float k = keys[i];
     const int v = vin[base + i];
     const int ti = i / kSortTile;
+    const float kb = sort_below(k);
     int pos[kSortTilesPerRun];
 #pragma unroll
     for (int tj = 0; tj < kSortTilesPerRun; tj++) pos[tj] = 0;
@@ -740,14 +751,14 @@ static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restr
 #pragma unroll
         for (int tj = 0; tj < kSortTilesPerRun; tj++) {
             const float o = keys[tj * kSortTile + pos[tj] + st - 1];
-            pos[tj] += (tj < ti ? o >= k : o > k) ? st : 0;   // tiles that stood earlier win ties
+            pos[tj] += o > (tj < ti ? kb : k) ? st : 0;   // tiles that stood earlier win ties
         }
     }
     int rank = i - ti * kSortTile;
 #pragma unroll
     for (int tj = 0; tj < kSortTilesPerRun; tj++) {
         const float o = keys[tj * kSortTile + pos[tj]];
-        const int cnt = pos[tj] + ((tj < ti ? o >= k : o > k) ? 1 : 0);
+        const int cnt = pos[tj] + (o > (tj < ti ? kb : k) ? 1 : 0);
         rank += tj == ti ? 0 : cnt;
     }
     kout[base + rank] = k;
@@ -769,6 +780,7 @@ static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restri
     const float k = keys[i];
     const int v = vin[i];
     const int ri = i / kSortRun, nruns = npad / kSortRun;
+    const float kb = sort_below(k);
     int pos[kSortMaxRuns];
 #pragma unroll
     for (int rj = 0; rj < kSortMaxRuns; rj++) pos[rj] = 0;
@@ -778,7 +790,7 @@ static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restri
         for (int rj = 0; rj < kSortMaxRuns; rj++) {
             if (rj < nruns) {
                 const float o = keys[rj * kSortRun + pos[rj] + st - 1];
-                pos[rj] += (rj < ri ? o >= k : o > k) ? st : 0;
+                pos[rj] += o > (rj < ri ? kb : k) ? st : 0;
             }
         }
     }
@@ -787,7 +799,7 @@ static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restri
     for (int rj = 0; rj < kSortMaxRuns; rj++) {
         if (rj < nruns && rj != ri) {
             const float o = keys[rj * kSortRun + pos[rj]];
-            rank += pos[rj] + ((rj < ri ? o >= k : o > k) ? 1 : 0);
+            rank += pos[rj] + (o > (rj < ri ? kb : k) ? 1 : 0);
         }
     }
     if (rank < n) {
@@ -820,18 +832,19 @@ static __global__ void __launch_bounds__(256) k_merge_far(const float *__restric
         pos[u] = 0;
     }
     const float *run = kin + g0;
+    const float kb = sort_below(k);
     for (int st = run_len >> 1; st > 0; st >>= 1) {
 #pragma unroll
         for (int u = 0; u < kSortFanIn; u++) {
             const int at = pos[u] + st - 1;
             const float o = run[min(u * run_len + at, gend - g0 - 1)];
-            pos[u] += (at < len[u] && (u < ri ? o >= k : o > k)) ? st : 0;   // runs that stood earlier win ties
+            pos[u] += (at < len[u] && o > (u < ri ? kb : k)) ? st : 0;   // runs that stood earlier win ties
         }
     }
 #pragma unroll
     for (int u = 0; u < kSortFanIn; u++) {
         const float o = run[min(u * run_len + pos[u], gend - g0 - 1)];
-        const int cnt = pos[u] + ((pos[u] < len[u] && (u < ri ? o >= k : o > k)) ? 1 : 0);
+        const int cnt = pos[u] + ((pos[u] < len[u] && o > (u < ri ? kb : k)) ? 1 : 0);
         rank += u != ri ? cnt : 0;
     }
     if (rank < nout) {

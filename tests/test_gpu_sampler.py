@@ -33,8 +33,14 @@ def check_probabilities(got, want):
     assert np.abs(got - want).max() <= 2e-7 * want.max(), np.abs(got - want).max()
 
 
+# sampler_wide 1 (the default): the sampling step is one launch over many workgroups; 0: one launch per stage
+WIDE = pytest.mark.parametrize("wide", ["1", "0"])
+
+
+@WIDE
 @pytest.mark.parametrize("vocab", [1003, 32000])
-def test_plain_sampling_matches_oracle(orc, vocab):
+def test_plain_sampling_matches_oracle(orc, monkeypatch, vocab, wide):
+    monkeypatch.setenv("L2J_SAMPLER_WIDE", wide)
     g = small_transformer(vocab)
     rng = np.random.default_rng(vocab)
     g.sampler_seed(77)
@@ -50,8 +56,10 @@ def test_plain_sampling_matches_oracle(orc, vocab):
             assert g.sample(t, 1.0, logits=lg, coin=coin) == o.sample(got, coin=coin), (call, kind, coin)
 
 
+@WIDE
 @pytest.mark.parametrize("vocab", [1003, 32000])
-def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, vocab):
+def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, monkeypatch, vocab, wide):
+    monkeypatch.setenv("L2J_SAMPLER_WIDE", wide)
     g = small_transformer(vocab)
     rng = np.random.default_rng(vocab + 1)
     g.sampler_seed(-12345)
@@ -66,10 +74,12 @@ def test_topp_sequence_matches_oracle_including_entries_of_earlier_calls(orc, vo
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
-@pytest.mark.parametrize("vocab", [4097, 32000, 70001])
-def test_topp_with_many_equal_probabilities_keeps_the_stable_order(orc, vocab):
+@WIDE
+@pytest.mark.parametrize("vocab", [255, 4097, 32000, 70001])
+def test_topp_with_many_equal_probabilities_keeps_the_stable_order(orc, monkeypatch, vocab, wide):
     # logits on a coarse grid: thousands of equal probabilities, inside tiles, across tiles and across runs of the sort,
     # and among the entries that earlier calls left behind; Arrays.sort is stable, so their order is the array's
+    monkeypatch.setenv("L2J_SAMPLER_WIDE", wide)
     g = small_transformer(vocab)
     rng = np.random.default_rng(vocab + 7)
     g.sampler_seed(3)
@@ -146,6 +156,49 @@ def test_running_sums_are_the_sequential_float32_sums(orc, monkeypatch, scan):
             want = np.cumsum(terms, dtype=np.float32)
         got = g.running_sums(terms)
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (name, int(np.argmax(got != want)))
+
+
+def test_the_one_launch_step_forms_the_sequential_sums_and_finds_where_they_pass_a_limit(orc):
+    """l2j_sum_probe asks the walk of the one-launch sampling step what the sampler asks it: the sum of all terms, and the
+    first index whose running sum exceeds a limit with that sum; numpy's float32 cumsum is the reference's loop."""
+    g = small_transformer(64)
+    rng = np.random.default_rng(23)
+    for name, terms in running_sum_cases():
+        with np.errstate(over="ignore", invalid="ignore"):
+            terms = np.asarray(terms, dtype=np.float32)
+            if terms.size > 36864:
+                continue
+            c = np.cumsum(terms, dtype=np.float32)
+            at = np.unique(np.concatenate([[0, terms.size - 1], rng.integers(0, terms.size, 150),
+                                           np.flatnonzero(np.diff(np.frexp(c)[1]))[:40]]))   # (also where the sum changes binade)
+            limits = np.concatenate([[0.0], c[at], np.nextafter(c[at], np.float32(-np.inf)), c[-1:] * 2 + 1]).astype(np.float32)
+            limits = limits[np.isfinite(limits) & (limits >= 0)]
+            idx, s, total = g.sum_probe(terms, limits)
+            assert np.float32(total).view(np.uint32) == c[-1].view(np.uint32), (name, total, c[-1])
+            for q, lim in enumerate(limits):
+                over = np.flatnonzero(c > lim)
+                want = int(over[0]) if over.size else -1
+                assert idx[q] == want, (name, q, float(lim), int(idx[q]), want)
+                if want >= 0:
+                    assert s[q].view(np.uint32) == c[want].view(np.uint32), (name, q, float(lim), want)
+
+
+@pytest.mark.parametrize("topp", [1.0, 0.9, 0.5])
+def test_one_launch_and_launch_per_stage_pick_the_same_tokens(orc, monkeypatch, topp):
+    vocab = 32000
+    rng = np.random.default_rng(15)
+    calls = [(logits_of(rng, vocab, kind), float(np.float32(rng.random()))) for kind in ("flat", "peaked", "mid", "peaked", "flat", "mid")]
+    seen = []
+    for wide in ("1", "0"):
+        monkeypatch.setenv("L2J_SAMPLER_WIDE", wide)
+        g = small_transformer(vocab)
+        g.sampler_seed(4)
+        out = []
+        for lg, coin in calls:
+            out.append((g.sample(0.9, topp, logits=lg, coin=coin), g.sample(0.9, topp, logits=lg), g.read(BUFFER.LOGITS).view(np.uint32)))
+        seen.append(out)
+    for a, b in zip(*seen):
+        assert a[0] == b[0] and a[1] == b[1] and np.array_equal(a[2], b[2])
 
 
 @pytest.mark.parametrize("topp", [1.0, 0.9])
