@@ -5,16 +5,16 @@
 // that only grows during the launch; the last workgroup to leave clears it).  What one stage hands to the next is stored
 // write-through and read with device-coherent loads.
 //
-//   A  max, exp((double)(x / t - max)) of the slice, its double-precision sum
-//   B  the slice reduced for the sequential float sum (below)
+//   A  max, exp((double)(x / t - max)) of the slice, and the slice reduced for the sequential float sum (below; the guess
+//      it needs, the sum of what stands before the slice, from fast exponentials of the logits the maximum was taken of)
 //   C  every workgroup walks the slices (the same walk everywhere: nobody waits for a result), divides its slice by
 //      the sum, writes the probabilities over the logits and flags its top-p candidates (J/Sampler.java:85-96)
 //   D  the ProbIndex array of this call (candidates in index order, then what the last call left, which is sorted)
 //      taken tile by tile and every tile of 256 sorted by counting
 //   E  runs of 16 tiles merged by counting (binary searches in LDS), F all runs merged: Arrays.sort, stable, descending
-//   G  the sorted candidates reduced like B; then workgroup 0 walks them until the sum exceeds topp, draws
+//   G  the sorted candidates reduced like A's slices; then workgroup 0 walks them until the sum exceeds topp, draws
 //      (java.util.Random), and walks again until the sum exceeds r (J/Sampler.java:99-119)
-// sample (topp > 0.999) is A, B, C, a reduction of the probabilities and one walk until the sum exceeds the draw.
+// sample (topp > 0.999) is A, C, a reduction of the probabilities and one walk until the sum exceeds the draw.
 //
 // The sequential float sums.  spec_sums (sampler_kernels.hpp) explains the arithmetic: inside a binade of the running
 // sum a run of terms is a pair of integer increments (for an even / odd sum before it), pairs compose, and the binade a
@@ -61,7 +61,7 @@ struct WideSync {
 // Device memory of a launch besides the arrays of SampleArgs.  The reductions exist twice: a workgroup may write its
 // second one while others still walk the first.
 struct WideWs {
-    double *ssum;               // [slices] double-precision sum of a slice's terms (A)
+    double *ssum;               // [slices] double-precision sum of a slice's terms (k_sum_probe)
     int *t_x0, *t_x1, *t_m;     // [2][slices] a slice as one pair; t_m 0: not uniform
     unsigned long long *seg;    // [2][slices] lanes that start a segment
     int *d_x0, *d_x1, *d_m;     // [2][slices * 64] per lane: the pair of its segment up to and including it, its binade code
@@ -603,9 +603,12 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
     const int i = g * kWideSlice + tid;
     unsigned bar = 0;
 
-    // ---- A: x / t, max (FindMax: the rounded quotient of the largest logit is the largest rounded quotient), exp
+    // ---- A: x / t, max (FindMax: the rounded quotient of the largest logit is the largest rounded quotient), exp, and B:
+    // the slice reduced for the sum of the exponentials.  B's guess, the sum of what stands before the slice, needs no
+    // other workgroup: every thread has loaded its share of all logits for the maximum, and the fast exponential will do.
     float mxl = -__builtin_inff();
     const int n4 = n & ~3;
+    double before = 0.0;   // (the sum before this slice, approximately)
     {   // (every load in flight at once, past the end the last one again: the loop is bound by their latency)
         constexpr int kMax4 = kSampleMaxVocab / (4 * kWideSlice);
         float4 x[kMax4];
@@ -615,9 +618,17 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
 #pragma unroll
             for (int u = 0; u < kMax4; u++) mxl = fmaxf(fmaxf(fmaxf(mxl, x[u].x), fmaxf(x[u].y, x[u].z)), x[u].w);
         }
+        for (int q = n4 + tid; q < n; q += kWideSlice) mxl = fmaxf(mxl, a.logits[q]);
+        mxl = block_max(mxl, red);
+        const float it = 1.0f / a.temperature;
+        float part = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kMax4; u++)   // (whole float4s: a slice starts at a multiple of 256, below n rounded down to 4)
+            if (4 * (tid + u * kWideSlice) < g * kWideSlice)
+                part += __expf((x[u].x - mxl) * it) + __expf((x[u].y - mxl) * it) + __expf((x[u].z - mxl) * it) + __expf((x[u].w - mxl) * it);
+        const double ds = wide_wave_sum((double)part);
+        if (lane == 0) dred[wave] = ds;
     }
-    for (int q = n4 + tid; q < n; q += kWideSlice) mxl = fmaxf(mxl, a.logits[q]);
-    mxl = block_max(mxl, red);
     const float mx = __fdiv_rn(mxl, a.temperature);
     int bad = 0;
     float e = 0.0f;
@@ -628,30 +639,14 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
     }
     st_coh(a.expbuf + i, e);
     es[tid] = e;
-    {
-        const double ds = wide_wave_sum((double)e);
-        if (lane == 0) dred[wave] = ds;
-        __syncthreads();
-        if (tid == 0) {
-            __hip_atomic_store(a.w.ssum + g, dred[0] + dred[1] + dred[2] + dred[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
-    wide_barrier(a.w, bar++);
-
-    // ---- B: the slice reduced for the sum of the exponentials
-    double before = 0.0;   // (wave 0: the sum before this slice, approximately)
-    if (wave == 0) {
-        for (int h = lane; h < g; h += 64) before += __hip_atomic_load(a.w.ssum + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        before = wide_wave_sum(before);
-        wide_reduce(a.w, 0, g, *reinterpret_cast<const float4 *>(es + 4 * lane), before);
-    }
+    __syncthreads();
+    before = dred[0] + dred[1] + dred[2] + dred[3];
+    if (wave == 0) wide_reduce(a.w, 0, g, *reinterpret_cast<const float4 *>(es + 4 * lane), before);
     wide_barrier(a.w, bar++);
 
     // ---- C: sum += x in element order (ExpSumNormalize), x /= sum, the probabilities replace the logits
     wide_stage(a.w, 0, L, G, a.expbuf, G * kWideSlice);
-    if (wave == 0) wide_plan(L, G);
-    __syncthreads();
-    if (wave == 0) wide_run(a.w, 0, L, G, a.expbuf, G * kWideSlice, 0.0f, false);
+    if (wave == 0) wide_walk(a.w, 0, L, G, a.expbuf, G * kWideSlice, 0.0f, false);   // (once: writing the list of steps first does not pay)
     __syncthreads();
     const float sum = L.total;
     float p = e;
