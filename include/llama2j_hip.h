@@ -85,7 +85,7 @@ int l2j_device_count(void);
 /* Launch shapes and algorithm switches of one context, the counterpart of the constants the reference compiles into
  * its kernels' launch code (the block sizes in the K/ classes, J/Run.java:27-28).  A context starts from the process
  * defaults (environment variable L2J_<NAME>, read once by l2j_create; unset: the built-in value), this call overrides
- * one of them, and the library never reads the environment afterwards.  Before l2j_finalize: "threads", "grid",
+ * one of them, and the library never reads the environment afterwards.  Before l2j_finalize: "threads" (workgroup size of the weight-streaming kernels; -1, the default: by the longest row), "grid",
  * "attn_threads", "attn_rows", "attn_nsplit", "fused_attn_rows", "fused_attn_splits", "barrier_spins", "fuse" (1 whole-token
  * kernel, 0 one launch per phase, -1 by model size), "layers_per_launch", "by_value", "self_contained", "fast_steps",
  * "token_special", "graph" (0: launch kernel by kernel instead of replaying captured hipGraphs), "graph_tokens" (tokens per

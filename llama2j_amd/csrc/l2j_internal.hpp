@@ -64,7 +64,7 @@ struct OptionDef {
     bool after_finalize;  // may still be changed once the launch shapes are fixed
 };
 inline const OptionDef kOptions[OPT_COUNT] = {
-    {"threads", 1024, false},          // workgroup size of the weight-streaming kernels
+    {"threads", kAuto, false},         // workgroup size of the weight-streaming kernels (auto: 1024; 512 / 640 for rows of at most 4096 / 1024 weights, measured)
     {"grid", kAuto, false},            // their workgroups (auto: one per compute unit)
     {"attn_threads", 256, false},      // k_attention as a kernel of its own
     {"attn_rows", 32, false},

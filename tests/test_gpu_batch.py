@@ -34,6 +34,20 @@ def check_against_oracle(m, prompt, steps, tokens, logits, what):
     assert worst < LOGIT_TOL, (what, worst)
     return worst
 
+def same_until_a_tie(got, want, logits, what):
+    """The batched path and the single-sequence path add the same products in different orders (their logits agree to a
+    few 1e-6 of the largest), so a sequence may part ways where its two best logits lie that close together, and only
+    there: the same tokens up to the first difference, and at that step the two tokens' logits (the batched path's) within
+    1e-5 of the largest."""
+    diff = np.flatnonzero(got != want)
+    if diff.size == 0:
+        return
+    pos = int(diff[0])
+    lg = logits[pos]
+    gap = abs(float(lg[got[pos]]) - float(lg[want[pos]]))
+    assert gap <= 1e-5 * float(np.abs(lg).max()), (what, pos, int(got[pos]), int(want[pos]), gap)
+
+
 SHAPES = [
     (512, 1024, 4, 8, 8, 1008, 64, 1),      # head 64, shared classifier
     (512, 1024, 2, 8, 2, 1008, 64, 0),      # grouped-query attention: 8 heads on 2 kv heads
@@ -112,7 +126,7 @@ def test_every_sequence_gets_what_it_gets_alone(orc, shape, n_seq):
         p = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
         g.reset()
         want, _ = g.decode_greedy(p, steps)          # stops after token 1; the batch runs on
-        np.testing.assert_array_equal(got[b, :len(want)], want, err_msg="sequence %d" % b)
+        same_until_a_tie(got[b, :len(want)], want, logits[:, b], "sequence %d" % b)
         np.testing.assert_array_equal(got[b, :len(p)], p)
     # every sequence against the oracle as well: its tokens, and the logits of every step
     m = oracle_of(orc, shape, 9)
