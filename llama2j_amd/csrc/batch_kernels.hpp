@@ -569,6 +569,8 @@ struct BAttn {
 // summed in order, RoPE on the pairs of q and k (K/ApplyRope.java:74-90), k and v into the cache row (J/Run.java:95-99; by
 // the first head of the kv group).  Then LPR lanes per cache row (four floats of the head each): the row slots of the
 // workgroup take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, sequences).
+constexpr int kBattnRows = 4;
+
 template <int LPR>
 __global__ void __launch_bounds__(256) k_battn(const BAttn a)
 {
@@ -613,29 +615,50 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
     const long base = (long)b * a.seq_stride + (long)kvh * a.cap * hs + 4 * j;   // the head's rows lie one after the other
     float m = -3.0e38f, l = 0.0f;
     float4 acc = zero;
-    for (int t0 = slot; t0 < len; t0 += 2 * NSLOT) {   // two rows in flight per slot
-        const int t1 = t0 + NSLOT;
-        const bool ok1 = t1 < len;
-        const bool c0 = on && t0 < pos, c1 = on && t1 < pos;   // rows of earlier positions come from the cache
-        float4 k0 = c0 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t0 * hs) : zero;
-        float4 v0 = c0 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t0 * hs) : zero;
-        float4 k1 = c1 ? *reinterpret_cast<const float4 *>(a.kc + base + (long)t1 * hs) : zero;
-        float4 v1 = c1 ? *reinterpret_cast<const float4 *>(a.vc + base + (long)t1 * hs) : zero;
-        if (t0 == pos) { k0 = kp; v0 = vp; }
-        if (t1 == pos) { k1 = kp; v1 = vp; }
-        float s0 = (q4.x * k0.x + q4.y * k0.y) + (q4.z * k0.z + q4.w * k0.w);
-        float s1 = (q4.x * k1.x + q4.y * k1.y) + (q4.z * k1.z + q4.w * k1.w);
+    constexpr int R = kBattnRows;   // rows in flight per slot
+    const int last = max(pos - 1, 0);
+    for (int tb = slot; tb < len; tb += R * NSLOT) {
+        // (unconditional loads from the global address space: a row past the cache's last is that last row again and is
+        // left out below; a load chosen by a condition became a flat load from one of two addresses)
+        float4 kk[R], vv[R];
 #pragma unroll
-        for (int off = LPR / 2; off > 0; off >>= 1) { s0 += __shfl_xor(s0, off); s1 += __shfl_xor(s1, off); }
-        s0 = __fdiv_rn(s0, a.sqrt_hs);
-        s1 = ok1 ? __fdiv_rn(s1, a.sqrt_hs) : -3.0e38f;
-        const float mb = fmaxf(m, fmaxf(s0, s1));
-        const float sc = expf(m - mb), p0 = expf(s0 - mb), p1 = ok1 ? expf(s1 - mb) : 0.0f;
-        l = l * sc + p0 + p1;
-        acc.x = acc.x * sc + p0 * v0.x + p1 * v1.x;
-        acc.y = acc.y * sc + p0 * v0.y + p1 * v1.y;
-        acc.z = acc.z * sc + p0 * v0.z + p1 * v1.z;
-        acc.w = acc.w * sc + p0 * v0.w + p1 * v1.w;
+        for (int r = 0; r < R; r++) {
+            const long at = base + (long)min(tb + r * NSLOT, last) * hs;
+            kk[r] = *reinterpret_cast<const float4 *>(a.kc + at);
+            vv[r] = *reinterpret_cast<const float4 *>(a.vc + at);
+        }
+        float sv[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int t = tb + r * NSLOT;
+            const bool cached = on && t < pos;
+            // (component by component: a choice between whole float4s went through scratch memory)
+            kk[r].x = t == pos ? kp.x : cached ? kk[r].x : 0.0f; kk[r].y = t == pos ? kp.y : cached ? kk[r].y : 0.0f;
+            kk[r].z = t == pos ? kp.z : cached ? kk[r].z : 0.0f; kk[r].w = t == pos ? kp.w : cached ? kk[r].w : 0.0f;
+            vv[r].x = t == pos ? vp.x : cached ? vv[r].x : 0.0f; vv[r].y = t == pos ? vp.y : cached ? vv[r].y : 0.0f;
+            vv[r].z = t == pos ? vp.z : cached ? vv[r].z : 0.0f; vv[r].w = t == pos ? vp.w : cached ? vv[r].w : 0.0f;
+            sv[r] = (q4.x * kk[r].x + q4.y * kk[r].y) + (q4.z * kk[r].z + q4.w * kk[r].w);
+        }
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) {
+#pragma unroll
+            for (int r = 0; r < R; r++) sv[r] += __shfl_xor(sv[r], off);
+        }
+        float mb = m;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            sv[r] = tb + r * NSLOT < len ? __fdiv_rn(sv[r], a.sqrt_hs) : -3.0e38f;
+            mb = fmaxf(mb, sv[r]);
+        }
+        const float sc = expf(m - mb);
+        l *= sc;
+        acc.x *= sc; acc.y *= sc; acc.z *= sc; acc.w *= sc;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float p = tb + r * NSLOT < len ? expf(sv[r] - mb) : 0.0f;
+            l += p;
+            acc.x += p * vv[r].x; acc.y += p * vv[r].y; acc.z += p * vv[r].z; acc.w += p * vv[r].w;
+        }
         m = mb;
     }
     if (j == 0) { sm_m[slot] = m; sm_l[slot] = l; }
