@@ -93,6 +93,25 @@ def test_topp_with_many_equal_probabilities_keeps_the_stable_order(orc, monkeypa
         check_probabilities(g.read(BUFFER.LOGITS), probs)
 
 
+@WIDE
+@pytest.mark.parametrize("vocab", [2, 3, 64, 256, 257, 512, 4096, 8193])
+def test_vocabularies_at_the_edges_of_slices_tiles_and_runs(orc, monkeypatch, vocab, wide):
+    """A slice of the one-launch step and a tile of the sort hold 256 probabilities, a run 4096: vocabularies of exactly
+    one, one more, and the smallest there are; top-p and plain calls mixed, so entries of earlier calls take part."""
+    monkeypatch.setenv("L2J_SAMPLER_WIDE", wide)
+    g = small_transformer(vocab)
+    rng = np.random.default_rng(vocab * 7 + 1)
+    g.sampler_seed(vocab)
+    o = orc.Sampler(vocab, vocab)
+    for call in range(10):
+        lg = logits_of(rng, vocab, ("flat", "peaked", "mid")[call % 3])
+        t = float(rng.choice([0.6, 0.9, 1.3]))
+        topp = float(rng.choice([0.4, 0.9, 0.97, 1.0]))
+        want, probs = o.step(lg, t, topp)
+        assert g.sample(t, topp, logits=lg) == want, (call, topp)
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
+
+
 def test_topp_worked_example_with_entries_of_an_earlier_call(orc):
     # the hand-worked case of the oracle's tests, on the device: eight tokens, padded with impossible ones
     vocab = 16
