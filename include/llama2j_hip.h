@@ -95,7 +95,8 @@ int l2j_device_count(void);
  * layers of a step in one resident kernel with grid barriers instead of eight launches per layer; the same results,
  * slower as measured, 0 by default; a bounded wait of that kernel that runs out is L2J_E_HIP), "sampler_wide" (1, the default: a
  * sampling step of a vocabulary of at most 36864 is one launch of a workgroup per 256 probabilities with grid barriers; a
- * bounded wait of it that runs out is L2J_E_HIP; 0: one launch per stage, as larger vocabularies always take).  l2j_get_option reads the value in force
+ * bounded wait of it that runs out is L2J_E_HIP, and the context sets the option to 0 itself: seed the sampler again and go on;
+ * 0: one launch per stage, as larger vocabularies always take).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);

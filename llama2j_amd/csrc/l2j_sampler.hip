@@ -243,7 +243,10 @@ int l2j::check_sampler_status(l2j_ctx *c)
     HIPCHK(hipMemcpy(&c->ss->nan, &c->h_ss->nan, sizeof(int), hipMemcpyHostToDevice));
     if (st & 4) {   // (the counters of the launch are not where the next one expects them)
         if (c->wide_mem) HIPCHK(hipMemset(c->wide_mem, 0, sizeof(WideSync)));
-        return fail(L2J_E_HIP, "sampler: a workgroup waited too long for the others (k_sample_wide needs a compute unit per 256 probabilities)");
+        c->opt[OPT_SAMPLER_WIDE] = 0;   // (something else holds compute units: from here on one launch per stage, which waits for nobody)
+        return fail(L2J_E_HIP, "sampler: a workgroup waited too long for the others (k_sample_wide needs a compute unit per 256 "
+                               "probabilities); the step was not completed, the context takes one launch per stage from now on: "
+                               "seed the sampler again (l2j_sampler_seed, or a new l2j_decode_sample)");
     }
     if (st & 1) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
     return fail(L2J_E_ARG, "sampler: no probability reaches the top-p cutoff (ArrayIndexOutOfBoundsException at J/Sampler.java:119)");

@@ -721,7 +721,7 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
         if (tid == 0) cp[0] = 0;
         __syncthreads();
     }
-    const int n0 = cp[G];
+    const int n0 = min(cp[G], n);   // (more only after a barrier that gave up: what follows stays inside the arrays)
     if (g == 0 && tid == 0) a.ss->n0 = n0;
     if (n0 <= 0) {   // no probability reaches the cutoff (NaNs, or topp near 0 on a flat distribution): the reference
         if (g == 0 && tid == 0) {   // indexes probIndex[-1] and throws; the host reports the call as failed
@@ -739,7 +739,7 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
             for (int st = 128; st > 0; st >>= 1)
                 if (h + st < G && cp[h + st] <= i) h += st;
             const unsigned long long cm[4] = {cmw[4 * h], cmw[4 * h + 1], cmw[4 * h + 2], cmw[4 * h + 3]};
-            val = h * kWideSlice + wide_kth_bit(cm, i - cp[h]);
+            val = min(h * kWideSlice + wide_kth_bit(cm, i - cp[h]), n - 1);
             key = ld_coh(a.logits + val);
         } else if (i < n) {
             key = a.old_prob[i];
@@ -887,7 +887,7 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
         if (tid == 0) {
             int pick = L.hit;
             if (pick < 0 || pick > last) pick = last;
-            const int token = ld_coh(a.new_idx + pick);
+            const int token = ld_coh(a.new_idx + min(pick, n - 1));
             a.ss->result = token;
             if (a.st) {
                 a.out_tokens[a.st->pos - 1] = token;

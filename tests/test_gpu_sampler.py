@@ -254,6 +254,29 @@ def test_temperature_zero_is_first_max_and_nan_is_an_error(orc):
     assert g.sample(1.0, 0.0, logits=lg, coin=0.9) == 17               # ties keep index order; cumulative > 0 at once
 
 
+def test_a_wait_of_the_one_launch_step_that_runs_out_is_an_error_and_the_context_falls_back(orc):
+    """barrier_spins 0: the first workgroup to reach a grid barrier gives up at once (every kernel still runs to its end).
+    The call fails, the context then samples with one launch per stage, and a newly seeded sampler gives the oracle's tokens."""
+    vocab = 1003
+    g = l2j.Transformer(l2j.Config(32, 64, 1, 2, 2, vocab, 8, 1))
+    g.fill_synthetic(3, 0.1)
+    g.set_option("barrier_spins", 0)
+    g.finalize()
+    assert g.get_option("sampler_wide") == 1
+    rng = np.random.default_rng(4)
+    lg = logits_of(rng, vocab, "mid")
+    g.sampler_seed(6)
+    with pytest.raises(L2JError):
+        g.sample(0.9, 0.9, logits=lg)
+    assert g.get_option("sampler_wide") == 0
+    g.sampler_seed(6)
+    o = orc.Sampler(6, vocab)
+    for topp in (0.9, 1.0, 0.5):
+        want, probs = o.step(lg, 0.9, topp)
+        assert g.sample(0.9, topp, logits=lg) == want
+        check_probabilities(g.read(BUFFER.LOGITS), probs)
+
+
 def test_largest_vocabulary_the_sampler_takes(orc):
     vocab = 36864
     g = small_transformer(vocab)
