@@ -178,7 +178,7 @@ __device__ __forceinline__ unsigned long long wide_segscan(int &x0, int &x1, int
 
 // Level 0 of slice g by one wave: lane l holds the terms 4 l .. 4 l + 3 of the slice, base = the (double-precision,
 // approximate) sum of everything before the slice.  Leaves the lanes' scanned pairs and the slice's own pair in set `set`.
-__device__ __forceinline__ void wide_reduce(const WideWs &w, int set, int g, float4 t, double base)
+__device__ __forceinline__ void wide_reduce(const WideWs &w, int set, int g, float4 t, double base, double mark = -1.0)
 {
     const int lane = threadIdx.x & 63;
     const double loc = (double)t.x + (double)t.y + (double)t.z + (double)t.w;
@@ -210,7 +210,10 @@ __device__ __forceinline__ void wide_reduce(const WideWs &w, int set, int g, flo
         const int s = set * kWideMaxSlices + g;
         st_coh(w.t_x0 + s, x0);
         st_coh(w.t_x1 + s, x1);
-        st_coh(w.t_m + s, (segs == 1ull) ? m : 0);
+        // (a slice near which the sum is expected to pass `mark` is handed over as not uniform: the walker stages those
+        // in LDS, and the walk that looks for the crossing inside it finds its lanes there instead of in memory)
+        const bool near = mark >= 0.0 && base <= mark * 1.002 && p_end >= mark * 0.998;
+        st_coh(w.t_m + s, (segs == 1ull && !near) ? m : 0);
         st_coh(w.seg + s, segs);
     }
 }
@@ -858,7 +861,7 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
         b2 = wide_wave_sum(b2);
         if (lane == 0) dred[wave] = b2;
         __syncthreads();
-        if (wave == 0) wide_reduce(a.w, 1, g, wide_terms(a.new_prob, g * kWideSlice + 4 * lane, n0), dred[0] + dred[1] + dred[2] + dred[3]);
+        if (wave == 0) wide_reduce(a.w, 1, g, wide_terms(a.new_prob, g * kWideSlice + 4 * lane, n0), dred[0] + dred[1] + dred[2] + dred[3], (double)a.topp);
     }
     wide_barrier(a.w, bar++);
 
