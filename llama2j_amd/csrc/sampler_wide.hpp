@@ -31,7 +31,7 @@
 // stretch's start by the pair before it) the slice, the lane, the term.
 //
 // What the stages cost on an MI355X (vocabulary 32000, flat distribution, in-kernel time stamps): a grid barrier of 125
-// workgroups 2.5-3 us (arrivals counted per group: one counter took 3.5-6 us, an atomic on one address every ~30 ns), a
+// workgroups 2.5-3 us (arrivals counted per group of sixteen at the time; one counter took 3.5-6 us, an atomic on one address every ~30 ns), a
 // dependent device-coherent load 1-2.5 us, A 4.3, B 1.6, staging + plan 7.7, the walk 6.8, D 4.8, E 3.2, F 7.0 (4.7 of it
 // the 128 KB of keys every workgroup fetches), G 3.2, the two walks of the pick 8.5 + 3.8: 77 us, against 105 us for the
 // six launches of the launch-per-stage form as it was, 88 us now that its sort probes the same way as E and F here.
@@ -47,7 +47,8 @@ constexpr int kWideMaxSlices = kSampleMaxVocab / kWideSlice;   // 144
 constexpr int kWideSlots = 16;                                 // mixed slices staged in LDS ahead of a walk
 constexpr int kWideItems = 192;                                // steps of a planned walk
 
-constexpr int kWideGroups = 8;   // arrivals are counted per group of workgroups first: a counter takes one atomic every ~30 ns
+constexpr int kWideGroups = 4;   // arrivals are counted per group of workgroups first: a counter takes one atomic every ~30 ns
+                                 // (per sampled token: 2, 3, 4 groups the same, 8 +1.3 us, 16 +5 us, one counter +12 us)
 struct WideSync {
     unsigned ctr;    // groups that have arrived at the barriers of the launch in flight
     unsigned pad0[15];
