@@ -266,6 +266,23 @@ def main():
             out["batched_decode"]["sixteen_sequences"] = {k: runs[16][k] for k in ("tok_s", "ms_per_step", "sequence_0_equals_the_single_decode")}
         except l2j.L2JError as e:  # shapes the batched path does not take (rows that are not whole groups of 256)
             out["batched_decode"] = {"error": str(e)}
+        # Nor this: the forward passes of 1024 consecutive positions of one sequence, 32 at a time through the same products
+        # (l2j_prefill), as a prompt of that length would be taken instead of one position per launch.
+        try:
+            n_pre = min(1024, shape[6] - 1)
+            ptoks = np.concatenate([[1], tokens[:min(len(tokens), n_pre - 1)],
+                                    synth_prompt(seed + 77, max(0, n_pre - 1 - len(tokens)), shape[5])]).astype(np.int32)[:n_pre]
+            g.reset()
+            g.prefill(ptoks[:32], want_logits=False)     # warm
+            g.reset()
+            _, psec = g.prefill(ptoks, want_logits=False)
+            out["prefill"] = {"positions": int(n_pre), "positions_per_s": round(n_pre / psec, 1), "ms": round(psec * 1e3, 3),
+                              "ms_per_32_positions": round(psec * 1e3 / ((n_pre + 31) // 32), 4),
+                              "note": "l2j_prefill: the forward passes of consecutive positions of one sequence, 32 per step on the "
+                                      "matrix cores, into the KV cache of the single-sequence path (device time)"}
+            g.reset()
+        except l2j.L2JError as e:
+            out["prefill"] = {"error": str(e)}
 
     if a.calibrate_copy > 0:
         g.calibration_copy(a.calibrate_copy << 20, 3)

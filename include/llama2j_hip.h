@@ -96,7 +96,10 @@ int l2j_device_count(void);
  * slower as measured, 0 by default; a bounded wait of that kernel that runs out is L2J_E_HIP), "sampler_wide" (1, the default: a
  * sampling step of a vocabulary of at most 36864 is one launch of a workgroup per 256 probabilities with grid barriers; a
  * bounded wait of it that runs out is L2J_E_HIP, and the context sets the option to 0 itself: seed the sampler again and go on;
- * 0: one launch per stage, as larger vocabularies always take).  l2j_get_option reads the value in force
+ * 0: one launch per stage, as larger vocabularies always take), "prefill" (0, the default: the decode loops take the prompt
+ * positions one by one, as the reference does; 1: the first whole steps of 32 prompt positions go through l2j_prefill, the
+ * loop goes on behind them: the same tokens but where two logits lie within rounding of each other; shapes l2j_prefill
+ * does not take run as with 0).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);
@@ -226,6 +229,16 @@ int l2j_read_checkpoint_header(const char *bin_path, l2j_config *cfg);
  * quantizes (on the GPU) and, when write_caches != 0, writes the cache; uploads; finalizes. */
 int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int write_caches, l2j_ctx **out);
 int l2j_get_config(l2j_ctx *ctx, l2j_config *cfg);
+
+/* The forward passes of n consecutive positions pos0 .. pos0 + n - 1 of one sequence, tokens[i] being the input token of
+ * position pos0 + i: what n calls of l2j_forward(tokens[i], pos0 + i) leave in the KV cache and return for the last of
+ * them, i.e. the prompt positions of the token loop (J/Run.java:623-640: the reference runs them one by one through
+ * Run.transformer), 32 positions per step through the batched products on the matrix cores (every weight read once per
+ * 32 positions).  logits (null: not wanted): the vocab_size logits of the last position; they are also what l2j_sample
+ * samples from next.  seconds (null: not wanted): device time of the steps.  The sums are formed in another order than
+ * l2j_forward's, so cache rows and logits agree with its to rounding (1e-6 of the largest), not bit for bit.  Shapes as for
+ * l2j_decode_greedy_batch (else L2J_E_SIZE: take l2j_forward); its buffers and its copy of the matrices are shared. */
+int l2j_prefill(l2j_ctx *ctx, const int32_t *tokens, int32_t n, int32_t pos0, float *logits, double *seconds);
 
 /* ======================================================================================================
  * Measurement and test entry points.  Not part of what a Mode.HIP binds: bench.py and the test-suite use them.

@@ -40,7 +40,7 @@ public final class ContextHIP implements AutoCloseable {
     // buffers of the token loop's thread, allocated once (no allocation per token)
     private final MemorySegment logitsSeg, intSeg, tokensSeg, promptSeg, countSeg, secondsSeg;
     private final MethodHandle lastError, ctxLastError, destroy, setOption, uploadQuant, uploadF32, finalizeH, reset, forward,
-            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSample, samplerSeed, sample;
+            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSample, samplerSeed, sample, prefill;
 
     private MethodHandle handle(String name, FunctionDescriptor fd) {
         return LINKER.downcallHandle(lib.find(name).orElseThrow(), fd);
@@ -66,6 +66,7 @@ public final class ContextHIP implements AutoCloseable {
                 JAVA_FLOAT, JAVA_FLOAT, JAVA_LONG, ADDRESS, ADDRESS, ADDRESS));
         samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
         sample = handle("l2j_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_FLOAT, JAVA_FLOAT, JAVA_FLOAT, ADDRESS));
+        prefill = handle("l2j_prefill", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
 
         MemorySegment out = arena.allocate(ADDRESS);
         MemorySegment cfg = arena.allocate(48, 4);   // l2j_config: twelve 32-bit fields
@@ -254,6 +255,20 @@ public final class ContextHIP implements AutoCloseable {
             for (int b = 0; b < batch; b++) MemorySegment.copy(out, JAVA_INT, (long) b * steps * Integer.BYTES, tokens[b], 0, steps);
             return tokens;
         }
+    }
+
+    /**
+     * Run.transformer(tokens[i], pos0 + i, ...) for every i (the prompt positions of Run.main's loop), 32 positions per
+     * step on the matrix cores (l2j_prefill); logits (may be null) receives those of the last position.  The token loop
+     * then goes on at position pos0 + tokens.length with forwardArgmax / forward.
+     */
+    public void prefill(int[] tokens, int pos0, float[] logits) {
+        try (Arena a = Arena.ofConfined()) {
+            MemorySegment ids = a.allocate((long) tokens.length * Integer.BYTES, 16);
+            MemorySegment.copy(tokens, 0, ids, JAVA_INT, 0, tokens.length);
+            check(call(prefill, ctx, ids, tokens.length, pos0, logits == null ? MemorySegment.NULL : logitsSeg, secondsSeg));
+        }
+        if (logits != null) MemorySegment.ofArray(logits).copyFrom(logitsSeg.asSlice(0, (long) logits.length * Float.BYTES));
     }
 
     /** The token loop of Run.main with Sampler(rngSeed) on the device (temperature, top-p as in CommandLine). */

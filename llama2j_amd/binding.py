@@ -108,6 +108,7 @@ def _signatures():
         "l2j_running_sums": (C.c_int, [vp, fp, C.c_int32, fp]),
         "l2j_running_sums_noalloc": (C.c_int, [vp, fp, C.c_int32, fp]),
         "l2j_sum_probe": (C.c_int, [vp, fp, C.c_int32, fp, C.c_int32, i32p, fp, fp]),
+        "l2j_prefill": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, fp, C.POINTER(C.c_double)]),
         "l2j_decode_sample": (C.c_int, [vp, i32p, C.c_int32, C.c_int32, C.c_float, C.c_float, C.c_int64, i32p, i32p,
                                         C.POINTER(C.c_double)]),
         "l2j_read": (C.c_int, [vp, C.c_int, C.c_int, C.c_uint64, fp, C.c_uint64]),
@@ -376,6 +377,16 @@ class Transformer:
         logits = np.empty(self.config.vocab_size, dtype=np.float32) if want_logits else None
         self._check(lib().l2j_forward(self._h, token, pos, _fp(logits) if want_logits else None))
         return logits
+
+    def prefill(self, tokens, pos0=0, want_logits=True):
+        """forward(tokens[i], pos0 + i) for every i, 32 positions per step on the matrix cores: (logits of the last
+        position or None, device seconds)."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        logits = np.empty(self.config.vocab_size, dtype=np.float32) if want_logits else None
+        sec = C.c_double(0.0)
+        self._check(lib().l2j_prefill(self._h, tokens.ctypes.data_as(C.POINTER(C.c_int32)), tokens.size, pos0,
+                                      _fp(logits) if want_logits else None, C.byref(sec)))
+        return logits, sec.value
 
     def forward_argmax(self, token, pos):
         nxt = C.c_int32(-1)

@@ -562,6 +562,10 @@ struct BAttn {
     const BatchState *st;
     int n_heads, kv_mul, head_size, kv_dim, dim;
     float sqrt_hs;
+    // MODE 1, 2 (the rows are consecutive positions of ONE sequence, st->pos + b, in one cache):
+    long head_stride;            // floats between two kv heads of a position's row
+    int row_stride;              // and between two positions
+    int nrows;                   // rows in use: the others neither store nor attend
 };
 
 // Attention of one head of one sequence over positions 0..pos (K/AttentionLoop.java:29-54, K/ExpSumNormalize.java:25-38,
@@ -571,7 +575,11 @@ struct BAttn {
 // workgroup take the positions in turn with an online softmax, and the slots are folded at the end.  grid (n_heads, sequences).
 constexpr int kBattnRows = 4;
 
-template <int LPR>
+// MODE 0: the sequences of a batch, all at position st->pos, each with a cache of its own (head-major).  MODE 1 and 2: the
+// rows are the positions st->pos + b of one sequence sharing one cache (any layout: head_stride, row_stride): 1 only stores
+// k and v of its position, 2 only attends (over the rows below its own position, which a launch in MODE 1 has stored,
+// and its own).
+template <int LPR, int MODE = 0>
 __global__ void __launch_bounds__(256) k_battn(const BAttn a)
 {
     constexpr int RPW = 64 / LPR, NSLOT = 4 * RPW;
@@ -580,7 +588,11 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
     __shared__ __align__(16) float sm_qkv[3][4 * LPR];
     const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     const int j = lane % LPR, slot = (tid >> 6) * RPW + lane / LPR;
-    const int pos = a.st->pos, len = pos + 1, hs = a.head_size, kvh = h / a.kv_mul;
+    if (MODE != 0 && b >= a.nrows) return;
+    if (MODE == 1 && h % a.kv_mul != 0) return;   // (one head of a group stores its kv head)
+    const int pos = a.st->pos + (MODE != 0 ? b : 0), len = pos + 1, hs = a.head_size, kvh = h / a.kv_mul;
+    const long hstride = MODE != 0 ? a.head_stride : (long)a.cap * hs;
+    const int rs = MODE != 0 ? a.row_stride : hs;
     const int half = hs >> 1;
     for (int p = tid; p < 3 * half; p += 256) {   // one thread per pair of q, k, v
         const int which = p / half, idx = p - which * half;
@@ -601,18 +613,19 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
             }
             sm_qkv[which][2 * idx] = v0;
             sm_qkv[which][2 * idx + 1] = v1;
-            if (which > 0 && h % a.kv_mul == 0)
-                *reinterpret_cast<float2 *>((which == 1 ? a.kc : a.vc) + (long)b * a.seq_stride + ((long)kvh * a.cap + pos) * hs + 2 * idx) =
+            if (MODE != 2 && which > 0 && h % a.kv_mul == 0)
+                *reinterpret_cast<float2 *>((which == 1 ? a.kc : a.vc) + (long)b * a.seq_stride + kvh * hstride + (long)pos * rs + 2 * idx) =
                     make_float2(v0, v1);
         }
     }
+    if (MODE == 1) return;
     __syncthreads();
     const bool on = 4 * j < hs;
     const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4 q4 = on ? *reinterpret_cast<const float4 *>(&sm_qkv[0][4 * j]) : zero;
     const float4 kp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[1][4 * j]) : zero;   // the row of this position
     const float4 vp = on ? *reinterpret_cast<const float4 *>(&sm_qkv[2][4 * j]) : zero;
-    const long base = (long)b * a.seq_stride + (long)kvh * a.cap * hs + 4 * j;   // the head's rows lie one after the other
+    const long base = (long)b * a.seq_stride + kvh * hstride + 4 * j;   // (MODE 0: the head's rows lie one after the other)
     float m = -3.0e38f, l = 0.0f;
     float4 acc = zero;
     constexpr int R = kBattnRows;   // rows in flight per slot
@@ -623,7 +636,7 @@ __global__ void __launch_bounds__(256) k_battn(const BAttn a)
         float4 kk[R], vv[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const long at = base + (long)min(tb + r * NSLOT, last) * hs;
+            const long at = base + (long)min(tb + r * NSLOT, last) * rs;
             kk[r] = *reinterpret_cast<const float4 *>(a.kc + at);
             vv[r] = *reinterpret_cast<const float4 *>(a.vc + at);
         }
@@ -736,6 +749,16 @@ static __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *
 }
 
 // y[b][r] = sum over the slices, in slice order
+// y[0..rows) = row `row` of the product whose slices lie in part, (slices, nseq, rows)
+static __global__ void __launch_bounds__(256) k_brow(const float *__restrict__ part, float *__restrict__ y, int rows, int slices, int nseq, int row)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < rows; i += gridDim.x * blockDim.x) {
+        float t = 0.0f;
+        for (int sl = 0; sl < slices; sl++) t += part[((long)sl * nseq + row) * rows + i];
+        y[i] = t;
+    }
+}
+
 static __global__ void __launch_bounds__(256) k_breduce(const float *__restrict__ part, float *__restrict__ y, int rows, int slices)
 {
     const long n = (long)kBatch * rows;

@@ -311,6 +311,55 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
 }
 
 
+// The forward passes of `rows` consecutive positions of one sequence (st: their tokens and the first position) as one batched
+// step into the context's own KV cache: launch_batch_step's kernels, the attention as two launches (every position stores
+// its k and v, then every position attends over the rows up to its own), and the classifier only when `last_logits`.
+void launch_prefill_block(l2j_ctx *c, BatchBufs &b, const BatchState *st, int rows, bool last_logits)
+{
+    const l2j_config &cf = c->cfg;
+    const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim, nseq = kMaxBatch;
+    const int sd = batch_slices(dim), sh = batch_slices(hidden);
+    hipStream_t s = c->stream;
+    hipLaunchKernelGGL(k_bembed, dim3(nseq), dim3(256), 0, s, c->emb, st, b.x, dim, (unsigned *)nullptr);
+    hipLaunchKernelGGL(k_brms, dim3(nseq), dim3(1024), 0, s, b.x, c->rmsw, b.xn, dim);
+    for (int l = 0; l < L; l++) {
+        launch_bgemm(c, {L2J_WQ, L2J_WK, L2J_WV}, l, b.xn, b.part, nseq);
+        BAttn t{};
+        t.pq = b.part[0]; t.pk = b.part[1]; t.pv = b.part[2]; t.slices = sd; t.rope = c->rope;
+        t.kc = c->kcache + (size_t)l * cf.seq_len * kvd; t.vc = c->vcache + (size_t)l * cf.seq_len * kvd;   // (position, kv_dim) per layer
+        t.seq_stride = 0; t.cap = cf.seq_len; t.out = b.xb; t.st = st;
+        t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
+        t.sqrt_hs = sqrtf((float)hs);
+        t.head_stride = hs; t.row_stride = kvd; t.nrows = rows;
+        const dim3 ag(cf.n_heads, nseq);
+        if (hs == 64) {
+            hipLaunchKernelGGL((k_battn<16, 1>), ag, dim3(256), 0, s, t);
+            hipLaunchKernelGGL((k_battn<16, 2>), ag, dim3(256), 0, s, t);
+        } else if (hs == 128) {
+            hipLaunchKernelGGL((k_battn<32, 1>), ag, dim3(256), 0, s, t);
+            hipLaunchKernelGGL((k_battn<32, 2>), ag, dim3(256), 0, s, t);
+        } else {
+            hipLaunchKernelGGL((k_battn<64, 1>), ag, dim3(256), 0, s, t);
+            hipLaunchKernelGGL((k_battn<64, 2>), ag, dim3(256), 0, s, t);
+        }
+        launch_bgemm(c, {L2J_WO}, l, b.xb, b.part, nseq);
+        hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim);
+        launch_bgemm(c, {L2J_W1, L2J_W3}, l, b.xn, b.part, nseq);
+        hipLaunchKernelGGL(k_bepi_swiglu, dim3(hidden / 256, nseq), dim3(256), 0, s, b.part[0], b.part[1], sd, hidden, c->silu,
+                           (cf.flags & L2J_F_EXACT_SILU) ? 1 : 0, b.hb);
+        launch_bgemm(c, {L2J_W2}, l, b.hb, b.part, nseq);
+        const float *wn = c->rmsw + (l + 1 < L ? (size_t)(l + 1) * dim : (size_t)2 * L * dim);
+        hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sh, b.x, wn, b.xn, dim);
+    }
+    if (last_logits) {
+        BGemmF32 g{};
+        g.w = c->wcls; g.rows = cf.vocab_size; g.K = dim; g.x = b.xn; g.part = b.part[0]; g.gps = kClsGps;
+        const dim3 cg((cf.vocab_size + kBgRowsPerWG - 1) / kBgRowsPerWG, cls_slices(dim));
+        hipLaunchKernelGGL(k_bgemm_f32<2>, cg, dim3(kBgThreads), batch_lds_f32(nseq), s, g);
+        hipLaunchKernelGGL(k_brow, dim3(64), dim3(256), 0, s, b.part[0], c->logits, cf.vocab_size, cls_slices(dim), nseq, rows - 1);
+    }
+}
+
 int hip_rc(hipError_t e, const char *what)
 {
     return fail(e == hipErrorOutOfMemory ? L2J_E_OOM : L2J_E_HIP, std::string("batched decode: ") + what + ": " + hipGetErrorString(e));
@@ -477,7 +526,67 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
 
 }  // namespace
 
+int l2j::prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t pos0, float *logits, double *seconds)
+{
+    if (!c || !tokens) return fail(L2J_E_ARG, "null argument");
+    if (!c->finalized) return fail(L2J_E_STATE, "prefill before l2j_finalize");
+    const l2j_config &cf = c->cfg;
+    const int hs = c->head_size;
+    if (cf.dim % 256 || cf.hidden_dim % 256 || c->kv_dim % 16 || cf.vocab_size % 16 || (hs != 64 && hs != 128 && hs != 256))
+        return fail(L2J_E_SIZE, "prefill needs dim and hidden_dim in whole groups of 256, kv_dim and vocab_size multiples of 16, "
+                                "head_size 64, 128 or 256 (as the batched decode); take l2j_forward position by position");
+    if (n <= 0 || pos0 < 0 || (long)pos0 + n > cf.seq_len) return fail(L2J_E_ARG, "positions pos0 .. pos0 + n - 1 must lie in 0 .. seq_len - 1");
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= cf.vocab_size) return fail(L2J_E_ARG, "token id out of range");
+    HIPCHK(hipSetDevice(cf.device));
+    if (!c->bt_ready) {   // the matrices once more, in the order the batched products read them
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        for (int t : {L2J_WQ, L2J_WK, L2J_WV, L2J_WO, L2J_W1, L2J_W2, L2J_W3}) {
+            const int trc = ensure_batch_tiles(c, t);
+            if (trc) return trc;
+        }
+        c->bt_ready = true;
+    }
+    int rc = c->batch && c->batch->nseq == kMaxBatch ? L2J_OK : ensure_batch(c, kMaxBatch, 1, 1);
+    if (rc) return rc;
+    BatchBufs &b = *c->batch;
+    const int nblocks = (n + kMaxBatch - 1) / kMaxBatch;
+    std::vector<BatchState> hst((size_t)nblocks);
+    for (int k = 0; k < nblocks; k++) {
+        hst[k] = BatchState{};
+        hst[k].pos = pos0 + k * kMaxBatch;
+        for (int r = 0; r < kMaxBatch; r++) hst[k].token[r] = tokens[std::min(k * kMaxBatch + r, n - 1)];   // (rows past the end: not stored, not read)
+    }
+    BatchState *dst = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&dst), (size_t)nblocks * sizeof(BatchState));
+    if (e != hipSuccess) return hip_rc(e, "prefill: positions");
+    e = hipMemcpyAsync(dst, hst.data(), (size_t)nblocks * sizeof(BatchState), hipMemcpyHostToDevice, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);   // (hst is pageable host memory)
+    if (e == hipSuccess) e = hipEventRecord(b.e0, c->stream);
+    for (int k = 0; k < nblocks && e == hipSuccess; k++) {
+        launch_prefill_block(c, b, dst + k, std::min(kMaxBatch, n - k * kMaxBatch), k + 1 == nblocks);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);
+    if (e == hipSuccess && logits) e = hipMemcpyAsync(logits, c->logits, (size_t)cf.vocab_size * sizeof(float), hipMemcpyDeviceToHost, c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    (void)hipFree(dst);
+    if (e != hipSuccess) return hip_rc(e, "prefill");
+    float ms = 0.0f;
+    if ((e = hipEventElapsedTime(&ms, b.e0, b.e1)) != hipSuccess) return hip_rc(e, "prefill: timing");
+    if (seconds) *seconds = (double)ms * 1e-3;
+    return L2J_OK;
+}
+
 extern "C" {
+
+int l2j_prefill(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t pos0, float *logits, double *seconds)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        return prefill_positions(c, tokens, n, pos0, logits, seconds);
+    }());
+}
 
 int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride,
                             int32_t steps, int32_t *out_tokens, double *seconds)

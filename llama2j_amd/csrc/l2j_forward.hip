@@ -359,10 +359,35 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
     }
     if ((rc = set_state(c, 1, 0, np))) return rc;  // token 1 = BOS at pos 0 (J/Run.java:614)
 
+    // Option prefill: the first P prompt positions (whole steps of 32; their outputs are the prompt's own ids, J/Run.java:635-637)
+    // through the batched products, the loop then goes on at position P.  Not when one of those ids is 1 (the loop would
+    // have stopped there, J/Run.java:670-672), nor for shapes the batched products do not take.
+    int P = 0;
+    double prefill_s = 0.0;
+    if (c->opt[OPT_PREFILL] != 0 && np >= 32 && steps > 32) {
+        P = std::min(np, steps - 1) / 32 * 32;
+        for (int i = 0; i < P; i++)
+            if (prompt[i] == 1) P = 0;
+        if (P > 0) {
+            std::vector<int32_t> in((size_t)P);
+            in[0] = 1;
+            for (int i = 1; i < P; i++) in[i] = prompt[i - 1];
+            rc = prefill_positions(c, in.data(), P, 0, nullptr, &prefill_s);
+            if (rc == L2J_E_SIZE) {
+                P = 0;   // (a shape for l2j_forward only)
+            } else if (rc) {
+                return rc;
+            } else {
+                for (int i = 0; i < P; i++) out_tokens[i] = prompt[i];
+                if ((rc = set_state(c, prompt[P - 1], P, np))) return rc;
+            }
+        }
+    }
+
     // The stop rule (next == 1) is checked per batch of tokens, and the clock runs from the end of the first token to
-    // the end of the token that ended the loop.
+    // the end of the token that ended the loop (plus, with option prefill, the device time of its steps).
     float total_ms = 0.f;
-    int pos = 0;
+    int pos = P;
     bool stopped = false;
     if (!sampled) {
         // Greedy: the last kernel of every token stores the device's wall clock for its position; a full batch is one
@@ -376,7 +401,7 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
             c->events.push_back(ev);
         }
         unsigned long long t_first = 0, t_last = 0;
-        int enq = 0, nbatch = 0, done_batches = 0;  // positions enqueued; batches enqueued and processed
+        int enq = P, nbatch = 0, done_batches = 0;  // positions enqueued; batches enqueued and processed
         auto enqueue = [&]() -> int {
             const int nb = std::min(batch, steps - enq);
             if (c->graph_n_exec && nb == c->graph_tokens) {
@@ -408,7 +433,7 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
                     break;
                 }
             }
-            if (pos == 0) t_first = c->h_tstamp[0];
+            if (pos == P) t_first = c->h_tstamp[P];
             t_last = c->h_tstamp[pos + used - 1];
             pos += used;
         }
@@ -430,7 +455,7 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
             for (int i = 0; i < nb; i++) {
                 HIPCHK(launch_one_token(c));
                 if (pos + i >= np) HIPCHK(launch_sampler(c, temperature, topp, -1.0f, true));  // J/Run.java:635-665
-                if (pos + i == 0) HIPCHK(hipEventRecord(ev_first, c->stream));
+                if (pos + i == P) HIPCHK(hipEventRecord(ev_first, c->stream));
                 HIPCHK(hipEventRecord(c->events[i], c->stream));
             }
             HIPCHK(hipMemcpyAsync(c->h_tokens, c->out_tokens + pos, (size_t)nb * sizeof(int), hipMemcpyDeviceToHost, c->stream));
@@ -447,12 +472,12 @@ int decode_loop(l2j_ctx *c, const int32_t *prompt, int32_t n_prompt, int32_t ste
                     break;
                 }
             }
-            if (pos + used - 1 > 0) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
+            if (pos + used - 1 > P) HIPCHK(hipEventElapsedTime(&total_ms, ev_first, c->events[used - 1]));
             pos += used;
         }
     }
     *n_out = pos;
-    if (seconds) *seconds = (double)total_ms * 1e-3;
+    if (seconds) *seconds = (double)total_ms * 1e-3 + prefill_s;
     return L2J_OK;
 }
 

@@ -55,7 +55,7 @@ struct QTensor {
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_BATCH_FUSE, OPT_SAMPLER_WIDE, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_BATCH_FUSE, OPT_SAMPLER_WIDE, OPT_PREFILL, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -85,6 +85,7 @@ inline const OptionDef kOptions[OPT_COUNT] = {
     {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
     {"batch_fuse", 0, true},           // batched decode: 1: the layers of a step in one launch with grid barriers (slower, measured); 0: eight launches per layer
     {"sampler_wide", 1, true},         // sampling step: 1: one launch over many workgroups (vocabularies that fit in LDS), 0: one launch per stage
+    {"prefill", 0, true},              // decode loops: 1: the prompt positions 32 at a time through the batched products (l2j_prefill), 0: one by one as the reference
 };
 
 inline int option_from_env(int i)
@@ -242,6 +243,8 @@ int resolve_scratch(int device);
 void free_sampler(l2j_ctx *c);
 int seed_sampler(l2j_ctx *c, int64_t rng_seed);
 hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin, bool in_loop);
+// l2j_batch.hip: l2j_prefill without the lock (the decode loops call it holding it)
+int prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t pos0, float *logits, double *seconds);
 int check_sampler_status(l2j_ctx *c);
 int check_sampler_args(float temperature, float topp);
 
