@@ -134,7 +134,9 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=97, help="forwards of the CPU baseline sample (0 = skip)")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel timing")
     ap.add_argument("--no-sampled", action="store_true", help="skip the extra decode with the device sampler")
-    ap.add_argument("--no-batched", action="store_true", help="skip the extra decodes of 32 and 16 sequences at once")
+    ap.add_argument("--no-batched", action="store_true", help="skip the extra decodes of 32 and 16 sequences at once (and the prefill)")
+    ap.add_argument("--prefill-only", action="store_true", help="of those extras only the prefill (its kernels are launched one by one, "
+                                                                  "which a profiler can follow; the batched decode replays a graph)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
     a = ap.parse_args()
@@ -241,7 +243,7 @@ def main():
             out["sampled_decode"] = {"error": str(e)}
         g.reset()
 
-    if not a.no_batched and not long_context:
+    if (not a.no_batched or a.prefill_only) and not long_context:
         # Not the metric either: 32 (and 16) sequences decoded at once (every weight read once per step for all of them, the
         # products on the bf16 matrix cores); sequence 0 has the prompt of the timed run and must repeat its tokens.
         try:
@@ -251,7 +253,7 @@ def main():
             wbytes = g.bytes_per_token(0)      # the weights, read once per step for all sequences
             kvbytes = g.bytes_per_token(int(round(bmean))) - wbytes   # one sequence's cache rows at the mean position
             runs = {}
-            for n_seq in (32, 16):
+            for n_seq in (() if a.prefill_only else (32, 16)):
                 prompts = [prompt] + [synth_prompt(seed + 1000 + b, n_prompt, shape[5]) for b in range(1, n_seq)]
                 g.decode_greedy_batch(prompts, min(bsteps, 8), n_seq=n_seq)          # warm
                 btoks, bsec = g.decode_greedy_batch(prompts, bsteps, n_seq=n_seq)
@@ -262,8 +264,9 @@ def main():
                                             "bytes_per_step": int(wbytes + n_seq * kvbytes),
                                             "note": "weights once + every sequence's KV cache rows at the mean position, over the whole step time"},
                                "sequence_0_equals_the_single_decode": bool(np.array_equal(btoks[0, :n0], tokens[:n0]))}
-            out["batched_decode"] = runs[32]
-            out["batched_decode"]["sixteen_sequences"] = {k: runs[16][k] for k in ("tok_s", "ms_per_step", "sequence_0_equals_the_single_decode")}
+            if runs:
+                out["batched_decode"] = runs[32]
+                out["batched_decode"]["sixteen_sequences"] = {k: runs[16][k] for k in ("tok_s", "ms_per_step", "sequence_0_equals_the_single_decode")}
         except l2j.L2JError as e:  # shapes the batched path does not take (rows that are not whole groups of 256)
             out["batched_decode"] = {"error": str(e)}
         # Nor this: the forward passes of 1024 consecutive positions of one sequence, 32 at a time through the same products
