@@ -153,3 +153,22 @@ def test_prefill_at_the_published_widths(orc, shape, n):
     print("prefill logits vs oracle at widths %s: max|d|/max|logit| = %.3g" % (shape[:2], worst), flush=True)
     assert worst < LOGIT_TOL
     m.close()
+
+
+def test_prefill_and_the_batched_decode_share_their_buffers(orc):
+    """Both run in the context's batch buffers (32 rows for prefill): calls of either kind in any order give what they give alone."""
+    shape = SHAPES[1]
+    g = model(shape)
+    rng = np.random.default_rng(3)
+    tokens = np.concatenate([[1], rng.integers(2, shape[5], size=44)]).astype(np.int32)
+    prompts = [rng.integers(2, shape[5], size=3).astype(np.int32) for _ in range(16)]
+    alone_logits, _ = g.prefill(tokens)
+    alone_tokens, _ = g.decode_greedy_batch(prompts, 24, n_seq=16)        # (buffers for 16 sequences replace prefill's)
+    g.reset()
+    again_logits, _ = g.prefill(tokens)                                   # (and prefill's replace those)
+    assert np.array_equal(again_logits.view(np.uint32), alone_logits.view(np.uint32))
+    again_tokens, _ = g.decode_greedy_batch(prompts + prompts, 24, n_seq=32)
+    np.testing.assert_array_equal(again_tokens[:16], alone_tokens)
+    g.reset()
+    third, _ = g.prefill(tokens)                                          # (in the buffers of the 32 sequences)
+    assert np.array_equal(third.view(np.uint32), alone_logits.view(np.uint32))
