@@ -566,6 +566,7 @@ struct BAttn {
     long head_stride;            // floats between two kv heads of a position's row
     int row_stride;              // and between two positions
     int nrows;                   // rows in use: the others neither store nor attend
+    int nseq;                    // rows of the products' partial sums (k_pflash; k_battn has them as its grid)
 };
 
 // Attention of one head of one sequence over positions 0..pos (K/AttentionLoop.java:29-54, K/ExpSumNormalize.java:25-38,
@@ -749,6 +750,119 @@ static __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *
 }
 
 // y[b][r] = sum over the slices, in slice order
+// Attention of 16 consecutive positions of one sequence for one head on the fp32 matrix cores (after k_battn<LPR, 1> has
+// stored their k and v): every cache row is fetched once for the 16 queries, instead of once per query.
+//   scores, transposed: S^T (16 keys x 16 queries) = K (16 keys x HS) . Q^T (HS x 16 queries), HS / 4 v_mfma_f32_16x16x4_f32;
+//     a lane (c = lane % 16, g = lane / 16) then holds S^T[key 4 g + e][query c], e = 0..3: the keys of a query lie in four
+//     lanes, so a query's maximum is two cross-lane steps, and the same registers are the B operand of
+//   values, transposed: O^T (HS x 16 queries) += V^T (HS x 16 keys) . P^T (16 keys x 16 queries), HS / 4 more;
+//   online softmax over the tiles of 16 keys (K/AttentionLoop.java:29-54, K/ExpSumNormalize.java:25-38,
+//     K/AccumWeightedValue.java restated as in k_battn), a query seeing the keys up to its own position.
+// The waves of the workgroup take every WAVES-th tile of keys and merge their (maximum, sum, values) through LDS.
+// The k index of a product may be permuted if both operands are: lane group g supplies the dimensions 16 u + 4 g + e
+// (one 16-byte load per u) and the keys 4 g + e.
+// grid: (n_heads, 2); 64 * WAVES threads; dynamic LDS: (16 HS + 32 WAVES + 16 WAVES HS) floats.
+template <int HS, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
+{
+    constexpr int U = HS / 16;
+    extern __shared__ __align__(16) float pf_lds[];
+    float *sq = pf_lds;                  // [16 queries][HS]
+    float *wm = pf_lds + 16 * HS;        // [WAVES][16]
+    float *wl = wm + WAVES * 16;         // [WAVES][16]
+    float *wo = wl + WAVES * 16;         // [WAVES][HS][16]
+    const int h = blockIdx.x, qb = blockIdx.y * 16, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    if (qb >= a.nrows) return;
+    const int vrows = min(16, a.nrows - qb);   // (rows past the end repeat the last one: their output is not used)
+    const int pos0 = a.st->pos + qb, kvh = h / a.kv_mul, half = HS / 2;
+    for (int p = tid; p < 16 * half; p += 64 * WAVES) {   // q of the rows: the slices of the product added up, RoPE at the row's position
+        const int r = p / half, idx = p - r * half, b = qb + min(r, vrows - 1);
+        float v0 = 0.0f, v1 = 0.0f;
+#pragma unroll 8
+        for (int s = 0; s < a.slices; s++) {
+            const float2 t = *reinterpret_cast<const float2 *>(a.pq + ((long)s * a.nseq + b) * a.dim + h * HS + 2 * idx);
+            v0 += t.x; v1 += t.y;
+        }
+        const float2 cs = a.rope[(long)(a.st->pos + b) * half + idx];
+        sq[r * HS + 2 * idx] = __fsub_rn(__fmul_rn(v0, cs.x), __fmul_rn(v1, cs.y));
+        sq[r * HS + 2 * idx + 1] = __fadd_rn(__fmul_rn(v0, cs.y), __fmul_rn(v1, cs.x));
+    }
+    __syncthreads();
+    float4 qv[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) qv[u] = *reinterpret_cast<const float4 *>(&sq[c * HS + 16 * u + 4 * g]);
+    const int qpos = pos0 + min(c, vrows - 1), lastkey = pos0 + vrows - 1, ntiles = lastkey / 16 + 1;
+    const float *kc = a.kc + kvh * a.head_stride, *vc = a.vc + kvh * a.head_stride;
+    const long rs = a.row_stride;
+    v4f32 o[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) o[u] = v4f32{0.f, 0.f, 0.f, 0.f};
+    float m = -3.0e38f, l = 0.0f;
+    for (int t = wave; t < ntiles; t += WAVES) {
+        const int k0 = t * 16;
+        const float *krow = kc + (long)min(k0 + c, lastkey) * rs + 4 * g;   // (past the last key: that key again, left out below)
+        float4 kf[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) kf[u] = *reinterpret_cast<const float4 *>(krow + 16 * u);
+        v4f32 st = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[u].x, qv[u].x, st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[u].y, qv[u].y, st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[u].z, qv[u].z, st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[u].w, qv[u].w, st, 0, 0, 0);
+        }
+        float sv[4], tmax = -3.0e38f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            sv[e] = k0 + 4 * g + e <= qpos ? __fdiv_rn(st[e], a.sqrt_hs) : -3.0e38f;   // (a query sees the keys up to its own position)
+            tmax = fmaxf(tmax, sv[e]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float mb = fmaxf(m, tmax), sc = expf(m - mb);
+        float pr[4];
+        l *= sc;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            pr[e] = k0 + 4 * g + e <= qpos ? expf(sv[e] - mb) : 0.0f;
+            l += pr[e];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) o[u] *= sc;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float *vrow = vc + (long)min(k0 + 4 * g + e, lastkey) * rs + c;
+#pragma unroll
+            for (int u = 0; u < U; u++) o[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(vrow[16 * u], pr[e], o[u], 0, 0, 0);
+        }
+        m = mb;
+    }
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    if (g == 0) { wm[wave * 16 + c] = m; wl[wave * 16 + c] = l; }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) wo[((wave * HS) + 16 * u + 4 * g + e) * 16 + c] = o[u][e];
+    __syncthreads();
+    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // the waves' parts of a query merged
+        const int q = idx / HS, d = idx - q * HS;
+        float M = wm[q];
+#pragma unroll
+        for (int w = 1; w < WAVES; w++) M = fmaxf(M, wm[w * 16 + q]);
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) {
+            const float wt = expf(wm[w * 16 + q] - M);   // a wave without a tile has m = -3e38: weight 0
+            L += wt * wl[w * 16 + q];
+            O += wt * wo[(w * HS + d) * 16 + q];
+        }
+        if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + d] = __fdiv_rn(O, L);
+    }
+}
+
 // y[0..rows) = row `row` of the product whose slices lie in part, (slices, nseq, rows)
 static __global__ void __launch_bounds__(256) k_brow(const float *__restrict__ part, float *__restrict__ y, int rows, int slices, int nseq, int row)
 {

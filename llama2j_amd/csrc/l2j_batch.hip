@@ -311,10 +311,14 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
 }
 
 
+constexpr int kPflashFrom = 640;   // (measured at the 7B shape: the two kernels take the same time around position 600)
+
+size_t pflash_lds(int hs, int waves) { return (size_t)(16 * hs + 32 * waves + 16 * waves * hs) * sizeof(float); }
+
 // The forward passes of `rows` consecutive positions of one sequence (st: their tokens and the first position) as one batched
 // step into the context's own KV cache: launch_batch_step's kernels, the attention as two launches (every position stores
 // its k and v, then every position attends over the rows up to its own), and the classifier only when `last_logits`.
-void launch_prefill_block(l2j_ctx *c, BatchBufs &b, const BatchState *st, int rows, bool last_logits)
+void launch_prefill_block(l2j_ctx *c, BatchBufs &b, const BatchState *st, int first_pos, int rows, bool last_logits)
 {
     const l2j_config &cf = c->cfg;
     const int dim = cf.dim, hidden = cf.hidden_dim, L = cf.n_layers, hs = c->head_size, kvd = c->kv_dim, nseq = kMaxBatch;
@@ -330,17 +334,23 @@ void launch_prefill_block(l2j_ctx *c, BatchBufs &b, const BatchState *st, int ro
         t.seq_stride = 0; t.cap = cf.seq_len; t.out = b.xb; t.st = st;
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
-        t.head_stride = hs; t.row_stride = kvd; t.nrows = rows;
-        const dim3 ag(cf.n_heads, nseq);
+        t.head_stride = hs; t.row_stride = kvd; t.nrows = rows; t.nseq = nseq;
+        const dim3 ag(cf.n_heads, nseq), fg(cf.n_heads, 2);
+        // 16 positions at a time on the fp32 matrix cores from where that is the faster way (a fixed cost of 18 us against
+        // 6, then 0.013 us per position against 0.068: every cache row fetched once per 16 queries instead of once per query)
+        const bool flash = c->opt[OPT_PREFILL_FLASH] == 2 || (c->opt[OPT_PREFILL_FLASH] == 1 && first_pos >= kPflashFrom);
         if (hs == 64) {
             hipLaunchKernelGGL((k_battn<16, 1>), ag, dim3(256), 0, s, t);
-            hipLaunchKernelGGL((k_battn<16, 2>), ag, dim3(256), 0, s, t);
+            if (flash) hipLaunchKernelGGL((k_pflash<64, 16>), fg, dim3(1024), pflash_lds(64, 16), s, t);
+            else hipLaunchKernelGGL((k_battn<16, 2>), ag, dim3(256), 0, s, t);
         } else if (hs == 128) {
             hipLaunchKernelGGL((k_battn<32, 1>), ag, dim3(256), 0, s, t);
-            hipLaunchKernelGGL((k_battn<32, 2>), ag, dim3(256), 0, s, t);
+            if (flash) hipLaunchKernelGGL((k_pflash<128, 16>), fg, dim3(1024), pflash_lds(128, 16), s, t);
+            else hipLaunchKernelGGL((k_battn<32, 2>), ag, dim3(256), 0, s, t);
         } else {
             hipLaunchKernelGGL((k_battn<64, 1>), ag, dim3(256), 0, s, t);
-            hipLaunchKernelGGL((k_battn<64, 2>), ag, dim3(256), 0, s, t);
+            if (flash) hipLaunchKernelGGL((k_pflash<256, 8>), fg, dim3(512), pflash_lds(256, 8), s, t);
+            else hipLaunchKernelGGL((k_battn<64, 2>), ag, dim3(256), 0, s, t);
         }
         launch_bgemm(c, {L2J_WO}, l, b.xb, b.part, nseq);
         hipLaunchKernelGGL(k_bres_rms, dim3(nseq), dim3(1024), 0, s, b.part[0], sd, b.x, c->rmsw + (size_t)(L + l) * dim, b.xn, dim);
@@ -550,6 +560,12 @@ int l2j::prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t
     int rc = c->batch && c->batch->nseq == kMaxBatch ? L2J_OK : ensure_batch(c, kMaxBatch, 1, 1);
     if (rc) return rc;
     BatchBufs &b = *c->batch;
+    if (!c->pflash_ready) {   // (more than the default 64 KB of dynamic LDS)
+        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<64, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(64, 16)));
+        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<128, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(128, 16)));
+        HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<256, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(256, 8)));
+        c->pflash_ready = true;
+    }
     const int nblocks = (n + kMaxBatch - 1) / kMaxBatch;
     std::vector<BatchState> hst((size_t)nblocks);
     for (int k = 0; k < nblocks; k++) {
@@ -564,7 +580,7 @@ int l2j::prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t
     if (e == hipSuccess) e = hipStreamSynchronize(c->stream);   // (hst is pageable host memory)
     if (e == hipSuccess) e = hipEventRecord(b.e0, c->stream);
     for (int k = 0; k < nblocks && e == hipSuccess; k++) {
-        launch_prefill_block(c, b, dst + k, std::min(kMaxBatch, n - k * kMaxBatch), k + 1 == nblocks);
+        launch_prefill_block(c, b, dst + k, pos0 + k * kMaxBatch, std::min(kMaxBatch, n - k * kMaxBatch), k + 1 == nblocks);
         e = hipGetLastError();
     }
     if (e == hipSuccess) e = hipEventRecord(b.e1, c->stream);

@@ -31,11 +31,13 @@ def caches(g, shape):
     return [np.stack([g.read(which, layer) for layer in range(shape[2])]) for which in (BUFFER.KCACHE, BUFFER.VCACHE)]
 
 
+@pytest.mark.parametrize("flash", [2, 0])    # the attention on the matrix cores at every position / at none (default: from position 640 on)
 @pytest.mark.parametrize("shape", SHAPES)
-def test_prefill_leaves_what_forward_position_by_position_leaves(orc, shape):
+def test_prefill_leaves_what_forward_position_by_position_leaves(orc, shape, flash):
     seq_len, kvd = shape[6], shape[0] // shape[3] * shape[4]
     rng = np.random.default_rng(shape[0] + shape[6])
     g = model(shape)
+    g.set_option("prefill_flash", flash)
     m = oracle_of(orc, shape, 9)
     for n in (1, 31, 32, 33, seq_len):
         tokens = np.concatenate([[1], rng.integers(2, shape[5], size=n - 1)]).astype(np.int32)   # BOS first (J/Run.java:612)
@@ -139,6 +141,7 @@ def test_prefill_at_the_published_widths(orc, shape, n):
     g = l2j.Transformer(l2j.Config(*shape))
     g.fill_synthetic(21, 0.02)
     g.finalize()
+    g.set_option("prefill_flash", 2)
     tokens = np.concatenate([[1], rng.integers(2, shape[5], size=n - 1)]).astype(np.int32)
     for i, t in enumerate(tokens):
         want = g.forward(int(t), i)
@@ -172,3 +175,26 @@ def test_prefill_and_the_batched_decode_share_their_buffers(orc):
     g.reset()
     third, _ = g.prefill(tokens)                                          # (in the buffers of the 32 sequences)
     assert np.array_equal(third.view(np.uint32), alone_logits.view(np.uint32))
+
+
+def test_prefill_past_the_position_where_the_attention_changes_kernels(orc):
+    """By default the attention of a step runs on the matrix cores from position 640 on: a prompt that crosses it, against
+    position-by-position forwards and the oracle."""
+    shape = (512, 1024, 2, 8, 2, 1008, 720, 0)
+    rng = np.random.default_rng(640)
+    g = model(shape)
+    n = 700
+    tokens = np.concatenate([[1], rng.integers(2, shape[5], size=n - 1)]).astype(np.int32)
+    for i, t in enumerate(tokens):
+        want = g.forward(int(t), i)
+    want_k, want_v = caches(g, shape)
+    g.reset()
+    got, _ = g.prefill(tokens)
+    got_k, got_v = caches(g, shape)
+    assert rel_err(got, want.astype(np.float64)) < CLOSE
+    assert rel_err(got_k, want_k.astype(np.float64)) < CLOSE and rel_err(got_v, want_v.astype(np.float64)) < CLOSE
+    m = oracle_of(orc, shape, 9)
+    for i, t in enumerate(tokens):
+        cpu = m.forward(int(t), i)
+    assert rel_err(got, cpu.astype(np.float64)) < LOGIT_TOL
+    m.close()
