@@ -100,7 +100,7 @@ int l2j_device_count(void);
  * positions one by one, as the reference does; 1: the first whole steps of 32 prompt positions go through l2j_prefill, the
  * loop goes on behind them: the same tokens but where two logits lie within rounding of each other; shapes l2j_prefill
  * does not take run as with 0), "prefill_flash" (the attention of l2j_prefill's steps: 1, the default: 16 positions at a time on
- * the fp32 matrix cores from position 640 on, where that is the faster form, every position for itself below; 2: always;
+ * the fp32 matrix cores from position 384 on, where that is the faster form, every position for itself below; 2: always;
  * 0: never).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */

@@ -311,7 +311,7 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
 }
 
 
-constexpr int kPflashFrom = 640;   // (measured at the 7B shape: the two kernels take the same time around position 600)
+constexpr int kPflashFrom = 384;   // (measured at the 7B shape, kernel trace: 28 us against 30 at position 320, 37 against 31 at 448)
 
 size_t pflash_lds(int hs, int waves) { return (size_t)(16 * hs + 32 * waves + 16 * waves * hs) * sizeof(float); }
 

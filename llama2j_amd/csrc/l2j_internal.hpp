@@ -85,7 +85,7 @@ inline const OptionDef kOptions[OPT_COUNT] = {
     {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
     {"batch_fuse", 0, true},           // batched decode: 1: the layers of a step in one launch with grid barriers (slower, measured); 0: eight launches per layer
     {"sampler_wide", 1, true},         // sampling step: 1: one launch over many workgroups (vocabularies that fit in LDS), 0: one launch per stage
-    {"prefill_flash", 1, true},        // l2j_prefill's attention: 1: 16 positions at a time on the fp32 matrix cores from position 640 on, every position for itself before; 2: always; 0: never
+    {"prefill_flash", 1, true},        // l2j_prefill's attention: 1: 16 positions at a time on the fp32 matrix cores from position 384 on, every position for itself before; 2: always; 0: never
     {"prefill", 0, true},              // decode loops: 1: the prompt positions 32 at a time through the batched products (l2j_prefill), 0: one by one as the reference
 };
 

@@ -31,7 +31,7 @@ def caches(g, shape):
     return [np.stack([g.read(which, layer) for layer in range(shape[2])]) for which in (BUFFER.KCACHE, BUFFER.VCACHE)]
 
 
-@pytest.mark.parametrize("flash", [2, 0])    # the attention on the matrix cores at every position / at none (default: from position 640 on)
+@pytest.mark.parametrize("flash", [2, 0])    # the attention on the matrix cores at every position / at none (default: from position 384 on)
 @pytest.mark.parametrize("shape", SHAPES)
 def test_prefill_leaves_what_forward_position_by_position_leaves(orc, shape, flash):
     seq_len, kvd = shape[6], shape[0] // shape[3] * shape[4]
@@ -178,12 +178,12 @@ def test_prefill_and_the_batched_decode_share_their_buffers(orc):
 
 
 def test_prefill_past_the_position_where_the_attention_changes_kernels(orc):
-    """By default the attention of a step runs on the matrix cores from position 640 on: a prompt that crosses it, against
+    """By default the attention of a step runs on the matrix cores from position 384 on: a prompt that crosses it, against
     position-by-position forwards and the oracle."""
-    shape = (512, 1024, 2, 8, 2, 1008, 720, 0)
+    shape = (512, 1024, 2, 8, 2, 1008, 480, 0)
     rng = np.random.default_rng(640)
     g = model(shape)
-    n = 700
+    n = 470
     tokens = np.concatenate([[1], rng.integers(2, shape[5], size=n - 1)]).astype(np.int32)
     for i, t in enumerate(tokens):
         want = g.forward(int(t), i)
