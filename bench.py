@@ -255,6 +255,8 @@ def main():
             runs = {}
             for n_seq in (() if a.prefill_only else (32, 16)):
                 prompts = [prompt] + [synth_prompt(seed + 1000 + b, n_prompt, shape[5]) for b in range(1, n_seq)]
+                if n_seq == 32:
+                    prompts32 = prompts
                 g.decode_greedy_batch(prompts, min(bsteps, 8), n_seq=n_seq)          # warm
                 btoks, bsec = g.decode_greedy_batch(prompts, bsteps, n_seq=n_seq)
                 per = bsec / (bsteps - 1)
@@ -265,6 +267,12 @@ def main():
                                             "note": "weights once + every sequence's KV cache rows at the mean position, over the whole step time"},
                                "sequence_0_equals_the_single_decode": bool(np.array_equal(btoks[0, :n0], tokens[:n0]))}
             if runs:
+                try:   # the same 32 loops with a sampler each, at the reference's default temperature and top-p (J/CommandLine.java:24-25)
+                    stoks32, ssec32 = g.decode_sample_batch(prompts32, bsteps, 0.9, 0.9, np.arange(32, dtype=np.int64) + seed, n_seq=32)
+                    runs[32]["sampled"] = {"temperature": 0.9, "topp": 0.9, "tok_s": round(32 * (bsteps - 1) / ssec32, 1),
+                                           "ms_per_step": round(ssec32 / (bsteps - 1) * 1e3, 4)}
+                except l2j.L2JError as e:   # a vocabulary above the one-launch sampling step's
+                    runs[32]["sampled"] = {"error": str(e)}
                 out["batched_decode"] = runs[32]
                 out["batched_decode"]["sixteen_sequences"] = {k: runs[16][k] for k in ("tok_s", "ms_per_step", "sequence_0_equals_the_single_decode")}
         except l2j.L2JError as e:  # shapes the batched path does not take (rows that are not whole groups of 256)

@@ -187,6 +187,16 @@ int l2j_sample(l2j_ctx *ctx, const float *logits_or_null, float temperature, flo
  * unforced token is sampled as in l2j_sample from a sampler seeded with rng_seed; the logits never leave the device. */
 int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int32_t steps, float temperature,
                       float topp, int64_t rng_seed, int32_t *out_tokens, int32_t *n_out, double *seconds);
+/* l2j_decode_greedy_batch with a sampler per sequence: sequence s owns a new Sampler(rng_seeds[s], vocab_size) and every
+ * unforced token of it is sampled as in l2j_sample (temperature 0: the argmax, no sampler is made), i.e. n_seq runs of the
+ * loop of l2j_decode_sample side by side; the reference has neither ("parallel processing of multiple queries" is on its
+ * wish-list, README.md:347).  The sampling steps are those of the single sequence, one launch per sequence and step, after
+ * the step's forward pass; they need the one-launch step (vocab_size <= 36864, options "sampler_wide" and "sampler_scan"
+ * on: else L2J_E_STATE).  The context's own sampler is not touched.  logits (may be NULL): as in
+ * l2j_decode_greedy_batch_logits, the logits of every step before sampling, (steps, n_seq, vocab_size) floats. */
+int l2j_decode_sample_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,
+                            int32_t prompt_stride, int32_t steps, float temperature, float topp, const int64_t *rng_seeds,
+                            int32_t *out_tokens, double *seconds, float *logits);
 
 /* ---- tokenizer: J/Tokenizer.java (host only) ----
  * Strings cross the boundary as NUL-terminated UTF-8; inside, comparisons are on UTF-16 code units as in Java. */

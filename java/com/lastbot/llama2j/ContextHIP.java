@@ -40,7 +40,7 @@ public final class ContextHIP implements AutoCloseable {
     // buffers of the token loop's thread, allocated once (no allocation per token)
     private final MemorySegment logitsSeg, intSeg, tokensSeg, promptSeg, countSeg, secondsSeg;
     private final MethodHandle lastError, ctxLastError, destroy, setOption, uploadQuant, uploadF32, finalizeH, reset, forward,
-            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSample, samplerSeed, sample, prefill;
+            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSampleBatch, decodeSample, samplerSeed, sample, prefill;
 
     private MethodHandle handle(String name, FunctionDescriptor fd) {
         return LINKER.downcallHandle(lib.find(name).orElseThrow(), fd);
@@ -62,6 +62,8 @@ public final class ContextHIP implements AutoCloseable {
                 FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS));
         decodeGreedyBatch = handle("l2j_decode_greedy_batch",
                 FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
+        decodeSampleBatch = handle("l2j_decode_sample_batch", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
+                JAVA_INT, JAVA_FLOAT, JAVA_FLOAT, ADDRESS, ADDRESS, ADDRESS, ADDRESS));
         decodeSample = handle("l2j_decode_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
                 JAVA_FLOAT, JAVA_FLOAT, JAVA_LONG, ADDRESS, ADDRESS, ADDRESS));
         samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
@@ -238,6 +240,15 @@ public final class ContextHIP implements AutoCloseable {
      * counterpart in the reference.
      */
     public int[][] decodeGreedyBatch(int[][] prompts, int steps) {
+        return decodeSampleBatch(prompts, steps, 0.0f, 0.0f, null);
+    }
+
+    /**
+     * decodeGreedyBatch with a Sampler(rngSeeds[b], vocab_size) per sequence on the device (l2j_decode_sample_batch):
+     * the unforced tokens of sequence b are sampled as decodeSample samples them.  Temperature 0 (rngSeeds may then be
+     * null): the greedy loops.
+     */
+    public int[][] decodeSampleBatch(int[][] prompts, int steps, float temperature, float topp, long[] rngSeeds) {
         if (prompts.length > 32) throw new IllegalArgumentException("at most 32 sequences");
         final int batch = prompts.length <= 16 ? 16 : 32;
         int stride = 1;
@@ -250,7 +261,14 @@ public final class ContextHIP implements AutoCloseable {
                 MemorySegment.copy(prompts[b], 0, ids, JAVA_INT, (long) b * stride * Integer.BYTES, prompts[b].length);
                 counts.setAtIndex(JAVA_INT, b, prompts[b].length);
             }
-            check(call(decodeGreedyBatch, ctx, ids, counts, batch, stride, steps, out, secondsSeg));
+            if (temperature == 0.0f) {
+                check(call(decodeGreedyBatch, ctx, ids, counts, batch, stride, steps, out, secondsSeg));
+            } else {
+                MemorySegment seeds = a.allocate((long) batch * Long.BYTES, 16);
+                for (int b = 0; b < batch; b++) seeds.setAtIndex(JAVA_LONG, b, b < rngSeeds.length ? rngSeeds[b] : 0L);
+                check(call(decodeSampleBatch, ctx, ids, counts, batch, stride, steps, temperature, topp, seeds, out, secondsSeg,
+                        MemorySegment.NULL));
+            }
             int[][] tokens = new int[batch][steps];
             for (int b = 0; b < batch; b++) MemorySegment.copy(out, JAVA_INT, (long) b * steps * Integer.BYTES, tokens[b], 0, steps);
             return tokens;

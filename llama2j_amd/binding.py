@@ -118,6 +118,8 @@ def _signatures():
         "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
         "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
         "l2j_decode_greedy_batch_logits": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, fp]),
+        "l2j_decode_sample_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_float,
+                                              C.POINTER(C.c_int64), i32p, C.POINTER(C.c_double), fp]),
         "l2j_batch_matmul": (C.c_int, [vp, C.c_int, C.c_int, fp, fp, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
         "l2j_bytes_per_token": (C.c_uint64, [cfgp, C.c_int32]),
         "l2j_quant_nbytes": (C.c_uint64, [C.c_uint64]),
@@ -455,6 +457,29 @@ class Transformer:
         sec = C.c_double(0.0)
         self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), C.byref(sec)))
         return out, sec.value
+
+    def decode_sample_batch(self, prompts, steps, temperature, topp, rng_seeds, n_seq=None, want_logits=False):
+        """decode_greedy_batch with a sampler per sequence (l2j_decode_sample_batch): sequence b samples its unforced
+        tokens from a sampler seeded with rng_seeds[b].  Returns (tokens, seconds after the first step), with want_logits
+        (tokens, seconds, logits of every step before sampling, of shape (steps, n_seq, vocab_size))."""
+        if n_seq is None:
+            n_seq = 16 if len(prompts) <= 16 else 32
+        assert len(prompts) <= n_seq
+        seeds = np.zeros(n_seq, dtype=np.int64)
+        seeds[:len(rng_seeds)] = rng_seeds
+        stride = max([len(p) for p in prompts] + [1])
+        ids = np.zeros((n_seq, stride), dtype=np.int32)
+        n = np.zeros(n_seq, dtype=np.int32)
+        for b, p in enumerate(prompts):
+            ids[b, :len(p)] = p
+            n[b] = len(p)
+        out = np.zeros((n_seq, steps), dtype=np.int32)
+        logits = np.empty((steps, n_seq, self.config.vocab_size), dtype=np.float32) if want_logits else None
+        sec = C.c_double(0.0)
+        self._check(lib().l2j_decode_sample_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, temperature, topp,
+                                                  seeds.ctypes.data_as(C.POINTER(C.c_int64)), _i32(out), C.byref(sec),
+                                                  _fp(logits) if want_logits else None))
+        return (out, sec.value, logits) if want_logits else (out, sec.value)
 
     def batch_matmul(self, tensor, layer, x, rows, groups_per_slice=2, rounds=1):
         """y[b] = W x[b] for sixteen activation vectors against one layer's matrix of a quantized tensor, by the

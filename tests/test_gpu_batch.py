@@ -226,3 +226,60 @@ def test_sequence_counts_other_than_16_and_32_are_an_error():
             g.decode_greedy_batch([np.array([5], dtype=np.int32)], 4, n_seq=n_seq)
         assert e.value.code == -1
     g.close()
+
+
+@pytest.mark.parametrize("n_seq,t,topp,vocab", [(16, 0.9, 0.9, 1008), (32, 1.0, 1.0, 1008), (32, 1.3, 0.6, 1008), (32, 1.0, 0.9, 32000),
+                                                (16, 0.7, 1.0, 32000)])
+def test_sampled_batch_gives_every_sequence_its_own_sampler(orc, n_seq, t, topp, vocab):
+    """l2j_decode_sample_batch: sequence b must get what the reference's loop with a Sampler(seed b) gives it (J/Run.java:623-685,
+    J/Sampler.java).  The oracle's sampler is fed the batched path's own logits of every step (they agree with the oracle's
+    forward pass to rounding only, and a draw within that of a step of the cumulative sum would part two correct runs):
+    every token identical; and the logits of a step must be those of the tokens sampled before it, which the
+    single-sequence forward pass, fed the sampled tokens, confirms."""
+    from tests.test_gpu_parity import make_pair
+    shape = SHAPES[0][:5] + (vocab,) + SHAPES[0][6:]    # (32000: a sampling step takes 125 compute units, two of them run side by side)
+    m, g = make_pair(orc, shape, seed=17, realistic=True)
+    rng = np.random.default_rng(n_seq)
+    steps = 28 if vocab < 10000 else 14
+    prompts = [rng.integers(3, vocab, size=int(rng.integers(0, 7))).astype(np.int32) for _ in range(n_seq - 2)]   # (two run without one)
+    seeds = rng.integers(-2**40, 2**40, size=n_seq).astype(np.int64)
+    got, sec, logits = g.decode_sample_batch(prompts, steps, t, topp, seeds, n_seq=n_seq, want_logits=True)
+    assert got.shape == (n_seq, steps) and sec > 0
+    for b in range(n_seq):
+        prompt = prompts[b] if b < len(prompts) else np.zeros(0, dtype=np.int32)
+        s = orc.Sampler(int(seeds[b]), vocab)
+        want = [int(prompt[pos]) if pos < len(prompt) else s.step(logits[pos, b], t, topp)[0] for pos in range(steps)]
+        np.testing.assert_array_equal(got[b], np.array(want, dtype=np.int32), err_msg="sequence %d" % b)
+    for b in (0, n_seq - 1):                                     # the sampled tokens are what the next step reads
+        g.reset()
+        tok = 1
+        for pos in range(steps):
+            lg = g.forward(tok, pos)
+            assert rel_err(logits[pos, b], lg.astype(np.float64)) < 1e-5, (b, pos)
+            tok = int(got[b, pos])
+    again, _ = g.decode_sample_batch(prompts, steps, t, topp, seeds, n_seq=n_seq)      # the seeds restart generators and arrays
+    np.testing.assert_array_equal(again, got)
+    other, _ = g.decode_sample_batch(prompts, steps, t, topp, seeds + 1, n_seq=n_seq)
+    assert not np.array_equal(other, got)
+    greedy, _ = g.decode_greedy_batch(prompts, steps, n_seq=n_seq)
+    cold, _ = g.decode_sample_batch(prompts, steps, 0.0, topp, seeds, n_seq=n_seq)     # temperature 0: Sampler.argmax
+    np.testing.assert_array_equal(cold, greedy)
+    g.close()
+
+
+def test_sampled_batch_refuses_what_the_one_launch_sampler_cannot_take():
+    g = l2j.Transformer(l2j.Config(*SHAPES[3]))
+    g.fill_synthetic(3, 0.02)
+    g.finalize()
+    p = [np.array([5, 6], dtype=np.int32)]
+    with pytest.raises(L2JError):
+        g.decode_sample_batch(p, 8, -1.0, 0.9, [1])
+    with pytest.raises(L2JError):
+        g.decode_sample_batch(p, 8, 1.0, 1.5, [1])
+    g.set_option("sampler_wide", 0)
+    with pytest.raises(L2JError, match="one-launch"):
+        g.decode_sample_batch(p, 8, 1.0, 0.9, [1])
+    g.set_option("sampler_wide", 1)
+    out, _ = g.decode_sample_batch(p, 8, 1.0, 0.9, [1])
+    assert out.shape == (16, 8) and np.array_equal(out[0, :2], p[0])
+    g.close()
