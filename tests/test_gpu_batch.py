@@ -283,3 +283,21 @@ def test_sampled_batch_refuses_what_the_one_launch_sampler_cannot_take():
     out, _ = g.decode_sample_batch(p, 8, 1.0, 0.9, [1])
     assert out.shape == (16, 8) and np.array_equal(out[0, :2], p[0])
     g.close()
+
+
+def test_a_wait_of_a_sampling_step_that_runs_out_fails_the_sampled_batch_and_nothing_else():
+    """barrier_spins 0: the first workgroup to reach a grid barrier of a sampling step gives up at once (every kernel still runs
+    to its end).  The call is an error; the greedy loops, which have no such wait, go on giving what they gave."""
+    shape = SHAPES[0]
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(5, 0.02)
+    g.set_option("barrier_spins", 0)
+    g.finalize()
+    p = [np.array([9, 8, 7], dtype=np.int32)]
+    before, _ = g.decode_greedy_batch(p, 12)
+    for _ in range(2):   # (the second call finds the step's counters cleared)
+        with pytest.raises(L2JError, match="waited too long"):
+            g.decode_sample_batch(p, 12, 1.0, 0.9, [3])
+    after, _ = g.decode_greedy_batch(p, 12)
+    np.testing.assert_array_equal(after, before)
+    g.close()
