@@ -100,8 +100,9 @@ int l2j_device_count(void);
  * positions one by one, as the reference does; 1: the first whole steps of 32 prompt positions go through l2j_prefill, the
  * loop goes on behind them: the same tokens but where two logits lie within rounding of each other; shapes l2j_prefill
  * does not take run as with 0), "prefill_flash" (the attention of l2j_prefill's steps: 1, the default: 16 positions at a time on
- * the fp32 matrix cores from position 384 on, where that is the faster form, every position for itself below; 2: always;
- * 0: never).  l2j_get_option reads the value in force
+ * the fp32 matrix cores from position 64 on, where that is the faster form, every position for itself below; 2: always;
+ * 0: never), "prefill_split" (workgroups that share the keys of a head and 16 positions there: 1 to 4; 0, the default:
+ * one below position 192, then as many of up to four as the GPU has compute units for).  l2j_get_option reads the value in force
  * ("fuse" reads 0 after such a switch; "wall_clock_khz", read-only: the rate of the device clock that l2j_decode_greedy
  * times itself with, 0 when the device does not tell it). */
 int l2j_set_option(l2j_ctx *ctx, const char *name, int32_t value);

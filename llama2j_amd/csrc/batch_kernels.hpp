@@ -567,6 +567,9 @@ struct BAttn {
     int row_stride;              // and between two positions
     int nrows;                   // rows in use: the others neither store nor attend
     int nseq;                    // rows of the products' partial sums (k_pflash; k_battn has them as its grid)
+    // k_pflash with the keys of a (head, 16 queries) pair split over gridDim.z workgroups:
+    float *pf_part;              // (head, half, z) x (16 maxima, 16 sums, 16 x head_size values): what each leaves for the last one
+    unsigned *pf_cnt;            // (head, half): how many have; zero between launches
 };
 
 // Attention of one head of one sequence over positions 0..pos (K/AttentionLoop.java:29-54, K/ExpSumNormalize.java:25-38,
@@ -761,7 +764,8 @@ static __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *
 // The waves of the workgroup take every WAVES-th tile of keys and merge their (maximum, sum, values) through LDS.
 // The k index of a product may be permuted if both operands are: lane group g supplies the dimensions 16 u + 4 g + e
 // (one 16-byte load per u) and the keys 4 g + e.
-// grid: (n_heads, 2); 64 * WAVES threads; dynamic LDS: (16 HS + 32 WAVES + 16 WAVES HS) floats.
+// grid: (n_heads, 2, 1..4): z splits the tiles of keys over that many workgroups, the last of which to finish merges what the
+// others left in device memory.  64 * WAVES threads; dynamic LDS: (16 HS + 32 WAVES + 16 WAVES HS) floats.
 template <int HS, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
 {
@@ -771,6 +775,8 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     float *wm = pf_lds + 16 * HS;        // [WAVES][16]
     float *wl = wm + WAVES * 16;         // [WAVES][16]
     float *wo = wl + WAVES * 16;         // [WAVES][HS][16]
+    __shared__ float ww[WAVES * 16], wM[16];
+    __shared__ int s_last;
     const int h = blockIdx.x, qb = blockIdx.y * 16, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
     if (qb >= a.nrows) return;
@@ -799,7 +805,11 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
 #pragma unroll
     for (int u = 0; u < U; u++) o[u] = v4f32{0.f, 0.f, 0.f, 0.f};
     float m = -3.0e38f, l = 0.0f;
-    for (int t = wave; t < ntiles; t += WAVES) {
+    // tile t of the keys goes to workgroup t % NS (z) and there to wave (t / NS) % WAVES: few tiles spread over the workgroups first
+    const int NS = gridDim.z;
+    const int mytiles = (ntiles - (int)blockIdx.z + NS - 1) / NS;   // of this workgroup
+    const int nw = min(WAVES, mytiles);                              // waves that have any
+    for (int t = blockIdx.z + NS * wave; t < ntiles; t += NS * WAVES) {
         const int k0 = t * 16;
         const float *krow = kc + (long)min(k0 + c, lastkey) * rs + 4 * g;   // (past the last key: that key again, left out below)
         float4 kf[U];
@@ -842,24 +852,85 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     if (g == 0) { wm[wave * 16 + c] = m; wl[wave * 16 + c] = l; }
+    if (wave < nw) {   // (the waves without a tile have nothing to add)
 #pragma unroll
-    for (int u = 0; u < U; u++)
+        for (int u = 0; u < U; u++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) wo[((wave * HS) + 16 * u + 4 * g + e) * 16 + c] = o[u][e];
+            for (int e = 0; e < 4; e++) wo[((wave * HS) + 16 * u + 4 * g + e) * 16 + c] = o[u][e];
+    }
     __syncthreads();
-    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // the waves' parts of a query merged
-        const int q = idx / HS, d = idx - q * HS;
+    if (tid < 16 * WAVES) {   // weight of wave w's part in query q's sum: tid = w * 16 + q (a workgroup without any tile leaves
+        const int q = tid & 15;   // maximum -3e38, sum 0 and values 0)
         float M = wm[q];
 #pragma unroll
         for (int w = 1; w < WAVES; w++) M = fmaxf(M, wm[w * 16 + q]);
+        ww[tid] = expf(wm[tid] - M);
+        if (tid < 16) wM[tid] = M;
+    }
+    __syncthreads();
+    if (NS == 1) {
+        for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // the waves' parts of a query merged
+            const int d = idx >> 4, q = idx & 15;   // (neighbouring lanes read neighbouring words of LDS: d * 16 + q = idx)
+            float L = 0.0f, O = 0.0f;
+#pragma unroll
+            for (int w = 0; w < WAVES; w++) {
+                if (w < nw) {
+                    const float wt = ww[w * 16 + q];
+                    L += wt * wl[w * 16 + q];
+                    O += wt * wo[(w * HS + d) * 16 + q];
+                }
+            }
+            if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + d] = __fdiv_rn(O, L);
+        }
+        return;
+    }
+    // The keys are split over NS workgroups: each leaves its maxima, sums and values (not yet divided) in device memory, and
+    // the last one to do so merges them all.
+    constexpr int PER = 32 + 16 * HS;
+    const int pair = h * gridDim.y + blockIdx.y;
+    float *mine = a.pf_part + ((long)pair * NS + blockIdx.z) * PER;
+    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // (values in the order they have in LDS: [dimension][query])
+        const int d = idx >> 4, q = idx & 15;
         float L = 0.0f, O = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) {
-            const float wt = expf(wm[w * 16 + q] - M);   // a wave without a tile has m = -3e38: weight 0
-            L += wt * wl[w * 16 + q];
-            O += wt * wo[(w * HS + d) * 16 + q];
+            if (w < nw) {
+                const float wt = ww[w * 16 + q];
+                L += wt * wl[w * 16 + q];
+                O += wt * wo[(w * HS + d) * 16 + q];
+            }
         }
-        if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + d] = __fdiv_rn(O, L);
+        st_coh(mine + 32 + idx, O);
+        if (d == 0) { st_coh(mine + q, wM[q]); st_coh(mine + 16 + q, L); }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (this thread's stores have arrived where the other workgroups read)
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(a.pf_cnt + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = old + 1u == (unsigned)NS;
+        if (s_last) __hip_atomic_store(a.pf_cnt + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // (for the next launch)
+    }
+    __syncthreads();
+    if (!s_last) return;
+    const float *all = a.pf_part + (long)pair * NS * PER;
+    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {
+        const int q = idx & 15;
+        float mz[4], M = -3.0e38f;
+#pragma unroll
+        for (int z = 0; z < 4; z++) {
+            mz[z] = z < NS ? ld_coh(all + (long)z * PER + q) : -3.0e38f;
+            M = fmaxf(M, mz[z]);
+        }
+        float L = 0.0f, O = 0.0f;
+#pragma unroll
+        for (int z = 0; z < 4; z++) {
+            if (z < NS) {
+                const float wt = expf(mz[z] - M);
+                L += wt * ld_coh(all + (long)z * PER + 16 + q);
+                O += wt * ld_coh(all + (long)z * PER + 32 + idx);
+            }
+        }
+        if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + (idx >> 4)] = __fdiv_rn(O, L);
     }
 }
 

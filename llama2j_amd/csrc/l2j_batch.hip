@@ -136,6 +136,8 @@ struct l2j::BatchBufs {
     size_t pi_stride = 0;
     // two sampling steps run side by side (a step keeps half of the compute units busy): the second one on a stream and in
     // work buffers of its own
+    float *pf_part = nullptr;      // l2j_prefill: what the workgroups that share a head's keys leave for the one that merges,
+    unsigned *pf_cnt = nullptr;    // and how many have (zero between launches)
     SamplerWork side_work;
     hipStream_t side = nullptr;
     hipEvent_t ev_fwd = nullptr, ev_side = nullptr;
@@ -149,7 +151,7 @@ struct l2j::BatchBufs {
         if (e0) (void)hipEventDestroy(e0);
         if (e1) (void)hipEventDestroy(e1);
         void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done, bar_ctr, fault, ssq, step_args,
-                      ss, pi_prob[0], pi_prob[1], pi_idx[0], pi_idx[1]};
+                      ss, pi_prob[0], pi_prob[1], pi_idx[0], pi_idx[1], pf_part, pf_cnt};
         for (void *p : ps) (void)hipFree(p);
         free_sampler_work(&side_work);
         if (side) (void)hipStreamDestroy(side);
@@ -326,7 +328,21 @@ void launch_batch_step(l2j_ctx *c, BatchBufs &b, int max_pos, int prompt_stride,
 }
 
 
-constexpr int kPflashFrom = 384;   // (measured at the 7B shape, kernel trace: 28 us against 30 at position 320, 37 against 31 at 448)
+// Measured at the 7B shape (kernel trace, per launch, a step's first position p): every row for itself (k_battn<LPR, 2>) 6.1 us at
+// p = 0, 8.8 at 32, 11.0 at 64 and 2.1 more per 32 positions; k_pflash in one workgroup per head and half 8.1, 9.7, 11.2 and
+// then 0.6-1 more per 32 positions; with the keys split over four workgroups 12.4 at p = 0, 14.4 at 160, 14.6 at 192, 18.0 at 608.
+constexpr int kPflashFrom = 64;         // k_pflash from this position on
+constexpr int kPflashSplitFrom = 192;   // and the keys of a head split over several workgroups from this one on
+
+constexpr int kPflashMaxSplit = 4;
+// Workgroups per (head, 16 positions): the keys split so that the launch has a workgroup for every compute unit.
+int pflash_split(l2j_ctx *c, int first_pos)
+{
+    const int opt = c->opt[OPT_PREFILL_SPLIT];
+    if (opt <= 0 && first_pos < kPflashSplitFrom) return 1;
+    const int fit = opt > 0 ? opt : c->n_cu / (2 * c->cfg.n_heads);
+    return std::min(kPflashMaxSplit, std::max(1, fit));
+}
 
 size_t pflash_lds(int hs, int waves) { return (size_t)(16 * hs + 32 * waves + 16 * waves * hs) * sizeof(float); }
 
@@ -350,9 +366,10 @@ void launch_prefill_block(l2j_ctx *c, BatchBufs &b, const BatchState *st, int fi
         t.n_heads = cf.n_heads; t.kv_mul = cf.n_heads / cf.n_kv_heads; t.head_size = hs; t.kv_dim = kvd; t.dim = dim;
         t.sqrt_hs = sqrtf((float)hs);
         t.head_stride = hs; t.row_stride = kvd; t.nrows = rows; t.nseq = nseq;
-        const dim3 ag(cf.n_heads, nseq), fg(cf.n_heads, 2);
-        // 16 positions at a time on the fp32 matrix cores from where that is the faster way (a fixed cost of 18 us against
-        // 6, then 0.013 us per position against 0.068: every cache row fetched once per 16 queries instead of once per query)
+        t.pf_part = b.pf_part; t.pf_cnt = b.pf_cnt;
+        const dim3 ag(cf.n_heads, nseq), fg(cf.n_heads, 2, pflash_split(c, first_pos));
+        // 16 positions at a time on the fp32 matrix cores from where that is the faster way: every cache row fetched once per 16
+        // queries instead of once per query
         const bool flash = c->opt[OPT_PREFILL_FLASH] == 2 || (c->opt[OPT_PREFILL_FLASH] == 1 && first_pos >= kPflashFrom);
         if (hs == 64) {
             hipLaunchKernelGGL((k_battn<16, 1>), ag, dim3(256), 0, s, t);
@@ -657,6 +674,12 @@ int l2j::prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<128, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(128, 16)));
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<256, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(256, 8)));
         c->pflash_ready = true;
+    }
+    if (!b.pf_part) {
+        int arc;
+        if ((arc = dev_alloc(&b.pf_part, (uint64_t)cf.n_heads * 2 * kPflashMaxSplit * (32 + 16 * hs)))) return arc;
+        if ((arc = dev_alloc(&b.pf_cnt, (uint64_t)cf.n_heads * 2))) return arc;
+        HIPCHK(hipMemset(b.pf_cnt, 0, (size_t)cf.n_heads * 2 * sizeof(unsigned)));
     }
     const int nblocks = (n + kMaxBatch - 1) / kMaxBatch;
     std::vector<BatchState> hst((size_t)nblocks);

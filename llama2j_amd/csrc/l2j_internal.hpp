@@ -55,7 +55,7 @@ struct QTensor {
 enum {
     OPT_THREADS = 0, OPT_GRID, OPT_ATTN_THREADS, OPT_ATTN_ROWS, OPT_ATTN_NSPLIT, OPT_FUSED_ATTN_ROWS, OPT_FUSED_ATTN_SPLITS,
     OPT_BARRIER_SPINS, OPT_FUSE, OPT_LAYERS_PER_LAUNCH, OPT_BY_VALUE, OPT_TOKEN_SPECIAL, OPT_SAMPLER_SCAN, OPT_SAMPLER_EXP_WGS,
-    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_BATCH_FUSE, OPT_SAMPLER_WIDE, OPT_PREFILL_FLASH, OPT_PREFILL, OPT_COUNT
+    OPT_GRAPH, OPT_SELF_CONTAINED, OPT_GRAPH_TOKENS, OPT_FAST_STEPS, OPT_FALLBACK, OPT_BATCH_FUSE, OPT_SAMPLER_WIDE, OPT_PREFILL_FLASH, OPT_PREFILL, OPT_PREFILL_SPLIT, OPT_COUNT
 };
 constexpr int kAuto = -1;
 struct OptionDef {
@@ -85,8 +85,9 @@ inline const OptionDef kOptions[OPT_COUNT] = {
     {"fallback", 1, true},             // a whole-token kernel whose bounded wait ran out: switch to one launch per phase and repeat
     {"batch_fuse", 0, true},           // batched decode: 1: the layers of a step in one launch with grid barriers (slower, measured); 0: eight launches per layer
     {"sampler_wide", 1, true},         // sampling step: 1: one launch over many workgroups (vocabularies that fit in LDS), 0: one launch per stage
-    {"prefill_flash", 1, true},        // l2j_prefill's attention: 1: 16 positions at a time on the fp32 matrix cores from position 384 on, every position for itself before; 2: always; 0: never
+    {"prefill_flash", 1, true},        // l2j_prefill's attention: 1: 16 positions at a time on the fp32 matrix cores from position 64 on, every position for itself before; 2: always; 0: never
     {"prefill", 0, true},              // decode loops: 1: the prompt positions 32 at a time through the batched products (l2j_prefill), 0: one by one as the reference
+    {"prefill_split", 0, true},        // workgroups that share the keys of one head and 16 positions in that attention: 1..4, 0: one below position 192, then as many as the GPU has compute units for
 };
 
 inline int option_from_env(int i)

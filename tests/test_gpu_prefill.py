@@ -31,7 +31,7 @@ def caches(g, shape):
     return [np.stack([g.read(which, layer) for layer in range(shape[2])]) for which in (BUFFER.KCACHE, BUFFER.VCACHE)]
 
 
-@pytest.mark.parametrize("flash", [2, 0])    # the attention on the matrix cores at every position / at none (default: from position 384 on)
+@pytest.mark.parametrize("flash", [2, 0])    # the attention on the matrix cores at every position / at none (default: from position 64 on)
 @pytest.mark.parametrize("shape", SHAPES)
 def test_prefill_leaves_what_forward_position_by_position_leaves(orc, shape, flash):
     seq_len, kvd = shape[6], shape[0] // shape[3] * shape[4]
@@ -178,8 +178,8 @@ def test_prefill_and_the_batched_decode_share_their_buffers(orc):
 
 
 def test_prefill_past_the_position_where_the_attention_changes_kernels(orc):
-    """By default the attention of a step runs on the matrix cores from position 384 on: a prompt that crosses it, against
-    position-by-position forwards and the oracle."""
+    """By default the attention of a step runs on the matrix cores from position 64 on, and from position 192 on the keys of a
+    head are split over several workgroups: a prompt that crosses both, against position-by-position forwards and the oracle."""
     shape = (512, 1024, 2, 8, 2, 1008, 480, 0)
     rng = np.random.default_rng(640)
     g = model(shape)
@@ -198,3 +198,26 @@ def test_prefill_past_the_position_where_the_attention_changes_kernels(orc):
         cpu = m.forward(int(t), i)
     assert rel_err(got, cpu.astype(np.float64)) < LOGIT_TOL
     m.close()
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_the_keys_of_a_head_split_over_one_to_four_workgroups(shape):
+    """Option prefill_split: as many workgroups share the keys of a head in the matrix-core attention, the last of them to finish
+    merging what the others left (also where there are fewer tiles of 16 keys than workgroups): the logits and cache rows of
+    position-by-position forwards, for every head size, and twice in a row (the counters of a launch are left at zero)."""
+    seq_len = shape[6]
+    rng = np.random.default_rng(seq_len)
+    g = model(shape)
+    g.set_option("prefill_flash", 2)
+    tokens = np.concatenate([[1], rng.integers(2, shape[5], size=seq_len - 1)]).astype(np.int32)
+    for i, t in enumerate(tokens):
+        want = g.forward(int(t), i)
+    want_k, want_v = caches(g, shape)
+    for split in (4, 3, 2, 1, 4):
+        g.set_option("prefill_split", split)
+        g.reset()
+        got, _ = g.prefill(tokens)
+        got_k, got_v = caches(g, shape)
+        assert rel_err(got, want.astype(np.float64)) < CLOSE, split
+        assert rel_err(got_k, want_k.astype(np.float64)) < CLOSE and rel_err(got_v, want_v.astype(np.float64)) < CLOSE, split
+    g.close()
