@@ -774,7 +774,7 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     float *sq = pf_lds;                  // [16 queries][HS]
     float *wm = pf_lds + 16 * HS;        // [WAVES][16]
     float *wl = wm + WAVES * 16;         // [WAVES][16]
-    float *wo = wl + WAVES * 16;         // [WAVES][HS][16]
+    float *wo = wl + WAVES * 16;         // [WAVES][HS / 4][16 queries][4]: dimension d of query q at (d / 4) * 64 + 4 q + d % 4
     __shared__ float ww[WAVES * 16], wM[16];
     __shared__ int s_last;
     const int h = blockIdx.x, qb = blockIdx.y * 16, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -854,9 +854,8 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     if (g == 0) { wm[wave * 16 + c] = m; wl[wave * 16 + c] = l; }
     if (wave < nw) {   // (the waves without a tile have nothing to add)
 #pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) wo[((wave * HS) + 16 * u + 4 * g + e) * 16 + c] = o[u][e];
+        for (int u = 0; u < U; u++)   // (a lane's four dimensions 16 u + 4 g + e of query c as one 16-byte store, a wave's stores 1 KB in a row)
+            *reinterpret_cast<v4f32 *>(&wo[wave * HS * 16 + (4 * u + g) * 64 + 4 * c]) = o[u];
     }
     __syncthreads();
     if (tid < 16 * WAVES) {   // weight of wave w's part in query q's sum: tid = w * 16 + q (a workgroup without any tile leaves
@@ -870,14 +869,14 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     __syncthreads();
     if (NS == 1) {
         for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // the waves' parts of a query merged
-            const int d = idx >> 4, q = idx & 15;   // (neighbouring lanes read neighbouring words of LDS: d * 16 + q = idx)
+            const int d = (idx >> 6) * 4 + (idx & 3), q = (idx >> 2) & 15;   // (neighbouring lanes read neighbouring words of LDS)
             float L = 0.0f, O = 0.0f;
 #pragma unroll
             for (int w = 0; w < WAVES; w++) {
                 if (w < nw) {
                     const float wt = ww[w * 16 + q];
                     L += wt * wl[w * 16 + q];
-                    O += wt * wo[(w * HS + d) * 16 + q];
+                    O += wt * wo[w * HS * 16 + idx];
                 }
             }
             if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + d] = __fdiv_rn(O, L);
@@ -889,15 +888,15 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     constexpr int PER = 32 + 16 * HS;
     const int pair = h * gridDim.y + blockIdx.y;
     float *mine = a.pf_part + ((long)pair * NS + blockIdx.z) * PER;
-    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // (values in the order they have in LDS: [dimension][query])
-        const int d = idx >> 4, q = idx & 15;
+    for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {   // (values in the order they have in LDS)
+        const int d = (idx >> 6) * 4 + (idx & 3), q = (idx >> 2) & 15;
         float L = 0.0f, O = 0.0f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) {
             if (w < nw) {
                 const float wt = ww[w * 16 + q];
                 L += wt * wl[w * 16 + q];
-                O += wt * wo[(w * HS + d) * 16 + q];
+                O += wt * wo[w * HS * 16 + idx];
             }
         }
         st_coh(mine + 32 + idx, O);
@@ -914,7 +913,7 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
     if (!s_last) return;
     const float *all = a.pf_part + (long)pair * NS * PER;
     for (int idx = tid; idx < HS * 16; idx += 64 * WAVES) {
-        const int q = idx & 15;
+        const int q = (idx >> 2) & 15;
         float mz[4], M = -3.0e38f;
 #pragma unroll
         for (int z = 0; z < 4; z++) {
@@ -930,7 +929,7 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
                 O += wt * ld_coh(all + (long)z * PER + 32 + idx);
             }
         }
-        if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + (idx >> 4)] = __fdiv_rn(O, L);
+        if (q < vrows) a.out[(long)(qb + q) * a.dim + h * HS + (idx >> 6) * 4 + (idx & 3)] = __fdiv_rn(O, L);
     }
 }
 
