@@ -765,14 +765,15 @@ static __global__ void __launch_bounds__(1024) k_bnext(const BNext a, unsigned *
 // The k index of a product may be permuted if both operands are: lane group g supplies the dimensions 16 u + 4 g + e
 // (one 16-byte load per u) and the keys 4 g + e.
 // grid: (n_heads, 2, 1..4): z splits the tiles of keys over that many workgroups, the last of which to finish merges what the
-// others left in device memory.  64 * WAVES threads; dynamic LDS: (16 HS + 32 WAVES + 16 WAVES HS) floats.
+// others left in device memory.  64 * WAVES threads; dynamic LDS: (16 (HS + 4) + 32 WAVES + 16 WAVES HS) floats.
 template <int HS, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
 {
     constexpr int U = HS / 16;
     extern __shared__ __align__(16) float pf_lds[];
-    float *sq = pf_lds;                  // [16 queries][HS]
-    float *wm = pf_lds + 16 * HS;        // [WAVES][16]
+    constexpr int SQ = HS + 4;           // (a row of q four floats longer: the sixteen rows a wave reads together start in different banks)
+    float *sq = pf_lds;                  // [16 queries][SQ]
+    float *wm = pf_lds + 16 * SQ;        // [WAVES][16]
     float *wl = wm + WAVES * 16;         // [WAVES][16]
     float *wo = wl + WAVES * 16;         // [WAVES][HS / 4][16 queries][4]: dimension d of query q at (d / 4) * 64 + 4 q + d % 4
     __shared__ float ww[WAVES * 16], wM[16];
@@ -791,13 +792,13 @@ __global__ void __launch_bounds__(64 * WAVES) k_pflash(const BAttn a)
             v0 += t.x; v1 += t.y;
         }
         const float2 cs = a.rope[(long)(a.st->pos + b) * half + idx];
-        sq[r * HS + 2 * idx] = __fsub_rn(__fmul_rn(v0, cs.x), __fmul_rn(v1, cs.y));
-        sq[r * HS + 2 * idx + 1] = __fadd_rn(__fmul_rn(v0, cs.y), __fmul_rn(v1, cs.x));
+        sq[r * SQ + 2 * idx] = __fsub_rn(__fmul_rn(v0, cs.x), __fmul_rn(v1, cs.y));
+        sq[r * SQ + 2 * idx + 1] = __fadd_rn(__fmul_rn(v0, cs.y), __fmul_rn(v1, cs.x));
     }
     __syncthreads();
     float4 qv[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) qv[u] = *reinterpret_cast<const float4 *>(&sq[c * HS + 16 * u + 4 * g]);
+    for (int u = 0; u < U; u++) qv[u] = *reinterpret_cast<const float4 *>(&sq[c * SQ + 16 * u + 4 * g]);
     const int qpos = pos0 + min(c, vrows - 1), lastkey = pos0 + vrows - 1, ntiles = lastkey / 16 + 1;
     const float *kc = a.kc + kvh * a.head_stride, *vc = a.vc + kvh * a.head_stride;
     const long rs = a.row_stride;

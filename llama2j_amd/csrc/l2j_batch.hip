@@ -344,7 +344,7 @@ int pflash_split(l2j_ctx *c, int first_pos)
     return std::min(kPflashMaxSplit, std::max(1, fit));
 }
 
-size_t pflash_lds(int hs, int waves) { return (size_t)(16 * hs + 32 * waves + 16 * waves * hs) * sizeof(float); }
+size_t pflash_lds(int hs, int waves) { return (size_t)(16 * (hs + 4) + 32 * waves + 16 * waves * hs) * sizeof(float); }
 
 // The forward passes of `rows` consecutive positions of one sequence (st: their tokens and the first position) as one batched
 // step into the context's own KV cache: launch_batch_step's kernels, the attention as two launches (every position stores
