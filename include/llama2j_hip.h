@@ -191,8 +191,9 @@ int l2j_decode_sample(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int
 /* l2j_decode_greedy_batch with a sampler per sequence: sequence s owns a new Sampler(rng_seeds[s], vocab_size) and every
  * unforced token of it is sampled as in l2j_sample (temperature 0: the argmax, no sampler is made), i.e. n_seq runs of the
  * loop of l2j_decode_sample side by side; the reference has neither ("parallel processing of multiple queries" is on its
- * wish-list, README.md:347).  The sampling steps are those of the single sequence, one launch per sequence and step, after
- * the step's forward pass; they need the one-launch step (vocab_size <= 36864, options "sampler_wide" and "sampler_scan"
+ * wish-list, README.md:347).  After a step's forward pass the sampling step of all sequences runs as one launch per stage
+ * (exponentials, probabilities and candidates, the sort's three stages, the pick), the sequences side by side in each;
+ * it keeps a sequence's probabilities in LDS (vocab_size <= 36864, option "sampler_scan"
  * on: else L2J_E_STATE).  The context's own sampler is not touched.  logits (may be NULL): as in
  * l2j_decode_greedy_batch_logits, the logits of every step before sampling, (steps, n_seq, vocab_size) floats. */
 int l2j_decode_sample_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,

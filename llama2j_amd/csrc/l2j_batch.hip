@@ -129,18 +129,9 @@ struct l2j::BatchBufs {
     int fuse_opt = 0;              // option batch_fuse when the step was planned
     int h_fault = 0;
     int *h_pin = nullptr;   // pinned: every transfer of a call goes through it, as in the single-sequence loops
-    // l2j_decode_sample_batch: a sampler per sequence (the reference's Sampler object: generator, flags, ProbIndex array twice)
-    SamplerState *ss = nullptr;                       // (sequence)
-    float *pi_prob[2] = {nullptr, nullptr};           // (sequence, pi_stride)
-    int *pi_idx[2] = {nullptr, nullptr};
-    size_t pi_stride = 0;
-    // two sampling steps run side by side (a step keeps half of the compute units busy): the second one on a stream and in
-    // work buffers of its own
+    BatchSamplers samplers;   // l2j_decode_sample_batch: a sampler per sequence (made by its first call)
     float *pf_part = nullptr;      // l2j_prefill: what the workgroups that share a head's keys leave for the one that merges,
     unsigned *pf_cnt = nullptr;    // and how many have (zero between launches)
-    SamplerWork side_work;
-    hipStream_t side = nullptr;
-    hipEvent_t ev_fwd = nullptr, ev_side = nullptr;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -151,12 +142,9 @@ struct l2j::BatchBufs {
         if (e0) (void)hipEventDestroy(e0);
         if (e1) (void)hipEventDestroy(e1);
         void *ps[] = {x, xn, xb, hb, logits, part[0], part[1], part[2], kc, vc, st, prompts, out, done, bar_ctr, fault, ssq, step_args,
-                      ss, pi_prob[0], pi_prob[1], pi_idx[0], pi_idx[1], pf_part, pf_cnt};
+                      pf_part, pf_cnt};
         for (void *p : ps) (void)hipFree(p);
-        free_sampler_work(&side_work);
-        if (side) (void)hipStreamDestroy(side);
-        if (ev_fwd) (void)hipEventDestroy(ev_fwd);
-        if (ev_side) (void)hipEventDestroy(ev_side);
+        free_batch_samplers(&samplers);
         if (h_pin) (void)hipHostFree(h_pin);
     }
 };
@@ -477,26 +465,17 @@ int ensure_batch(l2j_ctx *c, int nseq, int steps, int pstride)
 // The samplers of the sequences, as new Sampler(seeds[s], vocab_size) (J/Sampler.java:24-31) leaves them.
 int seed_batch_samplers(l2j_ctx *c, BatchBufs &b, const int64_t *seeds)
 {
-    const size_t n = (size_t)c->cfg.vocab_size, stride = (n + 4 + 3) / 4 * 4;   // (rows 16-byte aligned, read in 16-byte words)
-    if (!b.ss) {
-        int rc;
-        if ((rc = dev_alloc(&b.ss, (uint64_t)b.nseq))) return rc;
-        for (int i = 0; i < 2; i++) {
-            if ((rc = dev_alloc(&b.pi_prob[i], (uint64_t)b.nseq * stride))) return rc;
-            if ((rc = dev_alloc(&b.pi_idx[i], (uint64_t)b.nseq * stride))) return rc;
-        }
-        b.pi_stride = stride;
-        if ((rc = alloc_sampler_work(c, &b.side_work))) return rc;
-        HIPCHK(hipStreamCreateWithFlags(&b.side, hipStreamNonBlocking));
-        HIPCHK(hipEventCreateWithFlags(&b.ev_fwd, hipEventDisableTiming));
-        HIPCHK(hipEventCreateWithFlags(&b.ev_side, hipEventDisableTiming));
+    BatchSamplers &bs = b.samplers;
+    if (!bs.ss) {
+        const int rc = alloc_batch_samplers(c, b.nseq, &bs);
+        if (rc) return rc;
     }
     SamplerState h[kMaxBatch] = {};
     for (int s = 0; s < b.nseq; s++) h[s].rng = ((unsigned long long)seeds[s] ^ kJavaRandMult) & kJavaRandMask;
-    HIPCHK(hipMemcpyAsync(b.ss, h, (size_t)b.nseq * sizeof(SamplerState), hipMemcpyHostToDevice, c->stream));
+    HIPCHK(hipMemcpyAsync(bs.ss, h, (size_t)b.nseq * sizeof(SamplerState), hipMemcpyHostToDevice, c->stream));
     for (int i = 0; i < 2; i++) {
-        HIPCHK(hipMemsetAsync(b.pi_prob[i], 0, (size_t)b.nseq * stride * sizeof(float), c->stream));
-        HIPCHK(hipMemsetAsync(b.pi_idx[i], 0, (size_t)b.nseq * stride * sizeof(int), c->stream));
+        HIPCHK(hipMemsetAsync(bs.pi_prob[i], 0, (size_t)b.nseq * bs.pi_stride * sizeof(float), c->stream));
+        HIPCHK(hipMemsetAsync(bs.pi_idx[i], 0, (size_t)b.nseq * bs.pi_stride * sizeof(int), c->stream));
     }
     HIPCHK(hipStreamSynchronize(c->stream));   // (h is pageable host memory)
     return L2J_OK;
@@ -539,15 +518,8 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
     BatchBufs &b = *c->batch;
     const int vocab = cf.vocab_size, cap = b.cap_steps, pcap = b.cap_pstride;
     const size_t state_ints = sizeof(BatchState) / sizeof(int);
-    int cur[kMaxBatch] = {};   // which copy of its ProbIndex array a sequence's last top-p step left
-    SamplerWork own_work;
-    // (two steps side by side need two compute units per 256 probabilities)
-    const bool two_streams = 2 * ((vocab + 255) / 256) <= c->n_cu;
-    if (seeds) {
-        if ((rc = ensure_sampler_shared(c))) return rc;
-        if ((rc = seed_batch_samplers(c, b, seeds))) return rc;
-        own_work = sampler_work_of(c);
-    }
+    unsigned cur = 0;   // bit s: the copy of its ProbIndex array that sequence s's last top-p step left
+    if (seeds && (rc = seed_batch_samplers(c, b, seeds))) return rc;
     float *dlog = nullptr;
     if (logits_log) {
         hipError_t me = hipMalloc(reinterpret_cast<void **>(&dlog), (size_t)steps * nseq * vocab * sizeof(float));
@@ -555,7 +527,6 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
     }
     auto fail_hip = [&](hipError_t e, const char *what) {
         (void)hipStreamSynchronize(c->stream);
-        if (b.side) (void)hipStreamSynchronize(b.side);
         (void)hipFree(dlog);
         return hip_rc(e, what);
     };
@@ -579,27 +550,13 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
         }
         if (dlog && e == hipSuccess)
             e = hipMemcpyAsync(dlog + (size_t)pos * nseq * vocab, b.logits, (size_t)nseq * vocab * sizeof(float), hipMemcpyDeviceToDevice, c->stream);
-        // J/Run.java:643-665 for the sequences whose prompt is used up: the sampled token replaces the argmax k_bnext stored.
-        // Every other one of these steps goes to the second stream, between two events: after the forward pass, before the next.
+        // J/Run.java:643-665 for the sequences whose prompt is used up: the sampled token replaces the argmax k_bnext stored
         if (seeds && e == hipSuccess) {
-            int k = 0;
-            for (int s = 0; s < nseq && e == hipSuccess; s++) {
-                if (pos < n_prompt[s]) continue;
-                const bool aside = two_streams && (k++ & 1);
-                if (aside && k == 2) {
-                    e = hipEventRecord(b.ev_fwd, c->stream);
-                    if (e == hipSuccess) e = hipStreamWaitEvent(b.side, b.ev_fwd, 0);
-                    if (e != hipSuccess) break;
-                }
-                float *const prob[2] = {b.pi_prob[0] + (size_t)s * b.pi_stride, b.pi_prob[1] + (size_t)s * b.pi_stride};
-                int *const idx[2] = {b.pi_idx[0] + (size_t)s * b.pi_stride, b.pi_idx[1] + (size_t)s * b.pi_stride};
-                e = launch_sampler_of(c, aside ? b.side_work : own_work, aside ? b.side : c->stream, b.ss + s, prob, idx, &cur[s],
-                                      b.logits + (size_t)s * vocab, temperature, topp, -1.0f, nullptr, &b.st->token[s],
-                                      b.out + (size_t)s * cap + pos);
-            }
-            if (k >= 2 && two_streams && e == hipSuccess) {
-                e = hipEventRecord(b.ev_side, b.side);
-                if (e == hipSuccess) e = hipStreamWaitEvent(c->stream, b.ev_side, 0);
+            unsigned active = 0;
+            for (int s = 0; s < nseq; s++) active |= pos >= n_prompt[s] ? 1u << s : 0u;
+            if (active) {
+                e = launch_samplers(c, b.samplers, active, cur, b.logits, temperature, topp, b.st->token, b.out + pos, cap);
+                if ((double)topp <= 0.999) cur ^= active;   // (a top-p step leaves the array in its other copy)
             }
         }
         if (pos == 0 && e == hipSuccess) e = hipEventRecord(b.e0, c->stream);   // the clock starts after the first step (J/Run.java:682-684)
@@ -617,14 +574,9 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
     }
     if (seeds) {   // the reference's exceptions, and a wait that ran out, as in l2j_sample
         SamplerState h[kMaxBatch] = {};
-        if ((e = hipMemcpy(h, b.ss, (size_t)nseq * sizeof(SamplerState), hipMemcpyDeviceToHost)) != hipSuccess) return hip_rc(e, "sampler flags");
+        if ((e = hipMemcpy(h, b.samplers.ss, (size_t)nseq * sizeof(SamplerState), hipMemcpyDeviceToHost)) != hipSuccess) return hip_rc(e, "sampler flags");
         int st = 0;
         for (int s = 0; s < nseq; s++) st |= h[s].nan;
-        if (st & 4) {
-            if ((rc = reset_sampler_sync(own_work)) || (rc = reset_sampler_sync(b.side_work))) return rc;
-            return fail(L2J_E_HIP, "sampler: a workgroup waited too long for the others (k_sample_wide needs a compute unit per 256 "
-                                   "probabilities; is another process using the GPU?); the call was not completed");
-        }
         if (st & 1) return fail(L2J_E_ARG, "sampler: NaN among the logits (J/Sampler.java:88-90)");
         if (st & 2) return fail(L2J_E_ARG, "sampler: no probability reaches the top-p cutoff (ArrayIndexOutOfBoundsException at J/Sampler.java:119)");
     }

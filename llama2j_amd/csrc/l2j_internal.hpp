@@ -246,22 +246,26 @@ int resolve_scratch(int device);
 void free_sampler(l2j_ctx *c);
 int seed_sampler(l2j_ctx *c, int64_t rng_seed);
 hipError_t launch_sampler(l2j_ctx *c, float temperature, float topp, float coin, bool in_loop);
-// What a one-launch sampling step works in besides its sampler's own state: the sort's buffers, the exponentials, what the
-// workgroups hand each other.  One step at a time per set.
-struct SamplerWork {
-    float *sort_k[2] = {nullptr, nullptr};
+// The samplers of the sequences of the batched decode (each the reference's Sampler object: generator, flags, its ProbIndex
+// array twice) and what their steps work in; device memory, (sequence, stride) each.
+struct BatchSamplers {
+    int nseq = 0;
+    SamplerState *ss = nullptr;
+    float *pi_prob[2] = {nullptr, nullptr};
+    int *pi_idx[2] = {nullptr, nullptr};
+    size_t pi_stride = 0;
+    float *sort_k[2] = {nullptr, nullptr};   // the sort's tiles and runs
     int *sort_v[2] = {nullptr, nullptr};
-    float *sample_exp = nullptr;
-    unsigned char *wide_mem = nullptr;
+    size_t sort_stride = 0;
+    float *expbuf = nullptr;                 // the exponentials of a step
+    size_t exp_stride = 0;
 };
-hipError_t launch_sampler_of(l2j_ctx *c, const SamplerWork &work, hipStream_t stream, SamplerState *ss, float *const prob[2],
-                             int *const idx[2], int *cur_io, float *logits, float temperature, float topp, float coin, DevState *st,
-                             int *tok0, int *tok1);
-int ensure_sampler_shared(l2j_ctx *c);               // the context's own set (and its sampler) exist; the one-launch step is on
-SamplerWork sampler_work_of(l2j_ctx *c);             // the context's own set
-int alloc_sampler_work(l2j_ctx *c, SamplerWork *w);  // another set, for steps that run beside those in the context's
-void free_sampler_work(SamplerWork *w);
-int reset_sampler_sync(const SamplerWork &w);        // after a wait of the step ran out
+int alloc_batch_samplers(l2j_ctx *c, int nseq, BatchSamplers *bs);
+void free_batch_samplers(BatchSamplers *bs);
+// One sampling step for the sequences whose bit is set in `active` (cur: bit s = the copy of its array that sequence s's last
+// top-p step left), on the rows of logits; the tokens go to token[s] and out[s * out_stride].
+hipError_t launch_samplers(l2j_ctx *c, const BatchSamplers &bs, unsigned active, unsigned cur, float *logits, float temperature,
+                           float topp, int *token, int *out, long out_stride);
 // l2j_batch.hip: l2j_prefill without the lock (the decode loops call it holding it)
 int prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t pos0, float *logits, double *seconds);
 int check_sampler_status(l2j_ctx *c);

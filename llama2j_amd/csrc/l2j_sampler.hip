@@ -73,8 +73,9 @@ size_t sampler_lds_bytes(int n)
 constexpr size_t kWideSync = 0, kWideSsum = (sizeof(WideSync) + 63) / 64 * 64, kWideSeg = kWideSsum + 8 * kWideMaxSlices,
                  kWideCmask = kWideSeg + 16 * kWideMaxSlices, kWideT = kWideCmask + 32 * kWideMaxSlices, kWideD = kWideT + 3 * 8 * kWideMaxSlices, kWideBytes = kWideD + 3 * 8 * 64 * kWideMaxSlices;
 
-WideWs wide_ws(l2j_ctx *c, unsigned char *m)
+WideWs wide_ws(l2j_ctx *c)
 {
+    unsigned char *m = c->wide_mem;
     WideWs w{};
     w.sync = reinterpret_cast<WideSync *>(m + kWideSync);
     w.ssum = reinterpret_cast<double *>(m + kWideSsum);
@@ -158,77 +159,79 @@ namespace {
 
 }  // namespace
 
-// One sampling step in one launch (k_sample_wide) for a sampler whose state the caller names: its generator and flags ss,
-// the two copies of its ProbIndex array (*cur: the one the last call left; swapped by a top-p step), the logits it samples
-// from.  The sort's buffers and the kernel's workspace are the context's: steps on the context's stream follow each other.
-hipError_t l2j::launch_sampler_of(l2j_ctx *c, const SamplerWork &work, hipStream_t stream, SamplerState *ss, float *const prob[2],
-                                  int *const idx[2], int *cur_io, float *logits, float temperature, float topp, float coin, DevState *st,
-                                  int *tok0, int *tok1)
+// ---- a sampler per sequence of the batched decode: the launch-per-stage step with the sequence as grid z ----
+
+void l2j::free_batch_samplers(BatchSamplers *bs)
 {
-    const int n = c->cfg.vocab_size;
-    const int cur = *cur_io, other = cur ^ 1;
-    WideArgs wa{};
-    wa.logits = logits; wa.n = n;
-    wa.temperature = temperature; wa.topp = topp; wa.coin = coin;
-    wa.plain = (double)topp > 0.999;
-    wa.ss = ss;
-    wa.old_prob = prob[cur]; wa.old_idx = idx[cur];
-    wa.new_prob = prob[other]; wa.new_idx = idx[other];
-    wa.k0 = work.sort_k[0]; wa.v0 = work.sort_v[0]; wa.k1 = work.sort_k[1]; wa.v1 = work.sort_v[1];
-    wa.expbuf = work.sample_exp;
-    wa.st = st; wa.out_tokens = c->out_tokens;
-    wa.tok0 = tok0; wa.tok1 = tok1;
-    wa.w = wide_ws(c, work.wide_mem);
-    hipLaunchKernelGGL(k_sample_wide, dim3((n + kWideSlice - 1) / kWideSlice), dim3(kWideSlice), wide_lds_bytes(n), stream, wa);
-    if (!wa.plain) *cur_io = other;   // the array stays there until the next call
-    return hipGetLastError();
+    void *ps[] = {bs->ss, bs->pi_prob[0], bs->pi_prob[1], bs->pi_idx[0], bs->pi_idx[1], bs->sort_k[0], bs->sort_k[1], bs->sort_v[0],
+                  bs->sort_v[1], bs->expbuf};
+    for (void *p : ps) (void)hipFree(p);
+    *bs = BatchSamplers{};
 }
 
-// What the steps of launch_sampler_of share (the context's sampler buffers): made if they are not there yet.
-int l2j::ensure_sampler_shared(l2j_ctx *c)
+int l2j::alloc_batch_samplers(l2j_ctx *c, int nseq, BatchSamplers *bs)
 {
-    if (c->cfg.vocab_size > kSampleMaxVocab || c->opt[OPT_SAMPLER_WIDE] == 0 || c->opt[OPT_SAMPLER_SCAN] == 0)
-        return fail(L2J_E_STATE, "sampling for several sequences takes the one-launch sampling step: vocab_size up to 36864 and the "
-                                 "options sampler_wide and sampler_scan left on");
-    return c->ss ? L2J_OK : seed_sampler(c, 0);
-}
-
-// A wait of k_sample_wide ran out: its counters are not where the next launch expects them.
-int l2j::reset_sampler_sync(const SamplerWork &w)
-{
-    if (w.wide_mem) HIPCHK(hipMemset(w.wide_mem, 0, sizeof(WideSync)));
-    return L2J_OK;
-}
-
-SamplerWork l2j::sampler_work_of(l2j_ctx *c)
-{
-    SamplerWork w;
-    for (int i = 0; i < 2; i++) { w.sort_k[i] = c->sort_k[i]; w.sort_v[i] = c->sort_v[i]; }
-    w.sample_exp = c->sample_exp; w.wide_mem = c->wide_mem;
-    return w;
-}
-
-void l2j::free_sampler_work(SamplerWork *w)
-{
-    for (int i = 0; i < 2; i++) { (void)hipFree(w->sort_k[i]); (void)hipFree(w->sort_v[i]); }
-    (void)hipFree(w->sample_exp);
-    (void)hipFree(w->wide_mem);
-    *w = SamplerWork{};
-}
-
-int l2j::alloc_sampler_work(l2j_ctx *c, SamplerWork *w)
-{
-    const int n = c->cfg.vocab_size;
-    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
-    int rc = dev_alloc(&w->sample_exp, (uint64_t)npad + 4);
-    if (!rc) rc = dev_alloc(&w->wide_mem, kWideBytes);
+    const size_t n = (size_t)c->cfg.vocab_size;
+    if (n > (size_t)kSampleMaxVocab || c->opt[OPT_SAMPLER_SCAN] == 0)
+        return fail(L2J_E_STATE, "sampling for several sequences keeps a step's probabilities in LDS: vocab_size up to 36864 and the "
+                                 "option sampler_scan left on");
+    const size_t npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+    bs->nseq = nseq;
+    bs->pi_stride = (n + 4 + 3) / 4 * 4;   // (rows 16-byte aligned, read in 16-byte words)
+    bs->sort_stride = npad;
+    bs->exp_stride = npad + 4;
+    int rc = dev_alloc(&bs->ss, (uint64_t)nseq);
     for (int i = 0; i < 2 && !rc; i++) {
-        rc = dev_alloc(&w->sort_k[i], (uint64_t)npad);
-        if (!rc) rc = dev_alloc(&w->sort_v[i], (uint64_t)npad);
+        if (!rc) rc = dev_alloc(&bs->pi_prob[i], (uint64_t)nseq * bs->pi_stride);
+        if (!rc) rc = dev_alloc(&bs->pi_idx[i], (uint64_t)nseq * bs->pi_stride);
+        if (!rc) rc = dev_alloc(&bs->sort_k[i], (uint64_t)nseq * bs->sort_stride);
+        if (!rc) rc = dev_alloc(&bs->sort_v[i], (uint64_t)nseq * bs->sort_stride);
     }
-    if (!rc && hipMemset(w->wide_mem, 0, kWideBytes) != hipSuccess) rc = fail(L2J_E_HIP, "sampler: clearing the step's counters");
-    if (rc) free_sampler_work(w);
+    if (!rc) rc = dev_alloc(&bs->expbuf, (uint64_t)nseq * bs->exp_stride);
+    if (!rc) {   // (more than the default 64 KB of dynamic LDS)
+        const int lds = (int)sampler_lds_bytes((int)n);
+        if (hipFuncSetAttribute((const void *)k_sample_probs<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess ||
+            hipFuncSetAttribute((const void *)k_topp_pick<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+            rc = fail(L2J_E_HIP, "sampler: dynamic LDS of a step");
+    }
+    if (rc) free_batch_samplers(bs);
     return rc;
+}
+
+hipError_t l2j::launch_samplers(l2j_ctx *c, const BatchSamplers &bs, unsigned active, unsigned cur, float *logits, float temperature,
+                                float topp, int *token, int *out, long out_stride)
+{
+    const int n = c->cfg.vocab_size, nseq = bs.nseq;
+    const int npad = (n + kSortRun - 1) / kSortRun * kSortRun;
+    SampleArgs a{};
+    a.logits = logits; a.n = n;
+    a.temperature = temperature; a.topp = topp; a.coin = -1.0f;
+    a.plain = (double)topp > 0.999;
+    a.ss = bs.ss;
+    a.scan = 1;
+    a.nseq = nseq; a.active = active; a.cur = cur;
+    for (int i = 0; i < 2; i++) { a.pi_prob[i] = bs.pi_prob[i]; a.pi_idx[i] = bs.pi_idx[i]; }
+    a.logits_stride = n; a.pi_stride = (long)bs.pi_stride; a.exp_stride = (long)bs.exp_stride;
+    a.btoken = token; a.bout = out; a.bout_stride = out_stride;
+    const int front_wgs = std::min(1024, std::max(0, c->opt[OPT_SAMPLER_EXP_WGS]));   // (workgroups of k_sample_exp per sequence)
+    a.expbuf = front_wgs > 0 ? bs.expbuf : nullptr;
+    if (a.expbuf) hipLaunchKernelGGL(k_sample_exp, dim3(front_wgs, 1, nseq), dim3(1024), 0, c->stream, a);
+    const size_t lds = sampler_lds_bytes(n);
+    hipLaunchKernelGGL(k_sample_probs<true>, dim3(1, 1, nseq), dim3(1024), lds, c->stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || a.plain) return e;
+    SortBatch sb{};
+    sb.active = active; sb.cur = cur;
+    for (int i = 0; i < 2; i++) {
+        sb.pi_prob[i] = bs.pi_prob[i]; sb.pi_idx[i] = bs.pi_idx[i]; sb.out_prob[i] = bs.pi_prob[i]; sb.out_idx[i] = bs.pi_idx[i];
+        sb.sort_k[i] = bs.sort_k[i]; sb.sort_v[i] = bs.sort_v[i];
+    }
+    sb.pi_stride = (long)bs.pi_stride; sb.sort_stride = (long)bs.sort_stride;
+    hipLaunchKernelGGL(k_sort_tiles_b, dim3(npad / kSortTile, 1, nseq), dim3(kSortTile), 0, c->stream, sb, n);
+    hipLaunchKernelGGL(k_merge_tiles_b, dim3(npad / kSortRun, 16, nseq), dim3(256), 0, c->stream, sb);
+    hipLaunchKernelGGL(k_merge_far_b, dim3(npad / 256, 1, nseq), dim3(256), 0, c->stream, sb, npad, n);
+    hipLaunchKernelGGL(k_topp_pick<true>, dim3(1, 1, nseq), dim3(1024), lds, c->stream, a);
+    return hipGetLastError();
 }
 
 // The sampling step of J/Run.java:643-665 on c->logits; in_loop: the token replaces what k_finish stored.
@@ -248,10 +251,20 @@ hipError_t l2j::launch_sampler(l2j_ctx *c, float temperature, float topp, float 
     a.scan = c->opt[OPT_SAMPLER_SCAN] != 0 ? 1 : 0;
     const bool in_lds = n <= kSampleMaxVocab;   // else the kernels work in device memory, where k_sample_exp leaves the exponentials
     if (in_lds && c->opt[OPT_SAMPLER_WIDE] != 0 && a.scan) {
-        float *const prob[2] = {c->pi_prob[0], c->pi_prob[1]};
-        int *const idx[2] = {c->pi_idx[0], c->pi_idx[1]};
-        return launch_sampler_of(c, sampler_work_of(c), c->stream, c->ss, prob, idx, &c->pi_cur, c->logits, temperature, topp, coin, a.st,
-                                 nullptr, nullptr);
+        WideArgs wa{};
+        wa.logits = c->logits; wa.n = n;
+        wa.temperature = temperature; wa.topp = topp; wa.coin = coin;
+        wa.plain = a.plain;
+        wa.ss = c->ss;
+        wa.old_prob = c->pi_prob[cur]; wa.old_idx = c->pi_idx[cur];
+        wa.new_prob = c->pi_prob[other]; wa.new_idx = c->pi_idx[other];
+        wa.k0 = c->sort_k[0]; wa.v0 = c->sort_v[0]; wa.k1 = c->sort_k[1]; wa.v1 = c->sort_v[1];
+        wa.expbuf = c->sample_exp;
+        wa.st = a.st; wa.out_tokens = a.out_tokens;
+        wa.w = wide_ws(c);
+        hipLaunchKernelGGL(k_sample_wide, dim3((n + kWideSlice - 1) / kWideSlice), dim3(kWideSlice), wide_lds_bytes(n), c->stream, wa);
+        if (!a.plain) c->pi_cur = other;   // the array stays there until the next call
+        return hipGetLastError();
     }
     const int exp_wgs = std::min(1024, std::max(in_lds ? 0 : 1, c->opt[OPT_SAMPLER_EXP_WGS]));   // 0: the exponentials in k_sample_probs' one workgroup
     a.expbuf = exp_wgs > 0 ? c->sample_exp : nullptr;
@@ -416,7 +429,7 @@ int l2j_sum_probe(l2j_ctx *c, const float *terms, int32_t n, const float *limits
         if (e == hipSuccess && n_limits > 0) e = hipMemcpyAsync(d_lim, limits, (size_t)n_limits * sizeof(float), hipMemcpyHostToDevice, c->stream);
         if (e == hipSuccess) {
             hipLaunchKernelGGL(k_sum_probe, dim3(slices), dim3(kWideSlice), sizeof(WideWalk), c->stream, d, n, d_lim, n_limits, d_idx, d_sum,
-                               d_total, c->ss, wide_ws(c, c->wide_mem));
+                               d_total, c->ss, wide_ws(c));
             e = hipGetLastError();
         }
         if (e == hipSuccess && n_limits > 0) e = hipMemcpyAsync(index_out, d_idx, (size_t)n_limits * sizeof(int), hipMemcpyDeviceToHost, c->stream);

@@ -37,7 +37,38 @@ struct SampleArgs {
     int *out_tokens;         //   that k_finish stored for position st->pos - 1
     int scan;                // 1: the running sums by spec_sums, 0: one lane adds them all (vocabularies that fit in LDS only)
     float *expbuf;           // not null: k_sample_exp has left exp(x / temperature - max) here (n floats)
+    int *tok0, *tok1;        // null, or two more places that receive the token
+    // Several samplers in one launch (the sequences of the batched decode; nseq 0: one): grid z = sequence.  The fields above
+    // are those of sequence 0 (cand_*, sorted_* unused); the arrays of the others follow at these strides.
+    int nseq;
+    unsigned active;         // bit s: sequence s samples in this step (the others' workgroups leave at once)
+    unsigned cur;            // bit s: the copy of its ProbIndex array that sequence s's last top-p step left
+    float *pi_prob[2];       // the two copies, (sequence, pi_stride)
+    int *pi_idx[2];
+    long logits_stride, pi_stride, exp_stride;
+    int *btoken;             // (sequence): the token goes here (the sequence's next input)
+    int *bout;               // and to bout[s * bout_stride]
+    long bout_stride;
 };
+
+// The arguments of this workgroup's sequence; false: it does not sample in this step.
+__device__ __forceinline__ bool sample_seq(SampleArgs &a)
+{
+    if (a.nseq == 0) return true;
+    const int s = blockIdx.z;
+    if (!((a.active >> s) & 1u)) return false;
+    const int cur = (a.cur >> s) & 1u;
+    a.logits += s * a.logits_stride;
+    a.ss += s;
+    a.cand_prob = a.pi_prob[cur] + s * a.pi_stride;
+    a.cand_idx = a.pi_idx[cur] + s * a.pi_stride;
+    a.sorted_prob = a.pi_prob[cur ^ 1] + s * a.pi_stride;
+    a.sorted_idx = a.pi_idx[cur ^ 1] + s * a.pi_stride;
+    if (a.expbuf) a.expbuf += s * a.exp_stride;
+    a.tok0 = a.btoken + s;
+    a.tok1 = a.bout + s * a.bout_stride;
+    return true;
+}
 
 // java.util.Random.nextFloat(): next(24) / (float)(1 << 24)
 __device__ __forceinline__ float java_next_float(unsigned long long *rng)
@@ -386,8 +417,10 @@ __device__ __forceinline__ int spec_first_over(const float *p, const SpecThread 
 // The element-wise front of the step spread over many workgroups (the double-precision exponential of 32000 logits
 // takes 0.04 ms on one compute unit): every workgroup divides all the logits by the temperature and takes the maximum
 // (the same value everywhere: a maximum does not depend on the order), then exponentiates its own slice into expbuf.
-static __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
+static __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a0)
 {
+    SampleArgs a = a0;
+    if (!sample_seq(a)) return;
     __shared__ float red[16];
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
     float mx = -__builtin_inff();
@@ -440,8 +473,10 @@ union SamplerShared {
 // (dynamic LDS: (n rounded up to 32) + 32 floats, n <= kSampleMaxVocab); else in a.expbuf, where k_sample_exp has
 // left the exponentials (any n).
 template <bool IN_LDS>
-__global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
+__global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a0)
 {
+    SampleArgs a = a0;
+    if (!sample_seq(a)) return;
     extern __shared__ __align__(16) float lds_sp[];
     __shared__ SamplerShared u;
     __shared__ float red[16];
@@ -521,6 +556,8 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
         if (pick >= n) pick = n - 1;
         if (tid == 0) {
             a.ss->result = pick;
+            if (a.tok0) *a.tok0 = pick;
+            if (a.tok1) *a.tok1 = pick;
             if (a.st) {
                 a.out_tokens[a.st->pos - 1] = pick;
                 a.st->token = pick;
@@ -565,8 +602,10 @@ __global__ void __launch_bounds__(1024) k_sample_probs(const SampleArgs a)
 // J/Sampler.java:99-119 on the sorted ProbIndex array.  One workgroup.  IN_LDS: the candidates are copied to LDS first
 // (dynamic LDS as above, n0 <= n <= kSampleMaxVocab); else they are read where they are.
 template <bool IN_LDS>
-__global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
+__global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a0)
 {
+    SampleArgs a = a0;
+    if (!sample_seq(a)) return;
     extern __shared__ __align__(16) float lds_sp[];
     __shared__ SamplerShared u;
     __shared__ float s_cum, s_r, s_f;
@@ -611,6 +650,8 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
         if (tid == 0) {
             const int token = a.sorted_idx[pick];
             a.ss->result = token;
+            if (a.tok0) *a.tok0 = token;
+            if (a.tok1) *a.tok1 = token;
             if (a.st) {
                 a.out_tokens[a.st->pos - 1] = token;
                 a.st->token = token;
@@ -645,6 +686,8 @@ __global__ void __launch_bounds__(1024) k_topp_pick(const SampleArgs a)
     if (tid == 0) {
         const int token = a.sorted_idx[pick];
         a.ss->result = token;
+        if (a.tok0) *a.tok0 = token;
+        if (a.tok1) *a.tok1 = token;
         if (a.st) {
             a.out_tokens[a.st->pos - 1] = token;
             a.st->token = token;
@@ -703,8 +746,8 @@ __device__ __forceinline__ float sort_below(float k)
 }
 
 // grid: padded n / 256 workgroups of 256 threads
-static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
-                                                          float *__restrict__ kout, int *__restrict__ vout)
+__device__ __forceinline__ void sort_tiles_of(const float *__restrict__ kin, const int *__restrict__ vin, int n,
+                                              float *__restrict__ kout, int *__restrict__ vout)
 {
     // a pair stands before another when its probability is greater, or equal and its position lower: one unsigned
     // comparison of (probability bits, 255 - position); the bits of a non-negative float ascend with it, the padding's -1
@@ -729,8 +772,36 @@ static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__
 // grid: (padded n / 4096, 16) workgroups of 256 threads: a workgroup holds the keys of its run in LDS and places a
 // sixteenth of them, one per thread.  The fifteen binary searches of a pair advance together, step by step (their LDS reads are
 // independent: one after the other they cost fifteen times the latency).
-static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
-                                                     int *__restrict__ vout)
+static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__restrict__ kin, const int *__restrict__ vin, int n,
+                                                          float *__restrict__ kout, int *__restrict__ vout)
+{
+    sort_tiles_of(kin, vin, n, kout, vout);
+}
+
+// The sort for several samplers in one launch (grid z = sequence; SampleArgs says which take part and where their arrays
+// lie): a sequence's ProbIndex array goes from the copy its last step left through its own runs into the other copy.
+struct SortBatch {
+    unsigned active, cur;
+    const float *pi_prob[2];
+    const int *pi_idx[2];
+    float *out_prob[2];      // (the same two copies, as the destination of the last merge)
+    int *out_idx[2];
+    long pi_stride;
+    float *sort_k[2];        // (sequence, sort_stride) twice: tiles, then runs
+    int *sort_v[2];
+    long sort_stride;
+};
+
+static __global__ void __launch_bounds__(kSortTile) k_sort_tiles_b(const SortBatch b, int n)
+{
+    const int s = blockIdx.z, cur = (b.cur >> s) & 1u;
+    if (!((b.active >> s) & 1u)) return;
+    sort_tiles_of(b.pi_prob[cur] + s * b.pi_stride, b.pi_idx[cur] + s * b.pi_stride, n, b.sort_k[0] + s * b.sort_stride,
+                  b.sort_v[0] + s * b.sort_stride);
+}
+
+__device__ __forceinline__ void merge_tiles_of(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
+                                               int *__restrict__ vout)
 {
     __shared__ __align__(16) float keys[kSortRun];
     const int tid = threadIdx.x, base = blockIdx.x * kSortRun;
@@ -763,6 +834,20 @@ static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restr
     }
     kout[base + rank] = k;
     vout[base + rank] = v;
+}
+
+static __global__ void __launch_bounds__(256) k_merge_tiles(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
+                                                     int *__restrict__ vout)
+{
+    merge_tiles_of(kin, vin, kout, vout);
+}
+
+static __global__ void __launch_bounds__(256) k_merge_tiles_b(const SortBatch b)
+{
+    const int s = blockIdx.z;
+    if (!((b.active >> s) & 1u)) return;
+    merge_tiles_of(b.sort_k[0] + s * b.sort_stride, b.sort_v[0] + s * b.sort_stride, b.sort_k[1] + s * b.sort_stride,
+                   b.sort_v[1] + s * b.sort_stride);
 }
 
 constexpr int kSortMaxRuns = (kSampleMaxVocab + kSortRun - 1) / kSortRun;
@@ -815,8 +900,8 @@ static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restri
 // grid: padded n / 256 workgroups of 256 threads; run_len and group_len are powers of two, npad a multiple of 256.
 constexpr int kSortFanIn = 16;
 
-static __global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
-                                                    int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
+__device__ __forceinline__ void merge_far_of(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
+                                             int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
     const float k = kin[i];
@@ -851,6 +936,23 @@ static __global__ void __launch_bounds__(256) k_merge_far(const float *__restric
         kout[rank] = k;
         vout[rank] = v;
     }
+}
+
+static __global__ void __launch_bounds__(256) k_merge_far(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
+                                                    int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
+{
+    merge_far_of(kin, vin, npad, nout, run_len, group_len, kout, vout);
+}
+
+// The last merge of k_sort_tiles_b's sort (at most kSortFanIn runs of kSortRun pairs: padded n up to 65536): the runs of a
+// sequence into the other copy of its ProbIndex array, the keys read where they lie (32 sequences' keys fit the caches;
+// holding a sequence's keys in LDS as k_merge_runs does would leave one workgroup per compute unit).
+static __global__ void __launch_bounds__(256) k_merge_far_b(const SortBatch b, int npad, int nout)
+{
+    const int s = blockIdx.z, cur = (b.cur >> s) & 1u;
+    if (!((b.active >> s) & 1u)) return;
+    merge_far_of(b.sort_k[1] + s * b.sort_stride, b.sort_v[1] + s * b.sort_stride, npad, nout, kSortRun, kSortRun * kSortFanIn,
+                 b.out_prob[cur ^ 1] + s * b.pi_stride, b.out_idx[cur ^ 1] + s * b.pi_stride);
 }
 
 // J/Sampler.java:46-57 on an array given by the caller: first index of the strict maximum.  One workgroup.

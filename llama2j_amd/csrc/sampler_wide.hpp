@@ -86,8 +86,6 @@ struct WideArgs {
     float *expbuf;              // slices * 256 floats
     DevState *st;
     int *out_tokens;
-    int *tok0, *tok1;           // null, or two more places that receive the token (a sequence of the batched decode: its next
-                                // input token and its row of the output)
     WideWs w;
 };
 
@@ -690,8 +688,6 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
                     a.out_tokens[a.st->pos - 1] = pick;
                     a.st->token = pick;
                 }
-                if (a.tok0) *a.tok0 = pick;
-                if (a.tok1) *a.tok1 = pick;
             }
         }
         wide_leave(a.w, a.ss);
@@ -901,8 +897,6 @@ static __global__ void __launch_bounds__(kWideSlice) k_sample_wide(const WideArg
                 a.out_tokens[a.st->pos - 1] = token;
                 a.st->token = token;
             }
-            if (a.tok0) *a.tok0 = token;
-            if (a.tok1) *a.tok1 = token;
         }
     }
     wide_leave(a.w, a.ss);

@@ -267,7 +267,7 @@ def test_sampled_batch_gives_every_sequence_its_own_sampler(orc, n_seq, t, topp,
     g.close()
 
 
-def test_sampled_batch_refuses_what_the_one_launch_sampler_cannot_take():
+def test_sampled_batch_refuses_what_its_sampling_step_cannot_take():
     g = l2j.Transformer(l2j.Config(*SHAPES[3]))
     g.fill_synthetic(3, 0.02)
     g.finalize()
@@ -276,28 +276,28 @@ def test_sampled_batch_refuses_what_the_one_launch_sampler_cannot_take():
         g.decode_sample_batch(p, 8, -1.0, 0.9, [1])
     with pytest.raises(L2JError):
         g.decode_sample_batch(p, 8, 1.0, 1.5, [1])
-    g.set_option("sampler_wide", 0)
-    with pytest.raises(L2JError, match="one-launch"):
+    g.set_option("sampler_scan", 0)
+    with pytest.raises(L2JError, match="sampler_scan"):
         g.decode_sample_batch(p, 8, 1.0, 0.9, [1])
-    g.set_option("sampler_wide", 1)
+    g.set_option("sampler_scan", 1)
+    g.set_option("sampler_wide", 0)                      # (the one-launch step of the single sequence: not what the batch takes)
     out, _ = g.decode_sample_batch(p, 8, 1.0, 0.9, [1])
     assert out.shape == (16, 8) and np.array_equal(out[0, :2], p[0])
     g.close()
 
 
-def test_a_wait_of_a_sampling_step_that_runs_out_fails_the_sampled_batch_and_nothing_else():
-    """barrier_spins 0: the first workgroup to reach a grid barrier of a sampling step gives up at once (every kernel still runs
-    to its end).  The call is an error; the greedy loops, which have no such wait, go on giving what they gave."""
+def test_the_sampling_steps_of_the_batch_wait_for_nobody():
+    """barrier_spins 0 makes every bounded wait between workgroups give up at once; the batch's sampling steps have none (a
+    launch per stage, the sequences side by side in each): the tokens of a context with the default."""
     shape = SHAPES[0]
-    g = l2j.Transformer(l2j.Config(*shape))
-    g.fill_synthetic(5, 0.02)
-    g.set_option("barrier_spins", 0)
-    g.finalize()
-    p = [np.array([9, 8, 7], dtype=np.int32)]
-    before, _ = g.decode_greedy_batch(p, 12)
-    for _ in range(2):   # (the second call finds the step's counters cleared)
-        with pytest.raises(L2JError, match="waited too long"):
-            g.decode_sample_batch(p, 12, 1.0, 0.9, [3])
-    after, _ = g.decode_greedy_batch(p, 12)
-    np.testing.assert_array_equal(after, before)
-    g.close()
+    outs = []
+    for spins in (None, 0):
+        g = l2j.Transformer(l2j.Config(*shape))
+        g.fill_synthetic(5, 0.02)
+        if spins is not None:
+            g.set_option("barrier_spins", spins)
+        g.finalize()
+        out, _ = g.decode_sample_batch([np.array([9, 8, 7], dtype=np.int32)], 12, 1.0, 0.9, [3])
+        outs.append(out)
+        g.close()
+    np.testing.assert_array_equal(outs[0], outs[1])
