@@ -257,8 +257,6 @@ struct BatchSamplers {
     float *sort_k[2] = {nullptr, nullptr};   // the sort's tiles and runs
     int *sort_v[2] = {nullptr, nullptr};
     size_t sort_stride = 0;
-    float *expbuf = nullptr;                 // the exponentials of a step
-    size_t exp_stride = 0;
 };
 int alloc_batch_samplers(l2j_ctx *c, int nseq, BatchSamplers *bs);
 void free_batch_samplers(BatchSamplers *bs);

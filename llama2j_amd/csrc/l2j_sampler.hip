@@ -164,7 +164,7 @@ namespace {
 void l2j::free_batch_samplers(BatchSamplers *bs)
 {
     void *ps[] = {bs->ss, bs->pi_prob[0], bs->pi_prob[1], bs->pi_idx[0], bs->pi_idx[1], bs->sort_k[0], bs->sort_k[1], bs->sort_v[0],
-                  bs->sort_v[1], bs->expbuf};
+                  bs->sort_v[1]};
     for (void *p : ps) (void)hipFree(p);
     *bs = BatchSamplers{};
 }
@@ -179,7 +179,6 @@ int l2j::alloc_batch_samplers(l2j_ctx *c, int nseq, BatchSamplers *bs)
     bs->nseq = nseq;
     bs->pi_stride = (n + 4 + 3) / 4 * 4;   // (rows 16-byte aligned, read in 16-byte words)
     bs->sort_stride = npad;
-    bs->exp_stride = npad + 4;
     int rc = dev_alloc(&bs->ss, (uint64_t)nseq);
     for (int i = 0; i < 2 && !rc; i++) {
         if (!rc) rc = dev_alloc(&bs->pi_prob[i], (uint64_t)nseq * bs->pi_stride);
@@ -187,7 +186,6 @@ int l2j::alloc_batch_samplers(l2j_ctx *c, int nseq, BatchSamplers *bs)
         if (!rc) rc = dev_alloc(&bs->sort_k[i], (uint64_t)nseq * bs->sort_stride);
         if (!rc) rc = dev_alloc(&bs->sort_v[i], (uint64_t)nseq * bs->sort_stride);
     }
-    if (!rc) rc = dev_alloc(&bs->expbuf, (uint64_t)nseq * bs->exp_stride);
     if (!rc) {   // (more than the default 64 KB of dynamic LDS)
         const int lds = (int)sampler_lds_bytes((int)n);
         if (hipFuncSetAttribute((const void *)k_sample_probs<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess ||
@@ -211,11 +209,10 @@ hipError_t l2j::launch_samplers(l2j_ctx *c, const BatchSamplers &bs, unsigned ac
     a.scan = 1;
     a.nseq = nseq; a.active = active; a.cur = cur;
     for (int i = 0; i < 2; i++) { a.pi_prob[i] = bs.pi_prob[i]; a.pi_idx[i] = bs.pi_idx[i]; }
-    a.logits_stride = n; a.pi_stride = (long)bs.pi_stride; a.exp_stride = (long)bs.exp_stride;
+    a.logits_stride = n; a.pi_stride = (long)bs.pi_stride;
     a.btoken = token; a.bout = out; a.bout_stride = out_stride;
-    const int front_wgs = std::min(1024, std::max(0, c->opt[OPT_SAMPLER_EXP_WGS]));   // (workgroups of k_sample_exp per sequence)
-    a.expbuf = front_wgs > 0 ? bs.expbuf : nullptr;
-    if (a.expbuf) hipLaunchKernelGGL(k_sample_exp, dim3(front_wgs, 1, nseq), dim3(1024), 0, c->stream, a);
+    // (no k_sample_exp: with the sequences' workgroups side by side the exponentials cost less inside k_sample_probs than
+    // a launch of their own, in which every workgroup reads all of its sequence's logits for the maximum: 81 us measured)
     const size_t lds = sampler_lds_bytes(n);
     hipLaunchKernelGGL(k_sample_probs<true>, dim3(1, 1, nseq), dim3(1024), lds, c->stream, a);
     hipError_t e = hipGetLastError();

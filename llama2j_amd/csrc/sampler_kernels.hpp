@@ -39,13 +39,14 @@ struct SampleArgs {
     float *expbuf;           // not null: k_sample_exp has left exp(x / temperature - max) here (n floats)
     int *tok0, *tok1;        // null, or two more places that receive the token
     // Several samplers in one launch (the sequences of the batched decode; nseq 0: one): grid z = sequence.  The fields above
-    // are those of sequence 0 (cand_*, sorted_* unused); the arrays of the others follow at these strides.
+    // are those of sequence 0 (cand_*, sorted_* unused; expbuf null: k_sample_probs forms the exponentials itself, the
+    // sequences' workgroups side by side); the arrays of the others follow at these strides.
     int nseq;
     unsigned active;         // bit s: sequence s samples in this step (the others' workgroups leave at once)
     unsigned cur;            // bit s: the copy of its ProbIndex array that sequence s's last top-p step left
     float *pi_prob[2];       // the two copies, (sequence, pi_stride)
     int *pi_idx[2];
-    long logits_stride, pi_stride, exp_stride;
+    long logits_stride, pi_stride;
     int *btoken;             // (sequence): the token goes here (the sequence's next input)
     int *bout;               // and to bout[s * bout_stride]
     long bout_stride;
@@ -64,7 +65,6 @@ __device__ __forceinline__ bool sample_seq(SampleArgs &a)
     a.cand_idx = a.pi_idx[cur] + s * a.pi_stride;
     a.sorted_prob = a.pi_prob[cur ^ 1] + s * a.pi_stride;
     a.sorted_idx = a.pi_idx[cur ^ 1] + s * a.pi_stride;
-    if (a.expbuf) a.expbuf += s * a.exp_stride;
     a.tok0 = a.btoken + s;
     a.tok1 = a.bout + s * a.bout_stride;
     return true;
@@ -417,10 +417,8 @@ __device__ __forceinline__ int spec_first_over(const float *p, const SpecThread 
 // The element-wise front of the step spread over many workgroups (the double-precision exponential of 32000 logits
 // takes 0.04 ms on one compute unit): every workgroup divides all the logits by the temperature and takes the maximum
 // (the same value everywhere: a maximum does not depend on the order), then exponentiates its own slice into expbuf.
-static __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a0)
+static __global__ void __launch_bounds__(1024) k_sample_exp(const SampleArgs a)
 {
-    SampleArgs a = a0;
-    if (!sample_seq(a)) return;
     __shared__ float red[16];
     const int tid = threadIdx.x, n = a.n, nt = blockDim.x;
     float mx = -__builtin_inff();
@@ -900,6 +898,7 @@ static __global__ void __launch_bounds__(256) k_merge_runs(const float *__restri
 // grid: padded n / 256 workgroups of 256 threads; run_len and group_len are powers of two, npad a multiple of 256.
 constexpr int kSortFanIn = 16;
 
+template <int FANIN = kSortFanIn>
 __device__ __forceinline__ void merge_far_of(const float *__restrict__ kin, const int *__restrict__ vin, int npad, int nout,
                                              int run_len, int group_len, float *__restrict__ kout, int *__restrict__ vout)
 {
@@ -910,9 +909,9 @@ __device__ __forceinline__ void merge_far_of(const float *__restrict__ kin, cons
     const int off = i - g0, ri = off / run_len;
     const int gend = min(npad, g0 + group_len);
     int rank = g0 + off - ri * run_len;
-    int pos[kSortFanIn], len[kSortFanIn];
+    int pos[FANIN], len[FANIN];
 #pragma unroll
-    for (int u = 0; u < kSortFanIn; u++) {
+    for (int u = 0; u < FANIN; u++) {
         len[u] = max(0, min(run_len, gend - g0 - u * run_len));   // 0: no such run in this group
         pos[u] = 0;
     }
@@ -920,14 +919,14 @@ __device__ __forceinline__ void merge_far_of(const float *__restrict__ kin, cons
     const float kb = sort_below(k);
     for (int st = run_len >> 1; st > 0; st >>= 1) {
 #pragma unroll
-        for (int u = 0; u < kSortFanIn; u++) {
+        for (int u = 0; u < FANIN; u++) {
             const int at = pos[u] + st - 1;
             const float o = run[min(u * run_len + at, gend - g0 - 1)];
             pos[u] += (at < len[u] && o > (u < ri ? kb : k)) ? st : 0;   // runs that stood earlier win ties
         }
     }
 #pragma unroll
-    for (int u = 0; u < kSortFanIn; u++) {
+    for (int u = 0; u < FANIN; u++) {
         const float o = run[min(u * run_len + pos[u], gend - g0 - 1)];
         const int cnt = pos[u] + ((pos[u] < len[u] && o > (u < ri ? kb : k)) ? 1 : 0);
         rank += u != ri ? cnt : 0;
@@ -951,8 +950,12 @@ static __global__ void __launch_bounds__(256) k_merge_far_b(const SortBatch b, i
 {
     const int s = blockIdx.z, cur = (b.cur >> s) & 1u;
     if (!((b.active >> s) & 1u)) return;
-    merge_far_of(b.sort_k[1] + s * b.sort_stride, b.sort_v[1] + s * b.sort_stride, npad, nout, kSortRun, kSortRun * kSortFanIn,
-                 b.out_prob[cur ^ 1] + s * b.pi_stride, b.out_idx[cur ^ 1] + s * b.pi_stride);
+    const float *kin = b.sort_k[1] + s * b.sort_stride;
+    const int *vin = b.sort_v[1] + s * b.sort_stride;
+    float *kout = b.out_prob[cur ^ 1] + s * b.pi_stride;
+    int *vout = b.out_idx[cur ^ 1] + s * b.pi_stride;
+    if (npad <= 8 * kSortRun) merge_far_of<8>(kin, vin, npad, nout, kSortRun, kSortRun * kSortFanIn, kout, vout);   // (eight searches per pair)
+    else merge_far_of<kSortFanIn>(kin, vin, npad, nout, kSortRun, kSortRun * kSortFanIn, kout, vout);
 }
 
 // J/Sampler.java:46-57 on an array given by the caller: first index of the strict maximum.  One workgroup.
