@@ -572,7 +572,7 @@ int decode_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, in
         dlog = nullptr;
         if (e != hipSuccess) return hip_rc(e, "logits read-back");
     }
-    if (seeds) {   // the reference's exceptions, and a wait that ran out, as in l2j_sample
+    if (seeds) {   // the reference's exceptions, as in l2j_sample
         SamplerState h[kMaxBatch] = {};
         if ((e = hipMemcpy(h, b.samplers.ss, (size_t)nseq * sizeof(SamplerState), hipMemcpyDeviceToHost)) != hipSuccess) return hip_rc(e, "sampler flags");
         int st = 0;
@@ -627,11 +627,15 @@ int l2j::prefill_positions(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t
         HIPCHK(hipFuncSetAttribute(reinterpret_cast<const void *>(k_pflash<256, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)pflash_lds(256, 8)));
         c->pflash_ready = true;
     }
-    if (!b.pf_part) {
-        int arc;
-        if ((arc = dev_alloc(&b.pf_part, (uint64_t)cf.n_heads * 2 * kPflashMaxSplit * (32 + 16 * hs)))) return arc;
-        if ((arc = dev_alloc(&b.pf_cnt, (uint64_t)cf.n_heads * 2))) return arc;
-        HIPCHK(hipMemset(b.pf_cnt, 0, (size_t)cf.n_heads * 2 * sizeof(unsigned)));
+    if (!b.pf_cnt) {   // (the counters last: their presence says that both are there and cleared)
+        if (!b.pf_part && (rc = dev_alloc(&b.pf_part, (uint64_t)cf.n_heads * 2 * kPflashMaxSplit * (32 + 16 * hs)))) return rc;
+        unsigned *cnt = nullptr;
+        if ((rc = dev_alloc(&cnt, (uint64_t)cf.n_heads * 2))) return rc;
+        if (hipMemset(cnt, 0, (size_t)cf.n_heads * 2 * sizeof(unsigned)) != hipSuccess) {
+            (void)hipFree(cnt);
+            return fail(L2J_E_HIP, "prefill: clearing the counters of the attention's workgroups");
+        }
+        b.pf_cnt = cnt;
     }
     const int nblocks = (n + kMaxBatch - 1) / kMaxBatch;
     std::vector<BatchState> hst((size_t)nblocks);

@@ -208,7 +208,7 @@ hipError_t l2j::launch_samplers(l2j_ctx *c, const BatchSamplers &bs, unsigned ac
     a.ss = bs.ss;
     a.scan = 1;
     a.nseq = nseq; a.active = active; a.cur = cur;
-    for (int i = 0; i < 2; i++) { a.pi_prob[i] = bs.pi_prob[i]; a.pi_idx[i] = bs.pi_idx[i]; }
+    a.pi_prob0 = bs.pi_prob[0]; a.pi_prob1 = bs.pi_prob[1]; a.pi_idx0 = bs.pi_idx[0]; a.pi_idx1 = bs.pi_idx[1];
     a.logits_stride = n; a.pi_stride = (long)bs.pi_stride;
     a.btoken = token; a.bout = out; a.bout_stride = out_stride;
     // (no k_sample_exp: with the sequences' workgroups side by side the exponentials cost less inside k_sample_probs than
@@ -219,10 +219,8 @@ hipError_t l2j::launch_samplers(l2j_ctx *c, const BatchSamplers &bs, unsigned ac
     if (e != hipSuccess || a.plain) return e;
     SortBatch sb{};
     sb.active = active; sb.cur = cur;
-    for (int i = 0; i < 2; i++) {
-        sb.pi_prob[i] = bs.pi_prob[i]; sb.pi_idx[i] = bs.pi_idx[i]; sb.out_prob[i] = bs.pi_prob[i]; sb.out_idx[i] = bs.pi_idx[i];
-        sb.sort_k[i] = bs.sort_k[i]; sb.sort_v[i] = bs.sort_v[i];
-    }
+    sb.pi_prob0 = bs.pi_prob[0]; sb.pi_prob1 = bs.pi_prob[1]; sb.pi_idx0 = bs.pi_idx[0]; sb.pi_idx1 = bs.pi_idx[1];
+    sb.tiles_k = bs.sort_k[0]; sb.tiles_v = bs.sort_v[0]; sb.runs_k = bs.sort_k[1]; sb.runs_v = bs.sort_v[1];
     sb.pi_stride = (long)bs.pi_stride; sb.sort_stride = (long)bs.sort_stride;
     hipLaunchKernelGGL(k_sort_tiles_b, dim3(npad / kSortTile, 1, nseq), dim3(kSortTile), 0, c->stream, sb, n);
     hipLaunchKernelGGL(k_merge_tiles_b, dim3(npad / kSortRun, 16, nseq), dim3(256), 0, c->stream, sb);

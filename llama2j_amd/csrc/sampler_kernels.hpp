@@ -44,8 +44,8 @@ struct SampleArgs {
     int nseq;
     unsigned active;         // bit s: sequence s samples in this step (the others' workgroups leave at once)
     unsigned cur;            // bit s: the copy of its ProbIndex array that sequence s's last top-p step left
-    float *pi_prob[2];       // the two copies, (sequence, pi_stride)
-    int *pi_idx[2];
+    float *pi_prob0, *pi_prob1;   // the two copies, (sequence, pi_stride); named one by one: a member array indexed by a
+    int *pi_idx0, *pi_idx1;       // variable would move the whole argument to scratch memory
     long logits_stride, pi_stride;
     int *btoken;             // (sequence): the token goes here (the sequence's next input)
     int *bout;               // and to bout[s * bout_stride]
@@ -58,13 +58,13 @@ __device__ __forceinline__ bool sample_seq(SampleArgs &a)
     if (a.nseq == 0) return true;
     const int s = blockIdx.z;
     if (!((a.active >> s) & 1u)) return false;
-    const int cur = (a.cur >> s) & 1u;
+    const bool cur = (a.cur >> s) & 1u;
     a.logits += s * a.logits_stride;
     a.ss += s;
-    a.cand_prob = a.pi_prob[cur] + s * a.pi_stride;
-    a.cand_idx = a.pi_idx[cur] + s * a.pi_stride;
-    a.sorted_prob = a.pi_prob[cur ^ 1] + s * a.pi_stride;
-    a.sorted_idx = a.pi_idx[cur ^ 1] + s * a.pi_stride;
+    a.cand_prob = (cur ? a.pi_prob1 : a.pi_prob0) + s * a.pi_stride;
+    a.cand_idx = (cur ? a.pi_idx1 : a.pi_idx0) + s * a.pi_stride;
+    a.sorted_prob = (cur ? a.pi_prob0 : a.pi_prob1) + s * a.pi_stride;
+    a.sorted_idx = (cur ? a.pi_idx0 : a.pi_idx1) + s * a.pi_stride;
     a.tok0 = a.btoken + s;
     a.tok1 = a.bout + s * a.bout_stride;
     return true;
@@ -780,22 +780,21 @@ static __global__ void __launch_bounds__(kSortTile) k_sort_tiles(const float *__
 // lie): a sequence's ProbIndex array goes from the copy its last step left through its own runs into the other copy.
 struct SortBatch {
     unsigned active, cur;
-    const float *pi_prob[2];
-    const int *pi_idx[2];
-    float *out_prob[2];      // (the same two copies, as the destination of the last merge)
-    int *out_idx[2];
+    float *pi_prob0, *pi_prob1;   // the two copies of the ProbIndex arrays, (sequence, pi_stride)
+    int *pi_idx0, *pi_idx1;
     long pi_stride;
-    float *sort_k[2];        // (sequence, sort_stride) twice: tiles, then runs
-    int *sort_v[2];
+    float *tiles_k, *runs_k;      // (sequence, sort_stride): the sorted tiles, then the sorted runs
+    int *tiles_v, *runs_v;
     long sort_stride;
 };
 
 static __global__ void __launch_bounds__(kSortTile) k_sort_tiles_b(const SortBatch b, int n)
 {
-    const int s = blockIdx.z, cur = (b.cur >> s) & 1u;
+    const int s = blockIdx.z;
+    const bool cur = (b.cur >> s) & 1u;
     if (!((b.active >> s) & 1u)) return;
-    sort_tiles_of(b.pi_prob[cur] + s * b.pi_stride, b.pi_idx[cur] + s * b.pi_stride, n, b.sort_k[0] + s * b.sort_stride,
-                  b.sort_v[0] + s * b.sort_stride);
+    sort_tiles_of((cur ? b.pi_prob1 : b.pi_prob0) + s * b.pi_stride, (cur ? b.pi_idx1 : b.pi_idx0) + s * b.pi_stride, n,
+                  b.tiles_k + s * b.sort_stride, b.tiles_v + s * b.sort_stride);
 }
 
 __device__ __forceinline__ void merge_tiles_of(const float *__restrict__ kin, const int *__restrict__ vin, float *__restrict__ kout,
@@ -844,8 +843,8 @@ static __global__ void __launch_bounds__(256) k_merge_tiles_b(const SortBatch b)
 {
     const int s = blockIdx.z;
     if (!((b.active >> s) & 1u)) return;
-    merge_tiles_of(b.sort_k[0] + s * b.sort_stride, b.sort_v[0] + s * b.sort_stride, b.sort_k[1] + s * b.sort_stride,
-                   b.sort_v[1] + s * b.sort_stride);
+    merge_tiles_of(b.tiles_k + s * b.sort_stride, b.tiles_v + s * b.sort_stride, b.runs_k + s * b.sort_stride,
+                   b.runs_v + s * b.sort_stride);
 }
 
 constexpr int kSortMaxRuns = (kSampleMaxVocab + kSortRun - 1) / kSortRun;
@@ -948,12 +947,13 @@ static __global__ void __launch_bounds__(256) k_merge_far(const float *__restric
 // holding a sequence's keys in LDS as k_merge_runs does would leave one workgroup per compute unit).
 static __global__ void __launch_bounds__(256) k_merge_far_b(const SortBatch b, int npad, int nout)
 {
-    const int s = blockIdx.z, cur = (b.cur >> s) & 1u;
+    const int s = blockIdx.z;
+    const bool cur = (b.cur >> s) & 1u;
     if (!((b.active >> s) & 1u)) return;
-    const float *kin = b.sort_k[1] + s * b.sort_stride;
-    const int *vin = b.sort_v[1] + s * b.sort_stride;
-    float *kout = b.out_prob[cur ^ 1] + s * b.pi_stride;
-    int *vout = b.out_idx[cur ^ 1] + s * b.pi_stride;
+    const float *kin = b.runs_k + s * b.sort_stride;
+    const int *vin = b.runs_v + s * b.sort_stride;
+    float *kout = (cur ? b.pi_prob0 : b.pi_prob1) + s * b.pi_stride;
+    int *vout = (cur ? b.pi_idx0 : b.pi_idx1) + s * b.pi_stride;
     if (npad <= 8 * kSortRun) merge_far_of<8>(kin, vin, npad, nout, kSortRun, kSortRun * kSortFanIn, kout, vout);   // (eight searches per pair)
     else merge_far_of<kSortFanIn>(kin, vin, npad, nout, kSortRun, kSortRun * kSortFanIn, kout, vout);
 }
