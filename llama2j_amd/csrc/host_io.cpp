@@ -10,9 +10,11 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <vector>
@@ -274,32 +276,61 @@ int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int wr
     TRY(l2j_upload_f32(ctx, L2J_TOK_EMB, reinterpret_cast<const float *>(m.p + off), vd));
     off += vd * 4;
 
-    std::vector<uint8_t> bytes;
+    // The ten quantized tensors by a few threads, as the reference's readAsQuant takes them (ten virtual threads,
+    // J/TransformerWeights.java:52,204): the uploads themselves take turns inside the library, but reading a cache file (or
+    // writing one) goes on beside them.  A thread's error text is its own: the first failure's is handed to the caller's.
+    struct Job { int tensor; uint64_t off, nf, nb; };
+    std::vector<Job> jobs;
     for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++) {
         const uint64_t nf = quant_floats(cfg, t), nb = l2j_quant_nbytes(nf);
         if (!need(nf)) BAIL(L2J_E_IO, std::string("checkpoint too short: ") + kStems[t]);
-        char qpath[4096];
-        TRY(l2j_quant_cache_path(bin_path, t, qpath, sizeof qpath) < 0 ? L2J_E_ARG : 0);
-        struct stat st;
-        if (stat(qpath, &st) == 0) {
-            // cache branch: the floats are skipped (J/TransformerWeights.java:198-203,219-232)
-            bytes.resize(nb);
-            const int64_t got = l2j_read_quant_file(qpath, bytes.data(), nb);
-            if (got < 0) {
-                l2j_destroy(ctx);
-                return (int)got;
-            }
-            TRY(l2j_upload_quant(ctx, t, bytes.data(), (uint64_t)got));
-        } else {
-            TRY(l2j_upload_f32_quantize(ctx, t, 0, reinterpret_cast<const float *>(m.p + off), nf));
-            if (write_caches && nb <= 0x7fffffffull) {
-                bytes.resize(nb);
-                TRY(l2j_read_quant(ctx, t, 0, nb / kGroupBytes, bytes.data()));
-                TRY(l2j_write_quant_file(qpath, bytes.data(), nb));
-            }
-        }
+        jobs.push_back({t, off, nf, nb});
         off += nf * 4;
     }
+    std::sort(jobs.begin(), jobs.end(), [](const Job &a, const Job &b) { return a.nf > b.nf; });   // (the long ones first)
+    std::atomic<size_t> next{0};
+    std::mutex err_mu;
+    int first_rc = L2J_OK;
+    std::string first_msg;
+    auto work = [&]() {
+        std::vector<uint8_t> bytes;
+        for (size_t k = next.fetch_add(1); k < jobs.size(); k = next.fetch_add(1)) {
+            const Job &j = jobs[k];
+            int r = L2J_OK;
+            char qpath[4096];
+            struct stat st;
+            if (l2j_quant_cache_path(bin_path, j.tensor, qpath, sizeof qpath) < 0) {
+                r = fail(L2J_E_ARG, "cache file name too long");
+            } else if (stat(qpath, &st) == 0) {
+                // cache branch: the floats are skipped (J/TransformerWeights.java:198-203,219-232)
+                bytes.resize(j.nb);
+                const int64_t got = l2j_read_quant_file(qpath, bytes.data(), j.nb);
+                r = got < 0 ? (int)got : l2j_upload_quant(ctx, j.tensor, bytes.data(), (uint64_t)got);
+            } else {
+                r = l2j_upload_f32_quantize(ctx, j.tensor, 0, reinterpret_cast<const float *>(m.p + j.off), j.nf);
+                if (r == L2J_OK && write_caches && j.nb <= 0x7fffffffull) {
+                    bytes.resize(j.nb);
+                    r = l2j_read_quant(ctx, j.tensor, 0, j.nb / kGroupBytes, bytes.data());
+                    if (r == L2J_OK) r = l2j_write_quant_file(qpath, bytes.data(), j.nb);
+                }
+            }
+            if (r != L2J_OK) {
+                std::lock_guard<std::mutex> lock(err_mu);
+                if (first_rc == L2J_OK) { first_rc = r; first_msg = l2j_last_error(); }
+                next.store(jobs.size());   // (the others stop after the tensor they are at)
+                return;
+            }
+        }
+    };
+    {
+        const unsigned hw = std::thread::hardware_concurrency();
+        const size_t nthreads = std::min<size_t>(jobs.size(), std::max(1u, std::min(4u, hw ? hw : 1u)));
+        std::vector<std::thread> pool;
+        for (size_t i = 1; i < nthreads; i++) pool.emplace_back(work);
+        work();
+        for (std::thread &th : pool) th.join();
+    }
+    if (first_rc != L2J_OK) BAIL(first_rc, first_msg);
     off += 2ull * ((uint64_t)cfg.seq_len * (cfg.dim / cfg.n_heads) / 2) * 4;  // freq_cis_real, freq_cis_imag: skipped
     if (!cfg.shared_weights) {
         if (!need(vd)) BAIL(L2J_E_IO, "checkpoint too short: wcls");
