@@ -273,19 +273,25 @@ int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int wr
     } while (0)
 
     if (!need(vd)) BAIL(L2J_E_IO, "checkpoint too short: token_embedding_table");
-    TRY(l2j_upload_f32(ctx, L2J_TOK_EMB, reinterpret_cast<const float *>(m.p + off), vd));
+    const uint64_t emb_off = off;
     off += vd * 4;
 
-    // The ten quantized tensors by a few threads, as the reference's readAsQuant takes them (ten virtual threads,
+    // The tensors by a few threads, as the reference's readAsQuant takes them (ten virtual threads,
     // J/TransformerWeights.java:52,204): the uploads themselves take turns inside the library, but reading a cache file (or
     // writing one) goes on beside them.  A thread's error text is its own: the first failure's is handed to the caller's.
-    struct Job { int tensor; uint64_t off, nf, nb; };
+    struct Job { int tensor; uint64_t off, nf, nb; };   // (the two fp32 tensors too: nb = 0)
     std::vector<Job> jobs;
+    jobs.push_back({L2J_TOK_EMB, emb_off, vd, 0});
     for (int t = L2J_RMS_ATT; t <= L2J_RMS_FINAL; t++) {
         const uint64_t nf = quant_floats(cfg, t), nb = l2j_quant_nbytes(nf);
         if (!need(nf)) BAIL(L2J_E_IO, std::string("checkpoint too short: ") + kStems[t]);
         jobs.push_back({t, off, nf, nb});
         off += nf * 4;
+    }
+    off += 2ull * ((uint64_t)cfg.seq_len * (cfg.dim / cfg.n_heads) / 2) * 4;  // freq_cis_real, freq_cis_imag: skipped
+    if (!cfg.shared_weights) {
+        if (!need(vd)) BAIL(L2J_E_IO, "checkpoint too short: wcls");
+        jobs.push_back({L2J_WCLS, off, vd, 0});
     }
     std::sort(jobs.begin(), jobs.end(), [](const Job &a, const Job &b) { return a.nf > b.nf; });   // (the long ones first)
     std::atomic<size_t> next{0};
@@ -299,13 +305,22 @@ int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int wr
             int r = L2J_OK;
             char qpath[4096];
             struct stat st;
-            if (l2j_quant_cache_path(bin_path, j.tensor, qpath, sizeof qpath) < 0) {
+            if (j.nb == 0) {
+                r = l2j_upload_f32(ctx, j.tensor, reinterpret_cast<const float *>(m.p + j.off), j.nf);
+            } else if (l2j_quant_cache_path(bin_path, j.tensor, qpath, sizeof qpath) < 0) {
                 r = fail(L2J_E_ARG, "cache file name too long");
             } else if (stat(qpath, &st) == 0) {
-                // cache branch: the floats are skipped (J/TransformerWeights.java:198-203,219-232)
-                bytes.resize(j.nb);
-                const int64_t got = l2j_read_quant_file(qpath, bytes.data(), j.nb);
-                r = got < 0 ? (int)got : l2j_upload_quant(ctx, j.tensor, bytes.data(), (uint64_t)got);
+                // cache branch: the floats are skipped (J/TransformerWeights.java:198-203,219-232).  The file is uploaded out of
+                // a mapping of it (as l2j_read_quant_file checks it: the length prefix, then that many bytes).
+                Mapped q;
+                r = map_file(qpath, q);
+                if (r == L2J_OK) {
+                    int32_t n = -1;
+                    if (q.len >= 4) memcpy(&n, q.p, 4);
+                    if (n < 0) r = fail(L2J_E_IO, std::string("bad length prefix in ") + qpath);
+                    else if ((uint64_t)n > q.len - 4) r = fail(L2J_E_IO, std::string("short read from ") + qpath);
+                    else r = l2j_upload_quant(ctx, j.tensor, q.p + 4, (uint64_t)n);   // (a size other than the tensor's: L2J_E_SIZE)
+                }
             } else {
                 r = l2j_upload_f32_quantize(ctx, j.tensor, 0, reinterpret_cast<const float *>(m.p + j.off), j.nf);
                 if (r == L2J_OK && write_caches && j.nb <= 0x7fffffffull) {
@@ -324,18 +339,13 @@ int l2j_load_checkpoint(const char *bin_path, int device, uint32_t flags, int wr
     };
     {
         const unsigned hw = std::thread::hardware_concurrency();
-        const size_t nthreads = std::min<size_t>(jobs.size(), std::max(1u, std::min(4u, hw ? hw : 1u)));
+        const size_t nthreads = std::min<size_t>(jobs.size(), std::max(1u, std::min(6u, hw ? hw : 1u)));
         std::vector<std::thread> pool;
         for (size_t i = 1; i < nthreads; i++) pool.emplace_back(work);
         work();
         for (std::thread &th : pool) th.join();
     }
     if (first_rc != L2J_OK) BAIL(first_rc, first_msg);
-    off += 2ull * ((uint64_t)cfg.seq_len * (cfg.dim / cfg.n_heads) / 2) * 4;  // freq_cis_real, freq_cis_imag: skipped
-    if (!cfg.shared_weights) {
-        if (!need(vd)) BAIL(L2J_E_IO, "checkpoint too short: wcls");
-        TRY(l2j_upload_f32(ctx, L2J_WCLS, reinterpret_cast<const float *>(m.p + off), vd));
-    }
     TRY(l2j_finalize(ctx));
 #undef TRY
 #undef BAIL

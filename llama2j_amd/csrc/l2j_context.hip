@@ -22,29 +22,44 @@ int validate_config(const l2j_config &c)
     return L2J_OK;
 }
 
-int unpack_into(l2j_ctx *c, QTensor &t, uint64_t group0, const uint8_t *ref_bytes, uint64_t ngroups)
-{
-    // staged through a device buffer in slices of at most 64 MiB
-    const uint64_t slice_groups = (64ull << 20) / kGroupBytes;
-    uint8_t *stage = nullptr;
-    HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(ngroups, slice_groups) * kGroupBytes));
-    int rc = L2J_OK;
-    for (uint64_t g = 0; g < ngroups && rc == L2J_OK; g += slice_groups) {
-        const uint64_t ng = std::min(slice_groups, ngroups - g);
-        hipError_t e = hipMemcpy(stage, ref_bytes + g * kGroupBytes, ng * kGroupBytes, hipMemcpyHostToDevice);
-        if (e == hipSuccess) {
-            const int grid = (int)std::min<uint64_t>(ng, 1u << 20);
-            hipLaunchKernelGGL(k_unpack_groups, dim3(grid), dim3(64), 0, c->stream, stage, (long)ng, t.codes + (group0 + g) * kGroup,
-                               t.gs + group0 + g, t.mm + group0 + g);
-            e = hipGetLastError();
-            if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
-        }
-        if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("upload: ") + hipGetErrorString(e));
+// A slice of the caller's host memory in a device buffer of the call's own, copied on a stream of the call's own and
+// without the context's lock: the copies of calls on different threads (the loader's, or a JVM's ten virtual threads)
+// run side by side, and only the kernel that takes the slice apart runs under the lock.
+struct Staged {
+    void *dev = nullptr;
+    size_t cap = 0;
+    hipStream_t s = nullptr;
+    ~Staged()
+    {
+        if (dev) (void)hipFree(dev);
+        if (s) (void)hipStreamDestroy(s);
     }
-    (void)hipFree(stage);
-    return rc;
-}
+    int in(const void *host, size_t bytes, size_t cap_bytes)
+    {
+        if (!s) HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+        if (!dev) {
+            HIPCHK(hipMalloc(&dev, std::max<size_t>(cap_bytes, 1)));
+            cap = cap_bytes;
+        }
+        HIPCHK(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, s));
+        HIPCHK(hipStreamSynchronize(s));
+        return L2J_OK;
+    }
+};
 
+constexpr uint64_t kStageBytes = 1ull << 30;   // at most this much of a tensor at a time
+
+// `ngroups` groups of reference bytes, already in device memory, into the tensor's arrays from group0 on (under the lock)
+int unpack_staged(l2j_ctx *c, QTensor &t, uint64_t group0, const uint8_t *stage, uint64_t ngroups)
+{
+    const int grid = (int)std::min<uint64_t>(ngroups, 1u << 20);
+    hipLaunchKernelGGL(k_unpack_groups, dim3(grid), dim3(64), 0, c->stream, stage, (long)ngroups, t.codes + group0 * kGroup, t.gs + group0,
+                       t.mm + group0);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e != hipSuccess) return fail(L2J_E_HIP, std::string("upload: ") + hipGetErrorString(e));
+    return L2J_OK;
+}
 
 }  // namespace
 
@@ -259,15 +274,32 @@ static int upload_quant_range(l2j_ctx *c, int tensor, uint64_t group0, uint64_t 
 {
     if (nbytes != ngroups * kGroupBytes)
         return fail(L2J_E_SIZE, "totalByteSize != quant.numberOfBytesByFloatSize(floatSize)");
-    std::lock_guard<std::mutex> lock(c->upload_mu);
-    if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
-    HIPCHK(hipSetDevice(c->cfg.device));
     QTensor &t = c->qt[tensor];
-    if (whole) t.groups_loaded = 0;
-    invalidate_batch_tiles(c, tensor);
-    int rc = unpack_into(c, t, group0, bytes, ngroups);
-    if (rc == L2J_OK) t.groups_loaded += ngroups;
-    return rc;
+    std::lock_guard<std::mutex> tensor_lock(t.mu);
+    HIPCHK(hipSetDevice(c->cfg.device));
+    const uint64_t slice_groups = kStageBytes / kGroupBytes;
+    Staged st;
+    bool first = true;
+    for (uint64_t g = 0; g < ngroups || first; g += slice_groups) {
+        const uint64_t ng = std::min(slice_groups, ngroups - g);
+        if (ng) {
+            const int rc = st.in(bytes + g * kGroupBytes, ng * kGroupBytes, std::min(ngroups, slice_groups) * kGroupBytes);
+            if (rc) return rc;
+        }
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+        if (first) {
+            if (whole) t.groups_loaded = 0;
+            invalidate_batch_tiles(c, tensor);
+            first = false;
+        }
+        if (ng) {
+            const int rc = unpack_staged(c, t, group0 + g, static_cast<const uint8_t *>(st.dev), ng);
+            if (rc) return rc;
+            t.groups_loaded += ng;
+        }
+    }
+    return L2J_OK;
 }
 
 int l2j_upload_quant(l2j_ctx *c, int tensor, const uint8_t *ref_bytes, uint64_t nbytes)
@@ -316,29 +348,35 @@ int l2j_upload_f32_quantize(l2j_ctx *c, int tensor, uint64_t first, const float 
         if (first % kGroup) return fail(L2J_E_ARG, "first must be a multiple of the group size");
         if (first + nfloats > t.nfloats) return fail(L2J_E_SIZE, "range exceeds the tensor");
         if (nfloats % kGroup && first + nfloats != t.nfloats) return fail(L2J_E_ARG, "only the tensor's tail may be a partial group");
-        std::lock_guard<std::mutex> lock(c->upload_mu);
-        if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+        std::lock_guard<std::mutex> tensor_lock(t.mu);
         HIPCHK(hipSetDevice(c->cfg.device));
-        invalidate_batch_tiles(c, tensor);
-        const uint64_t slice = 16ull << 20;  // floats per staging slice (64 MiB)
-        float *stage = nullptr;
-        HIPCHK(hipMalloc(reinterpret_cast<void **>(&stage), std::min(slice, std::max<uint64_t>(nfloats, 1)) * sizeof(float)));
-        int rc = L2J_OK;
-        for (uint64_t o = 0; o < nfloats && rc == L2J_OK; o += slice) {
+        const uint64_t slice = kStageBytes / sizeof(float);   // floats per staging slice
+        Staged st;
+        bool first_slice = true;
+        for (uint64_t o = 0; o < nfloats || first_slice; o += slice) {
             const uint64_t nf = std::min(slice, nfloats - o);
             const uint64_t ng = (nf + kGroup - 1) / kGroup;
-            hipError_t e = hipMemcpy(stage, data + o, nf * sizeof(float), hipMemcpyHostToDevice);
-            if (e == hipSuccess) {
-                hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(256), 0, c->stream, stage, (long)nf,
-                                   (long)((first + o) / kGroup), (long)ng, (long)t.nfloats, 0ull, 0.0f, t.codes, t.gs, t.mm);
-                e = hipGetLastError();
-                if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+            if (nf) {   // (the copy: without the context's lock)
+                const int rc = st.in(data + o, nf * sizeof(float), std::min(slice, nfloats) * sizeof(float));
+                if (rc) return rc;
             }
-            if (e != hipSuccess) rc = fail(L2J_E_HIP, std::string("quantize: ") + hipGetErrorString(e));
-            else t.groups_loaded += ng;
+            std::lock_guard<std::mutex> lock(c->upload_mu);
+            if (c->finalized) return fail(L2J_E_STATE, "upload after l2j_finalize");
+            if (first_slice) {
+                invalidate_batch_tiles(c, tensor);
+                first_slice = false;
+            }
+            if (nf) {
+                hipLaunchKernelGGL(k_encode_groups, dim3((unsigned)std::min<uint64_t>(ng, 1u << 20)), dim3(256), 0, c->stream,
+                                   static_cast<const float *>(st.dev), (long)nf, (long)((first + o) / kGroup), (long)ng, (long)t.nfloats, 0ull,
+                                   0.0f, t.codes, t.gs, t.mm);
+                hipError_t e = hipGetLastError();
+                if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+                if (e != hipSuccess) return fail(L2J_E_HIP, std::string("quantize: ") + hipGetErrorString(e));
+                t.groups_loaded += ng;
+            }
         }
-        (void)hipFree(stage);
-        return rc;
+        return L2J_OK;
     }());
 }
 

@@ -47,6 +47,7 @@ struct QTensor {
     float2 *mm = nullptr;      // (min, max) per group
     uint64_t nfloats = 0, ngroups = 0;
     uint64_t groups_loaded = 0;
+    std::mutex mu;             // uploads of this tensor take turns (those of different tensors copy side by side)
 };
 
 // Launch-shape and algorithm switches of a context.  kAuto = the library picks (by shape, at l2j_finalize).  A context
