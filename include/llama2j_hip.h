@@ -168,6 +168,12 @@ int l2j_decode_greedy(l2j_ctx *ctx, const int32_t *prompt, int32_t n_prompt, int
  * *seconds (may be NULL): GPU time from the end of the first step to the end of the last. */
 int l2j_decode_greedy_batch(l2j_ctx *ctx, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq,
                             int32_t prompt_stride, int32_t steps, int32_t *out_tokens, double *seconds);
+/* Gives back what the calls for several sequences at once keep on the device (l2j_decode_greedy_batch,
+ * l2j_decode_sample_batch, l2j_prefill): the second copy of the quantized matrices, the activation buffers, the KV cache
+ * of the sequences, their samplers and the captured graph.  The next such call makes them again (and pays for it: the
+ * copy of the matrices is one pass over them).  The single-sequence path and its cache are not touched.  No counterpart
+ * in the reference. */
+int l2j_release_batch(l2j_ctx *ctx);
 
 /* ---- sampling on the device: J/Sampler.java and the sampling branch of J/Run.java:643-665 ----
  * The context holds one sampler = the reference's Sampler object: a java.util.Random and the ProbIndex

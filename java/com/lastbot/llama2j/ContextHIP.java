@@ -40,7 +40,7 @@ public final class ContextHIP implements AutoCloseable {
     // buffers of the token loop's thread, allocated once (no allocation per token)
     private final MemorySegment logitsSeg, intSeg, tokensSeg, promptSeg, countSeg, secondsSeg;
     private final MethodHandle lastError, ctxLastError, destroy, setOption, uploadQuant, uploadF32, finalizeH, reset, forward,
-            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSampleBatch, decodeSample, samplerSeed, sample, prefill;
+            forwardArgmax, decodeGreedy, decodeGreedyBatch, decodeSampleBatch, releaseBatch, decodeSample, samplerSeed, sample, prefill;
 
     private MethodHandle handle(String name, FunctionDescriptor fd) {
         return LINKER.downcallHandle(lib.find(name).orElseThrow(), fd);
@@ -64,6 +64,7 @@ public final class ContextHIP implements AutoCloseable {
                 FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS));
         decodeSampleBatch = handle("l2j_decode_sample_batch", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
                 JAVA_INT, JAVA_FLOAT, JAVA_FLOAT, ADDRESS, ADDRESS, ADDRESS, ADDRESS));
+        releaseBatch = handle("l2j_release_batch", FunctionDescriptor.of(JAVA_INT, ADDRESS));
         decodeSample = handle("l2j_decode_sample", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT,
                 JAVA_FLOAT, JAVA_FLOAT, JAVA_LONG, ADDRESS, ADDRESS, ADDRESS));
         samplerSeed = handle("l2j_sampler_seed", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_LONG));
@@ -273,6 +274,11 @@ public final class ContextHIP implements AutoCloseable {
             for (int b = 0; b < batch; b++) MemorySegment.copy(out, JAVA_INT, (long) b * steps * Integer.BYTES, tokens[b], 0, steps);
             return tokens;
         }
+    }
+
+    /** Frees what decodeGreedyBatch / decodeSampleBatch / prefill keep on the device (l2j_release_batch); they make it again. */
+    public void releaseBatch() {
+        check(call(releaseBatch, ctx));
     }
 
     /**

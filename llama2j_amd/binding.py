@@ -118,6 +118,7 @@ def _signatures():
         "l2j_calibration_copy": (C.c_int, [vp, C.c_uint64, C.c_int32]),
         "l2j_decode_greedy_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, C.POINTER(C.c_double)]),
         "l2j_decode_greedy_batch_logits": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, i32p, fp]),
+        "l2j_release_batch": (C.c_int, [vp]),
         "l2j_decode_sample_batch": (C.c_int, [vp, i32p, i32p, C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_float,
                                               C.POINTER(C.c_int64), i32p, C.POINTER(C.c_double), fp]),
         "l2j_batch_matmul": (C.c_int, [vp, C.c_int, C.c_int, fp, fp, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
@@ -457,6 +458,10 @@ class Transformer:
         sec = C.c_double(0.0)
         self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), C.byref(sec)))
         return out, sec.value
+
+    def release_batch(self):
+        """Frees what the calls for several sequences at once keep on the device (l2j_release_batch)."""
+        self._check(lib().l2j_release_batch(self._h))
 
     def decode_sample_batch(self, prompts, steps, temperature, topp, rng_seeds, n_seq=None, want_logits=False):
         """decode_greedy_batch with a sampler per sequence (l2j_decode_sample_batch): sequence b samples its unforced

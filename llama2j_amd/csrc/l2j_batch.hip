@@ -675,6 +675,19 @@ int l2j_prefill(l2j_ctx *c, const int32_t *tokens, int32_t n, int32_t pos0, floa
     }());
 }
 
+int l2j_release_batch(l2j_ctx *c)
+{
+    return ctx_rc(c, [&]() -> int {
+        std::lock_guard<std::mutex> forward_lock(g_forward_mu);
+        if (!c) return fail(L2J_E_ARG, "null context");
+        HIPCHK(hipSetDevice(c->cfg.device));
+        HIPCHK(hipStreamSynchronize(c->stream));
+        std::lock_guard<std::mutex> lock(c->upload_mu);
+        free_batch(c);
+        return L2J_OK;
+    }());
+}
+
 int l2j_decode_greedy_batch(l2j_ctx *c, const int32_t *prompts, const int32_t *n_prompt, int32_t n_seq, int32_t prompt_stride,
                             int32_t steps, int32_t *out_tokens, double *seconds)
 {

@@ -301,3 +301,40 @@ def test_the_sampling_steps_of_the_batch_wait_for_nobody():
         outs.append(out)
         g.close()
     np.testing.assert_array_equal(outs[0], outs[1])
+
+
+def test_release_batch_gives_the_memory_back_and_the_next_call_makes_it_again():
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = C.c_size_t(0), C.c_size_t(0)
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    shape = SHAPES[2]
+    g = l2j.Transformer(l2j.Config(*shape))
+    g.fill_synthetic(11, 0.02)
+    g.finalize()
+    prompts = [np.array([5, 9, 13], dtype=np.int32), np.array([7], dtype=np.int32)]
+    single, _ = g.decode_greedy(prompts[0], 24)
+    g.reset()
+    g.release_batch()                                  # (nothing to release yet: not an error)
+    before = free_bytes()
+    want, _ = g.decode_greedy_batch(prompts, 24)
+    sampled, _ = g.decode_sample_batch(prompts, 24, 0.9, 0.9, [1, 2])
+    tokens = np.concatenate([[1], prompts[0], np.arange(20, 40)]).astype(np.int32)
+    logits, _ = g.prefill(tokens)
+    held = before - free_bytes()
+    assert held > 10 << 20                             # the copy of the matrices, caches, buffers, samplers
+    g.release_batch()
+    assert abs(free_bytes() - before) <= 4 << 20
+    g.reset()
+    again, _ = g.decode_greedy_batch(prompts, 24)
+    np.testing.assert_array_equal(again, want)
+    np.testing.assert_array_equal(g.decode_sample_batch(prompts, 24, 0.9, 0.9, [1, 2])[0], sampled)
+    g.reset()
+    np.testing.assert_array_equal(g.prefill(tokens)[0].view(np.uint32), logits.view(np.uint32))
+    g.reset()
+    np.testing.assert_array_equal(g.decode_greedy(prompts[0], 24)[0], single)   # the single-sequence path: untouched
+    g.close()
