@@ -124,6 +124,50 @@ def cpu_baseline_long_context(shape, seed, g, gpu_tokens, positions):
     }
 
 
+def load_test(workload, directory):
+    """Not the metric: the load path (l2j_load_checkpoint = the TransformerWeights constructor,
+    J/TransformerWeights.java:43-144,191-356) at the workload's shape.  Writes a llama2.c v0 checkpoint of random floats
+    (27 GB at the 7B shape) into `directory` (memory-backed storage such as /dev/shm keeps the disk out of the figures),
+    loads it once without caches (quantizing on the GPU, writing the .quant caches) and twice from the caches, and removes
+    the files.  Prints one JSON line of its own."""
+    import shutil
+    import struct
+    import llama2j_amd as l2j
+    shape, seed, _ = WORKLOADS[workload]
+    dim, hidden, L, H, kvH, vocab, seq, shared = shape
+    d = os.path.join(directory, "l2j_load_test")
+    shutil.rmtree(d, ignore_errors=True)
+    os.makedirs(d)
+    try:
+        kvd = dim * kvH // H
+        sizes = [vocab * dim, L * dim, L * dim * dim, L * dim * kvd, L * dim * kvd, L * dim * dim, L * dim, L * dim * hidden,
+                 L * hidden * dim, L * dim * hidden, dim, seq * (dim // H) // 2 * 2] + ([] if shared else [vocab * dim])
+        block = (np.random.default_rng(seed).standard_normal(16 << 20) * 0.02).astype("<f4")
+        path = os.path.join(d, "model.bin")
+        with open(path, "wb") as f:                      # J/Run.java:561-573: seven ints, then the tensors in file order
+            f.write(struct.pack("<7i", dim, hidden, L, H, kvH, vocab if shared else -vocab, seq))
+            for n in sizes:
+                for o in range(0, n, block.size):
+                    f.write(block[:min(block.size, n - o)].data)
+        out = {"load_test": workload, "bin_bytes": os.path.getsize(path), "directory": directory}
+        tokens, same = None, True
+        for name, write in (("first_load_s", True), ("cached_load_s", False), ("cached_load_again_s", False)):
+            t0 = time.perf_counter()
+            g = l2j.Transformer.from_checkpoint(path, write_caches=write)
+            g.sync()
+            out[name] = round(time.perf_counter() - t0, 3)
+            toks, sec = g.decode_greedy(np.array([5, 9, 13], dtype=np.int32), 24)
+            same = same and (tokens is None or bool(np.array_equal(tokens, toks)))
+            tokens = toks
+            g.close()
+        out["same_tokens_after_every_load"] = same
+        out["cache_bytes"] = sum(os.path.getsize(os.path.join(d, x)) for x in os.listdir(d) if x.endswith(".quant"))
+        print(json.dumps(out))
+    finally:
+        shutil.rmtree(d, ignore_errors=True)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,7 +183,12 @@ def main():
                                                                   "which a profiler can follow; the batched decode replays a graph)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also run a plain copy kernel of this size (scales rocprofv3 byte counters)")
+    ap.add_argument("--load-test", metavar="DIR", default=None,
+                    help="instead of the decode: time l2j_load_checkpoint on a synthetic checkpoint of the workload's shape written into DIR "
+                         "(e.g. /dev/shm; 27 GB + 7 GB of caches at the 7B shape, removed afterwards)")
     a = ap.parse_args()
+    if a.load_test:
+        return load_test(a.workload, a.load_test)
     if a.gpus != 1:
         print("bench.py: this path runs on ONE GPU (batch-1 decode, no multi-GPU split); --gpus %d is not supported" % a.gpus,
               file=sys.stderr)
