@@ -459,6 +459,16 @@ class Transformer:
         self._check(lib().l2j_decode_greedy_batch(self._h, _i32(ids), _i32(n), n_seq, stride, steps, _i32(out), C.byref(sec)))
         return out, sec.value
 
+    @staticmethod
+    def until_bos(tokens):
+        """The rows of decode_greedy_batch / decode_sample_batch as Run.main's loop would have left them: each cut behind its
+        first token 1, where the reference's loop stops (J/Run.java:670-672); the batch runs every sequence to the last step."""
+        out = []
+        for row in np.asarray(tokens):
+            ones = np.flatnonzero(row == 1)
+            out.append(row[:ones[0] + 1] if ones.size else row)
+        return out
+
     def release_batch(self):
         """Frees what the calls for several sequences at once keep on the device (l2j_release_batch)."""
         self._check(lib().l2j_release_batch(self._h))

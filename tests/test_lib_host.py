@@ -117,3 +117,10 @@ def test_error_paths_without_gpu():
     assert L.l2j_forward(None, 1, 0, None) == -1
     assert L.l2j_finalize(None) == -1
     L.l2j_destroy(None)  # no-op
+
+
+def test_rows_of_a_batch_are_cut_where_the_reference_loop_stops():
+    import llama2j_amd as l2j
+    rows = np.array([[5, 9, 1, 7, 1], [4, 4, 4, 4, 4], [1, 2, 3, 4, 5]], dtype=np.int32)
+    cut = l2j.Transformer.until_bos(rows)
+    assert [list(r) for r in cut] == [[5, 9, 1], [4, 4, 4, 4, 4], [1]]
